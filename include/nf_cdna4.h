@@ -1,0 +1,129 @@
+/*
+ * nf_cdna4.h -- C ABI of libnf_cdna4.so: hand-written gfx950 (MI355X) kernels for
+ * the three neural-field hot paths of triton_helpers.layers.
+ *
+ * Every entry point takes raw device pointers, sizes and strides in ELEMENTS,
+ * dtype codes and a HIP stream handle (hipStream_t passed as void*; NULL = the
+ * default stream).  Nothing is allocated, freed or synchronised inside the
+ * library; work is enqueued on the given stream and the call returns.  All
+ * functions return 0 on success, a negative NF_E* code on an argument error,
+ * or a positive hipError_t; nf_last_error() returns a thread-local message.
+ *
+ * The functions replace the Triton launches of the reference (paths relative
+ * to the reference repository):
+ *   nf_hash_encode_fwd     <- _fwd_kernel[grid](...)   triton_helpers/layers/hash_encoding/kernel.py:575-590 (kernel :155-306)
+ *   nf_hash_encode_bwd     <- _bwd_kernel[grid](...)   triton_helpers/layers/hash_encoding/kernel.py:641-656 (kernel :309-440)
+ *   nf_hash_encode_indices <- embedding_lookup         triton_helpers/layers/hash_encoding/kernel.py:88-152
+ *                             (exposed by the reference only through its test kernels,
+ *                              tests/test_layers/test_hash_encoding.py:178-215)
+ *   nf_mlp_fwd             <- _fwd_kernel[grid](...)   triton_helpers/layers/fully_fused_mlp/kernel.py:553-562 (kernel :181-261)
+ *   nf_mlp_bwd             <- _bwd_kernel_rfs[grid](...) + host sum(0)
+ *                                                      triton_helpers/layers/fully_fused_mlp/kernel.py:612-633 (kernel :307-500)
+ *   nf_revmlp_fwd / nf_revmlp_bwd : no counterpart in the reference (it has no
+ *                             reversible MLP); same conventions as nf_mlp_*.
+ */
+#ifndef NF_CDNA4_H
+#define NF_CDNA4_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NF_ABI_VERSION 1
+
+/* element types */
+enum { NF_F32 = 0, NF_F16 = 1, NF_BF16 = 2 };
+
+/* activations (triton_helpers/ops.py:37-66; GELU = exact erf form, used by the reversible MLP) */
+enum { NF_ACT_NONE = 0, NF_ACT_RELU = 1, NF_ACT_SILU = 2, NF_ACT_RELU2 = 3, NF_ACT_GELU = 4 };
+
+/* error codes (negative) */
+enum {
+  NF_OK = 0,
+  NF_EINVAL = -1,      /* bad argument value                           */
+  NF_EUNSUPPORTED = -2,/* valid request this build has no kernel for    */
+  NF_EALIGN = -3       /* pointer / stride alignment requirement unmet  */
+};
+
+#define NF_MAX_LEVELS 32
+#define NF_MAX_DIMS 4
+
+/* Level geometry of a hash encoding, computed on the host
+ * (triton_helpers/layers/hash_encoding/helpers.py:26-115). */
+typedef struct nf_hash_geom {
+  int32_t dims;                 /* D, 1..NF_MAX_DIMS                                  */
+  int32_t feat;                 /* F, features per table row                          */
+  int32_t levels;               /* L, 1..NF_MAX_LEVELS                                */
+  int32_t first_hash_level;     /* first level that hashes (>= levels: none)          */
+  int64_t max_rows;             /* T, cap on rows per level                           */
+  int32_t res[NF_MAX_LEVELS];   /* N_l                                                */
+  int64_t rows[NF_MAX_LEVELS];  /* T_l = min((N_l+1)^D, T)                            */
+  int64_t row_offset[NF_MAX_LEVELS]; /* first row of level l in the stacked table     */
+} nf_hash_geom;
+
+/* flags for the hash-encoding entry points */
+enum {
+  NF_HASH_FORCE_GENERIC = 1    /* use the one-thread-per-(point,level) kernel even where the tiled kernel applies */
+};
+
+int nf_abi_version(void);
+const char* nf_last_error(void);
+
+/* out[n, l*F + f] = sum_j w_j(x_n, l) * table[row_offset[l] + row_j(x_n, l), f]
+ * coords [n_points, D] (coords_dtype, strides in elements), coordinates in [0, scale];
+ * table  [E, F] row-contiguous (table_dtype); out rows of table_dtype, row stride
+ * out_stride_n elements (>= L*F; extra columns are left untouched);
+ * primes: device pointer to >= D int64 hashing primes. */
+int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t coords_stride_n, int64_t coords_stride_d,
+                       const void* table, int table_dtype, void* out, int64_t out_stride_n, int64_t n_points,
+                       const nf_hash_geom* geom, const int64_t* primes, float scale, int flags, void* stream);
+
+/* dtable[row_offset[l] + row_j, f] += w_j * dout[n, l*F + f]   (float32 accumulators,
+ * NOT cleared by the call).  dout rows of dout_dtype with row stride dout_stride_n. */
+int nf_hash_encode_bwd(const void* coords, int coords_dtype, int64_t coords_stride_n, int64_t coords_stride_d,
+                       const void* dout, int dout_dtype, int64_t dout_stride_n, float* dtable, int64_t n_points,
+                       const nf_hash_geom* geom, const int64_t* primes, float scale, int flags, void* stream);
+
+/* Level-local table rows of all 2^D corners: out_rows [n_points, L, 2^D] int64, and
+ * (optional, may be NULL) the interpolation weights out_w [n_points, L, 2^D] float32. */
+int nf_hash_encode_indices(const void* coords, int coords_dtype, int64_t coords_stride_n, int64_t coords_stride_d,
+                           int64_t* out_rows, float* out_w, int64_t n_points, const nf_hash_geom* geom,
+                           const int64_t* primes, float scale, void* stream);
+
+/* Fully fused MLP.  x [rows, d_in] (row stride x_stride), y [rows, d_out] (row stride y_stride);
+ * w_in [d_hidden, d_in], w_hid [(depth-1)*d_hidden, d_hidden], w_out [d_out, d_hidden], all
+ * row-contiguous in `dtype`; biases b_in [d_hidden], b_hid [depth-1, d_hidden], b_out [d_out]
+ * may each be NULL.  depth >= 1 counts the input layer plus the hidden layers. */
+int nf_mlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_stride, const void* w_in, const void* b_in,
+               const void* w_hid, const void* b_hid, const void* w_out, const void* b_out, int64_t rows, int d_in,
+               int d_hidden, int d_out, int depth, int act, int dtype, void* stream);
+
+/* Backward.  dx [rows, d_in] in `dtype`; the dw_ and db_ arguments are float32 accumulators shaped like the
+ * weights/biases, NOT cleared by the call (db_* may be NULL; dx may be NULL). */
+int nf_mlp_bwd(const void* x, int64_t x_stride, const void* dy, int64_t dy_stride, void* dx, int64_t dx_stride,
+               const void* w_in, const void* b_in, const void* w_hid, const void* b_hid, const void* w_out,
+               const void* b_out, float* dw_in, float* db_in, float* dw_hid, float* db_hid, float* dw_out,
+               float* db_out, int64_t rows, int d_in, int d_hidden, int d_out, int depth, int act, int dtype,
+               void* stream);
+
+/* Reversible MLP of `blocks` additive couplings over rows of width 2*half:
+ *   y1 = x1 + F_k(x2),  y2 = x2 + G_k(y1),  F/G(u) = act(u W1^T + b1) W2^T + b2.
+ * w1, w2 [blocks*2*half, half] (F_k then G_k per block), b1, b2 [blocks*2, half] or NULL. */
+int nf_revmlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_stride, const void* w1, const void* b1,
+                  const void* w2, const void* b2, int64_t rows, int half, int blocks, int act, int dtype,
+                  void* stream);
+
+/* Backward from the OUTPUT y: the inputs are recomputed block by block inside the kernel.
+ * dx [rows, 2*half] in `dtype`; x_rec (may be NULL) receives the reconstructed input;
+ * dw1, dw2, db1, db2 are float32 accumulators, NOT cleared by the call (db1, db2 may be NULL). */
+int nf_revmlp_bwd(const void* y, int64_t y_stride, const void* dy, int64_t dy_stride, void* dx, int64_t dx_stride,
+                  void* x_rec, int64_t x_rec_stride, const void* w1, const void* b1, const void* w2, const void* b2,
+                  float* dw1, float* db1, float* dw2, float* db2, int64_t rows, int half, int blocks, int act,
+                  int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NF_CDNA4_H */

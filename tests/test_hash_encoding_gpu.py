@@ -1,0 +1,267 @@
+"""GPU parity of the hash-encoding kernels against the CPU oracle (through the C ABI).
+
+Tolerances: corner rows bit-exact; float32 forward rtol 1e-5 (plus an absolute
+floor of 1e-5 x the largest table magnitude, for outputs that cancel to ~0);
+backward rtol 1e-3 (atomic order differs) with atol 1e-4 for N(0,1) upstream
+gradients; 16-bit tables: the reference's own atol 1e-2 and, tighter, one ulp
+of the 16-bit result.
+"""
+import json
+import os
+
+import pytest
+import torch
+
+from oracle import hash_encoding as O
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "hash_geometry.json")))
+DEV = "cuda"
+
+
+def _hk():
+    from triton_helpers_amd.layers.hash_encoding import kernel
+
+    return kernel
+
+
+def _table(T, L, D, lo, hi, F=2, dtype=torch.float32, amp=1e-4, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    E = O.level_row_offsets(L, T, D, lo, hi)[-1]
+    return ((torch.rand(E, F, generator=g) * 2 - 1) * amp).to(dtype)
+
+
+CASES = [
+    # (N, D, F, T, L, lo, hi, scale)  -- the first six follow the reference's matrix
+    # (tests/test_layers/test_hash_encoding.py:400-410), the rest add the bench geometry and odd shapes
+    (4, 2, 2, 25, 2, 2, 4, 1.0),
+    (4, 2, 2, 81, 8, 2, 128, 1.0),
+    (4, 3, 2, 2**14, 16, 16, 512, 1.0),
+    (100, 3, 2, 2**14, 16, 16, 512, 1.0),
+    (100, 3, 2, 2**20, 16, 16, 512, 1.0),
+    (100, 3, 2, 2**14, 16, 16, 512, 2.0),
+    (4099, 3, 2, 2**19, 16, 16, 7006, 1.0),
+    (777, 3, 2, 5000, 8, 4, 300, 1.0),  # T not a power of two: exact 64-bit remainder
+    (513, 3, 4, 2**12, 4, 8, 64, 1.0),
+    (300, 1, 2, 64, 4, 8, 512, 1.0),
+    (300, 3, 1, 2**12, 8, 16, 256, 0.5),
+]
+
+
+@pytest.mark.parametrize("N,D,F,T,L,lo,hi,scale", CASES)
+def test_corner_rows_bit_exact(N, D, F, T, L, lo, hi, scale):
+    torch.manual_seed(0)
+    x = torch.rand(N, D)
+    want = O.encode_indices(x, None, T, L, lo, hi)
+    xs = x * scale if scale != 1.0 else x
+    if scale not in (1.0, 2.0):  # keep only points that survive the round trip through the scale exactly
+        keep = ((xs / scale) == x).all(1)
+        x, xs, want = x[keep], xs[keep], want[keep]
+    got, w = _hk().hash_encoding_indices(xs.to(DEV), None, T, lo, hi, L, scale=scale, return_weights=True)
+    assert torch.equal(got.cpu(), want)
+    res = O.level_resolutions(L, lo, hi)
+    wref = torch.stack([O.corner_weights(x, D, r) for r in res], 1)
+    torch.testing.assert_close(w.cpu(), wref, rtol=1e-6, atol=1e-7)
+
+
+def test_corner_rows_reference_literals():
+    """The reference's literal tables (test_hash_encoding.py:240-251, 285-296) straight from the device code."""
+    from tests.test_oracle_hash import DENSE_ROWS, HASHED_ROWS, QUADRANT_X
+
+    x = torch.tensor(QUADRANT_X, dtype=torch.float32, device=DEV)
+    # a single level of resolution 2: min_res = max_res is degenerate for the growth factor, so use L=2 and read level 0
+    dense = _hk().hash_encoding_indices(x, None, 9, 2, 4, 2)[:, 0]
+    hashed = _hk().hash_encoding_indices(x, None, 7, 2, 4, 2)[:, 0]
+    assert dense.cpu().tolist() == DENSE_ROWS
+    assert hashed.cpu().tolist() == HASHED_ROWS
+
+
+@pytest.mark.parametrize("N,D,F,T,L,lo,hi,scale", CASES)
+@pytest.mark.parametrize("force_generic", [False, True])
+def test_forward_fp32_tables(N, D, F, T, L, lo, hi, scale, force_generic, monkeypatch):
+    hk = _hk()
+    monkeypatch.setattr(hk, "_FLAGS", 1 if force_generic else 0)
+    torch.manual_seed(0)
+    x = torch.rand(N, D)
+    table = _table(T, L, D, lo, hi, F)
+    want = O.encode_forward(x, table, None, T, L, lo, hi)
+    got = hk.hash_encoding(x.to(DEV) * scale, table.to(DEV), None, None, T, lo, hi, L, scale=scale)
+    assert got.dtype == torch.float32 and got.shape == (N, L * F)
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-5 * 1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,D,F,T,L,lo,hi,scale", CASES)
+def test_forward_16bit_tables(N, D, F, T, L, lo, hi, scale, dtype):
+    hk = _hk()
+    torch.manual_seed(0)
+    x = torch.rand(N, D)
+    table = _table(T, L, D, lo, hi, F, dtype=dtype, amp=1.0)
+    want32 = O.encode_forward(x, table.float(), None, T, L, lo, hi)
+    got = hk.hash_encoding(x.to(DEV) * scale, table.to(DEV), None, None, T, lo, hi, L, scale=scale)
+    assert got.dtype == dtype
+    # reference tolerance (test_hash_encoding.py:432)
+    torch.testing.assert_close(got.cpu().float(), want32, rtol=0, atol=1e-2)
+    # tighter: the float32 result rounded once to the 16-bit type, allow one ulp
+    eps = 2.0**-10 if dtype == torch.float16 else 2.0**-7
+    torch.testing.assert_close(got.cpu().float(), want32, rtol=eps, atol=eps * 1e-3)
+
+
+def test_tiled_and_generic_agree_bitwise(monkeypatch):
+    hk = _hk()
+    g = GOLDEN["bench"]
+    torch.manual_seed(1)
+    x = torch.rand(5000, 3, device=DEV)
+    table = _table(g["T"], 16, 3, 16, 7006, dtype=torch.float16, amp=1.0).to(DEV)
+    monkeypatch.setattr(hk, "_FLAGS", 0)
+    a = hk.hash_encoding(x, table, None, None, g["T"], 16, 7006, 16)
+    monkeypatch.setattr(hk, "_FLAGS", 1)
+    b = hk.hash_encoding(x, table, None, None, g["T"], 16, 7006, 16)
+    assert torch.equal(a, b)
+
+
+def test_forward_config0_full_size():
+    """BASELINE configs[0]: N=65536, L=16, F=2, T=2^19, fp32 table U(-1e-4, 1e-4), seed 0."""
+    g = GOLDEN["bench"]
+    torch.manual_seed(0)
+    x = torch.rand(65536, 3)
+    table = (torch.rand(g["total_rows"], 2) * 2 - 1) * 1e-4
+    want = O.encode_forward(x, table, None, g["T"], 16, 16, 7006)
+    got = _hk().hash_encoding(x.to(DEV), table.to(DEV), None, None, g["T"], 16, 7006, 16)
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-9)
+    rows = _hk().hash_encoding_indices(x.to(DEV), None, g["T"], 16, 7006, 16)
+    assert torch.equal(rows.cpu(), O.encode_indices(x, None, g["T"], 16, 16, 7006))
+
+
+@pytest.mark.parametrize("N,D,F,T,L,lo,hi,scale", CASES + [(65536, 3, 2, 2**20, 16, 16, 512, 1.0), (131072, 3, 2, 2**14, 16, 16, 512, 1.0)])
+@pytest.mark.parametrize("do_dtype,force_generic", [(torch.float32, True), (torch.float16, False), (torch.float16, True)])
+def test_backward_vs_oracle(N, D, F, T, L, lo, hi, scale, do_dtype, force_generic, monkeypatch):
+    hk = _hk()
+    monkeypatch.setattr(hk, "_FLAGS", 1 if force_generic else 0)
+    torch.manual_seed(0)
+    x = torch.rand(N, D)
+    E = O.level_row_offsets(L, T, D, lo, hi)[-1]
+    do = torch.randn(N, L * F).to(do_dtype)
+    want = O.encode_backward(x, do, E, F, None, T, L, lo, hi)
+    got = hk.hash_encoding_table_grad(x.to(DEV) * scale, do.to(DEV), E, F, None, T, lo, hi, L, scale)
+    assert got.dtype == torch.float32
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-3, atol=1e-4)
+
+
+def test_autograd_round_trip_fp16_table():
+    """hash_encoding(...).backward(do) through the autograd Function: grad lands in the table's dtype."""
+    hk = _hk()
+    g = GOLDEN["default"]
+    torch.manual_seed(0)
+    x = torch.rand(2, 500, 3)
+    table = torch.randn(g["total_rows"], 2).half()
+    e = table.to(DEV).requires_grad_(True)
+    o = hk.hash_encoding(x.to(DEV), e, max_entries_per_level=g["T"])
+    assert o.shape == (2, 500, 32) and o.dtype == torch.float16
+    do = torch.randn(2, 500, 32).half()
+    o.backward(do.to(DEV))
+    assert e.grad is not None and e.grad.dtype == torch.float16
+    want = O.encode_backward(x.view(-1, 3), do.view(-1, 32), g["total_rows"], 2, None, g["T"], 16, 16, 512)
+    torch.testing.assert_close(e.grad.cpu().float(), want, rtol=2e-3, atol=2e-3)
+
+
+def test_features_are_appended_and_ignored_in_backward():
+    hk = _hk()
+    g = GOLDEN["default"]
+    torch.manual_seed(0)
+    x = torch.rand(333, 3)
+    feats = torch.randn(333, 5).half()
+    table = torch.randn(g["total_rows"], 2).half()
+    e = table.to(DEV).requires_grad_(True)
+    o = hk.hash_encoding(x.to(DEV), e, feats.to(DEV), max_entries_per_level=g["T"])
+    assert o.shape == (333, 37)
+    want = O.encode_forward(x, table.float(), None, g["T"], 16, 16, 512)
+    torch.testing.assert_close(o[:, :32].cpu().float(), want, rtol=2.0**-10, atol=1e-3)
+    assert torch.equal(o[:, 32:].cpu(), feats)
+    do = torch.randn(333, 37).half()
+    o.backward(do.to(DEV))
+    wantg = O.encode_backward(x, do[:, :32], g["total_rows"], 2, None, g["T"], 16, 16, 512)
+    torch.testing.assert_close(e.grad.cpu().float(), wantg, rtol=2e-3, atol=2e-3)
+
+
+def test_module_autocast():
+    # reference test_hash_encoding.py:507-530
+    from triton_helpers_amd.layers.hash_encoding import HashEncoding
+
+    layer = HashEncoding(2**14, 16, 3, 2, 16, 512).to(DEV)
+    x = torch.rand(16, 40, 3, device=DEV)
+    with torch.autocast(device_type="cuda", dtype=torch.float16):
+        o = layer(x)
+    assert o.dtype == torch.float16 and o.shape == (16, 40, 32)
+    layer2 = HashEncoding(2**8, 4, 3, 2, 16, 512).to(DEV)
+    with torch.autocast(device_type="cuda", dtype=torch.float16):
+        o2 = layer2(x)
+    o2.sum().backward()
+    assert layer2.embeddings.grad is not None
+    assert set(layer.state_dict().keys()) == {"embeddings", "pi"}
+
+
+def test_argument_errors():
+    hk = _hk()
+    g = GOLDEN["default"]
+    table = torch.zeros(g["total_rows"], 2, device=DEV)
+    x = torch.rand(10, 3, device=DEV)
+    with pytest.raises(AssertionError):
+        hk.hash_encoding(x.cpu(), table, max_entries_per_level=g["T"])  # mixed devices
+    with pytest.raises(AssertionError):
+        hk.hash_encoding(x, table, max_entries_per_level=g["T"], levels=12)  # not a power of two
+    with pytest.raises(ValueError):
+        hk.hash_encoding(torch.rand(10, 4, device=DEV), table, max_entries_per_level=g["T"])  # D>3 without pi
+    with pytest.raises(AssertionError):
+        hk.hash_encoding(x.long(), table, max_entries_per_level=g["T"])
+    with pytest.raises(AssertionError):
+        hk.hash_encoding(x, table[:100], max_entries_per_level=g["T"])  # table too small for the geometry
+
+
+def test_empty_and_edge_coordinates():
+    hk = _hk()
+    g = GOLDEN["default"]
+    table = _table(g["T"], 16, 3, 16, 512).to(DEV)
+    o = hk.hash_encoding(torch.empty(0, 3, device=DEV), table, max_entries_per_level=g["T"])
+    assert o.shape == (0, 32)
+    # x == scale is legal (cell N_l, corners up to N_l + 1); must match the oracle and stay in range
+    x = torch.tensor([[1.0, 1.0, 1.0], [0.0, 0.0, 0.0], [1.0, 0.0, 0.5]])
+    got = hk.hash_encoding(x.to(DEV), table, max_entries_per_level=g["T"])
+    want = O.encode_forward(x, table.cpu(), None, g["T"], 16, 16, 512)
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-9)
+
+
+def test_full_size_properties_config1():
+    """BASELINE configs[1] at full size (N=2^20): size-independent checks.
+
+    * sum over level l / feature f of the table gradient == sum_n do[n, l*F+f] (weights sum to one);
+    * linearity of the backward in do;
+    * a constant table encodes to that constant;
+    * a 4096-point sample of the full-size forward equals the oracle.
+    """
+    hk = _hk()
+    g = GOLDEN["bench"]
+    T, E = g["T"], g["total_rows"]
+    torch.manual_seed(0)
+    x = torch.rand(2**20, 3)
+    table = ((torch.rand(E, 2) * 2 - 1) * 1e-4).half()
+    do = torch.randn(2**20, 32).half()
+    xd, td, dod = x.to(DEV), table.to(DEV), do.to(DEV)
+    out = hk.hash_encoding(xd, td, None, None, T, 16, 7006, 16)
+    idx = torch.randperm(2**20)[:4096]
+    want = O.encode_forward(x[idx], table.float(), None, T, 16, 16, 7006)
+    torch.testing.assert_close(out[idx.to(DEV)].cpu().float(), want, rtol=2.0**-10, atol=1e-9)
+
+    grad = hk.hash_encoding_table_grad(xd, dod, E, 2, None, T, 16, 7006, 16)
+    offs = O.level_row_offsets(16, T, 3, 16, 7006)
+    colsum = dod.float().sum(0).cpu().double()
+    for l in range(16):
+        s = grad[offs[l] : offs[l + 1]].double().sum(0).cpu()
+        torch.testing.assert_close(s, colsum[2 * l : 2 * l + 2], rtol=1e-3, atol=0.5)
+    grad2 = hk.hash_encoding_table_grad(xd, (dod * 2), E, 2, None, T, 16, 7006, 16)
+    torch.testing.assert_close(grad2, grad * 2, rtol=1e-3, atol=1e-3)
+
+    const = torch.full((E, 2), 0.25, dtype=torch.float16, device=DEV)
+    oc = hk.hash_encoding(xd, const, None, None, T, 16, 7006, 16)
+    torch.testing.assert_close(oc.float(), torch.full_like(oc, 0.25, dtype=torch.float32), rtol=1e-3, atol=0)

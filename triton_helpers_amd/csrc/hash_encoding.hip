@@ -1,0 +1,534 @@
+// Multiresolution hash encoding for gfx950: forward gather, backward scatter-add,
+// and an index/weight dump used for bit-exact index checks.
+//
+// Arithmetic contract (follows the PyTorch path of the reference,
+// triton_helpers/layers/hash_encoding/kernel.py:448-479):
+//   pos   = fp32(x / scale) * fp32(N_l)          one rounding per operation, no FMA
+//   cell  = floor(pos),  frac = pos - floor(pos)
+//   dense level  ((N_l+1)^D <= T):  row = sum_d (cell_d + bit_d) * N_l^d
+//   hashed level:                   row = (xor_d (cell_d + bit_d) * pi_d) mod T_l   (64-bit products)
+//   weight_j = prod_d (bit_d ? frac_d : 1 - frac_d),   out = sum_j weight_j * table[row_j]
+// The file is compiled with -ffp-contract=off so that none of this is fused.
+#include "nf_common.h"
+
+namespace nf {
+
+struct DevGeom {
+  int dims, feat, levels, first_hash;
+  uint64_t max_rows;
+  int res[NF_MAX_LEVELS];
+  uint32_t rows[NF_MAX_LEVELS];
+  int64_t row_offset[NF_MAX_LEVELS];
+};
+
+// ---------------------------------------------------------------------------
+// Generic path: one thread per (point, level); any D <= 4, any F, any dtype mix.
+// ---------------------------------------------------------------------------
+template <int D>
+struct Cell {
+  uint32_t c[D];
+  float frac[D];
+};
+
+template <int D>
+__device__ __forceinline__ Cell<D> locate(const void* coords, int cdt, int64_t sn, int64_t sd, int64_t n, float scale,
+                                          int res) {
+  Cell<D> r;
+  const float fres = (float)res;
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    float x = load_as_f32(coords, n * sn + d * sd, cdt);
+    if (scale != 1.0f) x = x / scale;
+    float pos = x * fres;
+    float fl = floorf(pos);
+    r.c[d] = (uint32_t)(int)fl;
+    r.frac[d] = pos - fl;
+  }
+  return r;
+}
+
+template <int D>
+__device__ __forceinline__ uint64_t corner_row(const Cell<D>& cell, int j, bool hashed, uint32_t res, uint32_t rows,
+                                               const uint64_t* pi) {
+  if (!hashed) {
+    uint64_t idx = 0, stride = 1;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      idx += (uint64_t)(cell.c[d] + ((j >> d) & 1)) * stride;
+      stride *= res;
+    }
+    return idx;
+  }
+  uint64_t h = 0;
+#pragma unroll
+  for (int d = 0; d < D; ++d) h ^= (uint64_t)(cell.c[d] + ((j >> d) & 1)) * pi[d];
+  // power-of-two sizes take the mask; anything else the exact 64-bit remainder
+  return (rows & (rows - 1)) == 0 ? (h & (uint64_t)(rows - 1)) : (h % (uint64_t)rows);
+}
+
+template <int D>
+__device__ __forceinline__ float corner_weight(const Cell<D>& cell, int j) {
+  float w = ((j & 1) ? cell.frac[0] : 1.0f - cell.frac[0]);
+#pragma unroll
+  for (int d = 1; d < D; ++d) w = w * (((j >> d) & 1) ? cell.frac[d] : 1.0f - cell.frac[d]);
+  return w;
+}
+
+template <int D>
+__device__ __forceinline__ void load_primes(const int64_t* primes, uint64_t* pi) {
+#pragma unroll
+  for (int d = 0; d < D; ++d) pi[d] = (uint64_t)primes[d];
+}
+
+template <int D, typename TT>
+__global__ __launch_bounds__(256) void hash_fwd_generic_k(const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                          const typename TT::storage* table,
+                                                          typename TT::storage* out, int64_t out_stride, int64_t N,
+                                                          DevGeom g, const int64_t* primes, float scale) {
+  const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int l = blockIdx.y;
+  if (n >= N) return;
+  uint64_t pi[D];
+  load_primes<D>(primes, pi);
+  const bool hashed = l >= g.first_hash;
+  const Cell<D> cell = locate<D>(coords, cdt, csn, csd, n, scale, g.res[l]);
+  const typename TT::storage* tab = table + g.row_offset[l] * g.feat;
+  uint64_t rows[1 << D];
+  float w[1 << D];
+#pragma unroll
+  for (int j = 0; j < (1 << D); ++j) {
+    rows[j] = corner_row<D>(cell, j, hashed, (uint32_t)g.res[l], g.rows[l], pi);
+    w[j] = corner_weight<D>(cell, j);
+  }
+  for (int f = 0; f < g.feat; ++f) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < (1 << D); ++j) acc = acc + w[j] * TT::to_f32(tab[rows[j] * g.feat + f]);
+    out[n * out_stride + (int64_t)l * g.feat + f] = TT::from_f32(acc);
+  }
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void hash_bwd_generic_k(const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                          const void* dout, int ddt, int64_t dout_stride,
+                                                          float* dtable, int64_t N, DevGeom g, const int64_t* primes,
+                                                          float scale) {
+  const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int l = blockIdx.y;
+  if (n >= N) return;
+  uint64_t pi[D];
+  load_primes<D>(primes, pi);
+  const bool hashed = l >= g.first_hash;
+  const Cell<D> cell = locate<D>(coords, cdt, csn, csd, n, scale, g.res[l]);
+  float* tab = dtable + g.row_offset[l] * g.feat;
+  for (int f = 0; f < g.feat; ++f) {
+    const float go = load_as_f32(dout, n * dout_stride + (int64_t)l * g.feat + f, ddt);
+#pragma unroll
+    for (int j = 0; j < (1 << D); ++j) {
+      const uint64_t row = corner_row<D>(cell, j, hashed, (uint32_t)g.res[l], g.rows[l], pi);
+      unsafeAtomicAdd(tab + row * g.feat + f, corner_weight<D>(cell, j) * go);
+    }
+  }
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void hash_indices_k(const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                      int64_t* out_rows, float* out_w, int64_t N, DevGeom g,
+                                                      const int64_t* primes, float scale) {
+  const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int l = blockIdx.y;
+  if (n >= N) return;
+  uint64_t pi[D];
+  load_primes<D>(primes, pi);
+  const bool hashed = l >= g.first_hash;
+  const Cell<D> cell = locate<D>(coords, cdt, csn, csd, n, scale, g.res[l]);
+  const int64_t base = (n * g.levels + l) * (1 << D);
+#pragma unroll
+  for (int j = 0; j < (1 << D); ++j) {
+    out_rows[base + j] = (int64_t)corner_row<D>(cell, j, hashed, (uint32_t)g.res[l], g.rows[l], pi);
+    if (out_w) out_w[base + j] = corner_weight<D>(cell, j);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Tiled path: D = 3, F = 2, 16-bit tables (one table row = one dword), L % 4 == 0.
+//
+// A workgroup of 256 threads owns P = 256*PPT consecutive points and walks the
+// levels in order, so that the workgroups resident on an XCD touch the same
+// one or two level tables at a time and those stay in that XCD's L2.  Results
+// are staged in LDS as stage[level][point] (row stride P+2 dwords) and leave
+// as full 16-byte pieces of contiguous output rows; the backward stages the
+// incoming gradient rows the same way before scattering.
+// ---------------------------------------------------------------------------
+constexpr int TILE_THREADS = 256;
+
+struct Corner8 {
+  uint32_t row[8];
+};
+
+__device__ __forceinline__ Corner8 rows_d3(const uint32_t c[3], bool hashed, uint32_t res, uint32_t mask,
+                                           const uint32_t pi[3]) {
+  Corner8 r;
+  if (hashed) {
+    // (c+1)*pi == c*pi + pi in 32-bit wrap-around arithmetic; the low 32 bits of the
+    // 64-bit products are all a power-of-two modulus keeps.
+    const uint32_t x0 = c[0] * pi[0], x1 = x0 + pi[0];
+    const uint32_t y0 = c[1] * pi[1], y1 = y0 + pi[1];
+    const uint32_t z0 = c[2] * pi[2], z1 = z0 + pi[2];
+    r.row[0] = (x0 ^ y0 ^ z0) & mask;
+    r.row[1] = (x1 ^ y0 ^ z0) & mask;
+    r.row[2] = (x0 ^ y1 ^ z0) & mask;
+    r.row[3] = (x1 ^ y1 ^ z0) & mask;
+    r.row[4] = (x0 ^ y0 ^ z1) & mask;
+    r.row[5] = (x1 ^ y0 ^ z1) & mask;
+    r.row[6] = (x0 ^ y1 ^ z1) & mask;
+    r.row[7] = (x1 ^ y1 ^ z1) & mask;
+  } else {
+    const uint32_t r2 = res * res;
+    const uint32_t b = c[0] + c[1] * res + c[2] * r2;
+    r.row[0] = b;
+    r.row[1] = b + 1;
+    r.row[2] = b + res;
+    r.row[3] = b + res + 1;
+    r.row[4] = b + r2;
+    r.row[5] = b + r2 + 1;
+    r.row[6] = b + r2 + res;
+    r.row[7] = b + r2 + res + 1;
+  }
+  return r;
+}
+
+__device__ __forceinline__ void weights_d3(const float f[3], float w[8]) {
+  const float gx = 1.0f - f[0], gy = 1.0f - f[1], gz = 1.0f - f[2];
+  w[0] = (gx * gy) * gz;
+  w[1] = (f[0] * gy) * gz;
+  w[2] = (gx * f[1]) * gz;
+  w[3] = (f[0] * f[1]) * gz;
+  w[4] = (gx * gy) * f[2];
+  w[5] = (f[0] * gy) * f[2];
+  w[6] = (gx * f[1]) * f[2];
+  w[7] = (f[0] * f[1]) * f[2];
+}
+
+template <typename TT, int PPT>
+__global__ __launch_bounds__(TILE_THREADS) void hash_fwd_tiled_k(const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                                 const uint32_t* table, uint16_t* out,
+                                                                 int64_t out_stride, int64_t N, DevGeom g,
+                                                                 const int64_t* primes, float scale) {
+  constexpr int P = TILE_THREADS * PPT;
+  constexpr int LD = P + 2;
+  extern __shared__ uint32_t stage[];
+  const int t = threadIdx.x;
+  const int64_t p0 = (int64_t)blockIdx.x * P;
+  const int L = g.levels;
+
+  float x[PPT][3];
+#pragma unroll
+  for (int i = 0; i < PPT; ++i) {
+    int64_t n = p0 + t + TILE_THREADS * i;
+    if (n >= N) n = N - 1;
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+      float v = load_as_f32(coords, n * csn + d * csd, cdt);
+      x[i][d] = scale != 1.0f ? v / scale : v;
+    }
+  }
+  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], (uint32_t)primes[2]};
+
+  for (int l = 0; l < L; ++l) {
+    const uint32_t res = (uint32_t)g.res[l];
+    const float fres = (float)g.res[l];
+    const bool hashed = l >= g.first_hash;
+    const uint32_t mask = g.rows[l] - 1;
+    const uint32_t* tab = table + g.row_offset[l];
+    uint32_t v[PPT][8];
+    float w[PPT][8];
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+      uint32_t c[3];
+      float fr[3];
+#pragma unroll
+      for (int d = 0; d < 3; ++d) {
+        const float pos = x[i][d] * fres;
+        const float fl = floorf(pos);
+        c[d] = (uint32_t)(int)fl;
+        fr[d] = pos - fl;
+      }
+      const Corner8 r = rows_d3(c, hashed, res, mask, pi);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[i][j] = tab[r.row[j]];
+      weights_d3(fr, w[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+      float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        a0 = a0 + w[i][j] * TT::to_f32((uint16_t)(v[i][j] & 0xffffu));
+        a1 = a1 + w[i][j] * TT::to_f32((uint16_t)(v[i][j] >> 16));
+      }
+      stage[l * LD + t + TILE_THREADS * i] = (uint32_t)TT::from_f32(a0) | ((uint32_t)TT::from_f32(a1) << 16);
+    }
+  }
+  __syncthreads();
+
+  // Each point's L*4 bytes leave as L/4 pieces of 16 bytes; consecutive lanes take
+  // consecutive pieces, so a wave writes 1 KiB of contiguous output per instruction.
+  const int pieces = L >> 2;
+  const int total = P * pieces;
+  for (int c = t; c < total; c += TILE_THREADS) {
+    const int p = c / pieces, q = c - p * pieces;
+    const int64_t n = p0 + p;
+    if (n < N) {
+      uint4 val;
+      val.x = stage[(4 * q + 0) * LD + p];
+      val.y = stage[(4 * q + 1) * LD + p];
+      val.z = stage[(4 * q + 2) * LD + p];
+      val.w = stage[(4 * q + 3) * LD + p];
+      *reinterpret_cast<uint4*>(out + n * out_stride + 8 * q) = val;
+    }
+  }
+}
+
+template <typename GT, int PPT>
+__global__ __launch_bounds__(TILE_THREADS) void hash_bwd_tiled_k(const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                                 const uint16_t* dout, int64_t dout_stride,
+                                                                 float* dtable, int64_t N, DevGeom g,
+                                                                 const int64_t* primes, float scale) {
+  constexpr int P = TILE_THREADS * PPT;
+  constexpr int LD = P + 2;
+  extern __shared__ uint32_t stage[];
+  const int t = threadIdx.x;
+  const int64_t p0 = (int64_t)blockIdx.x * P;
+  const int L = g.levels;
+
+  const int pieces = L >> 2;
+  const int total = P * pieces;
+  for (int c = t; c < total; c += TILE_THREADS) {
+    const int p = c / pieces, q = c - p * pieces;
+    const int64_t n = p0 + p;
+    uint4 val = make_uint4(0u, 0u, 0u, 0u);
+    if (n < N) val = *reinterpret_cast<const uint4*>(dout + n * dout_stride + 8 * q);
+    stage[(4 * q + 0) * LD + p] = val.x;
+    stage[(4 * q + 1) * LD + p] = val.y;
+    stage[(4 * q + 2) * LD + p] = val.z;
+    stage[(4 * q + 3) * LD + p] = val.w;
+  }
+
+  float x[PPT][3];
+  bool valid[PPT];
+#pragma unroll
+  for (int i = 0; i < PPT; ++i) {
+    int64_t n = p0 + t + TILE_THREADS * i;
+    valid[i] = n < N;
+    if (n >= N) n = N - 1;
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+      float v = load_as_f32(coords, n * csn + d * csd, cdt);
+      x[i][d] = scale != 1.0f ? v / scale : v;
+    }
+  }
+  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], (uint32_t)primes[2]};
+  __syncthreads();
+
+  for (int l = 0; l < L; ++l) {
+    const uint32_t res = (uint32_t)g.res[l];
+    const float fres = (float)g.res[l];
+    const bool hashed = l >= g.first_hash;
+    const uint32_t mask = g.rows[l] - 1;
+    float* tab = dtable + g.row_offset[l] * 2;
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+      const uint32_t packed = stage[l * LD + t + TILE_THREADS * i];
+      // a zero upstream gradient (both features) contributes nothing
+      if (!valid[i] || (packed & 0x7fff7fffu) == 0u) continue;
+      const float g0 = GT::to_f32((uint16_t)(packed & 0xffffu));
+      const float g1 = GT::to_f32((uint16_t)(packed >> 16));
+      uint32_t c[3];
+      float fr[3];
+#pragma unroll
+      for (int d = 0; d < 3; ++d) {
+        const float pos = x[i][d] * fres;
+        const float fl = floorf(pos);
+        c[d] = (uint32_t)(int)fl;
+        fr[d] = pos - fl;
+      }
+      const Corner8 r = rows_d3(c, hashed, res, mask, pi);
+      float w[8];
+      weights_d3(fr, w);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float* dst = tab + 2 * (size_t)r.row[j];
+        unsafeAtomicAdd(dst, w[j] * g0);
+        unsafeAtomicAdd(dst + 1, w[j] * g1);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+static int make_dev_geom(const nf_hash_geom* geom, DevGeom* d) {
+  NF_REQUIRE(geom != nullptr, NF_EINVAL, "geom is NULL");
+  NF_REQUIRE(geom->dims >= 1 && geom->dims <= NF_MAX_DIMS, NF_EINVAL, "dims=%d outside 1..%d", geom->dims,
+             NF_MAX_DIMS);
+  NF_REQUIRE(geom->feat >= 1, NF_EINVAL, "feat=%d must be positive", geom->feat);
+  NF_REQUIRE(geom->levels >= 1 && geom->levels <= NF_MAX_LEVELS, NF_EINVAL, "levels=%d outside 1..%d", geom->levels,
+             NF_MAX_LEVELS);
+  d->dims = geom->dims;
+  d->feat = geom->feat;
+  d->levels = geom->levels;
+  d->first_hash = geom->first_hash_level;
+  d->max_rows = (uint64_t)geom->max_rows;
+  for (int l = 0; l < geom->levels; ++l) {
+    NF_REQUIRE(geom->res[l] >= 1, NF_EINVAL, "res[%d]=%d must be positive", l, geom->res[l]);
+    NF_REQUIRE(geom->rows[l] >= 1 && geom->rows[l] < (int64_t)1 << 32, NF_EINVAL, "rows[%d]=%lld outside 1..2^32-1", l,
+               (long long)geom->rows[l]);
+    NF_REQUIRE(geom->row_offset[l] >= 0, NF_EINVAL, "row_offset[%d] negative", l);
+    // a dense level must be able to hold every corner the stride-N_l indexing can produce
+    if (l < geom->first_hash_level) {
+      double need = 1.0;
+      for (int k = 0; k < geom->dims; ++k) need *= (double)geom->res[l] + 1.0;
+      NF_REQUIRE(need <= (double)geom->rows[l], NF_EINVAL, "level %d marked dense but (res+1)^D > rows", l);
+    }
+    d->res[l] = geom->res[l];
+    d->rows[l] = (uint32_t)geom->rows[l];
+    d->row_offset[l] = geom->row_offset[l];
+  }
+  return 0;
+}
+
+static bool tiled_ok(const nf_hash_geom* g, int table_dt, const void* rows_ptr, int64_t row_stride) {
+  if (g->dims != 3 || g->feat != 2 || table_dt == NF_F32) return false;
+  if (g->levels % 4 != 0 || g->levels > 16) return false;
+  for (int l = g->first_hash_level; l < g->levels; ++l) {
+    if (l < 0) return false;
+    const int64_t r = g->rows[l];
+    if ((r & (r - 1)) != 0) return false;
+  }
+  if (((uintptr_t)rows_ptr & 15u) != 0 || (row_stride * 2) % 16 != 0) return false;
+  return true;
+}
+
+template <int D, typename TT>
+static void launch_fwd_generic(const void* coords, int cdt, int64_t csn, int64_t csd, const void* table, void* out,
+                               int64_t out_stride, int64_t N, const DevGeom& g, const int64_t* primes, float scale,
+                               hipStream_t s) {
+  dim3 grid((unsigned)((N + 255) / 256), (unsigned)g.levels);
+  hipLaunchKernelGGL((hash_fwd_generic_k<D, TT>), grid, dim3(256), 0, s, coords, cdt, csn, csd,
+                     (const typename TT::storage*)table, (typename TT::storage*)out, out_stride, N, g, primes, scale);
+}
+
+template <int D>
+static int dispatch_fwd_generic(int table_dt, const void* coords, int cdt, int64_t csn, int64_t csd, const void* table,
+                                void* out, int64_t out_stride, int64_t N, const DevGeom& g, const int64_t* primes,
+                                float scale, hipStream_t s) {
+  switch (table_dt) {
+    case NF_F32: launch_fwd_generic<D, F32>(coords, cdt, csn, csd, table, out, out_stride, N, g, primes, scale, s); break;
+    case NF_F16: launch_fwd_generic<D, F16>(coords, cdt, csn, csd, table, out, out_stride, N, g, primes, scale, s); break;
+    default: launch_fwd_generic<D, BF16>(coords, cdt, csn, csd, table, out, out_stride, N, g, primes, scale, s); break;
+  }
+  return check_launch("hash_fwd_generic");
+}
+
+}  // namespace nf
+
+using namespace nf;
+
+extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t csn, int64_t csd, const void* table,
+                                  int table_dtype, void* out, int64_t out_stride_n, int64_t n_points,
+                                  const nf_hash_geom* geom, const int64_t* primes, float scale, int flags,
+                                  void* stream) {
+  DevGeom g;
+  if (int rc = make_dev_geom(geom, &g)) return rc;
+  NF_REQUIRE(dtype_ok(coords_dtype) && dtype_ok(table_dtype), NF_EINVAL, "unknown dtype code");
+  NF_REQUIRE(n_points >= 0, NF_EINVAL, "n_points negative");
+  NF_REQUIRE(out_stride_n >= (int64_t)g.levels * g.feat, NF_EINVAL, "out_stride_n=%lld < levels*feat",
+             (long long)out_stride_n);
+  NF_REQUIRE(scale > 0.0f, NF_EINVAL, "scale must be positive");
+  if (n_points == 0) return 0;
+  NF_REQUIRE(coords && table && out && primes, NF_EINVAL, "NULL pointer argument");
+  NF_REQUIRE(n_points <= ((int64_t)1 << 31) * 256 - 1, NF_EINVAL, "n_points too large");
+  hipStream_t s = (hipStream_t)stream;
+
+  if (!(flags & NF_HASH_FORCE_GENERIC) && tiled_ok(geom, table_dtype, out, out_stride_n)) {
+    constexpr int PPT = 2;
+    constexpr int P = TILE_THREADS * PPT;
+    const size_t lds = (size_t)g.levels * (P + 2) * sizeof(uint32_t);
+    dim3 grid((unsigned)((n_points + P - 1) / P));
+    if (table_dtype == NF_F16)
+      hipLaunchKernelGGL((hash_fwd_tiled_k<F16, PPT>), grid, dim3(TILE_THREADS), lds, s, coords, coords_dtype, csn,
+                         csd, (const uint32_t*)table, (uint16_t*)out, out_stride_n, n_points, g, primes, scale);
+    else
+      hipLaunchKernelGGL((hash_fwd_tiled_k<BF16, PPT>), grid, dim3(TILE_THREADS), lds, s, coords, coords_dtype, csn,
+                         csd, (const uint32_t*)table, (uint16_t*)out, out_stride_n, n_points, g, primes, scale);
+    return check_launch("hash_fwd_tiled");
+  }
+  switch (g.dims) {
+    case 1: return dispatch_fwd_generic<1>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
+    case 2: return dispatch_fwd_generic<2>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
+    case 3: return dispatch_fwd_generic<3>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
+    default: return dispatch_fwd_generic<4>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
+  }
+}
+
+extern "C" int nf_hash_encode_bwd(const void* coords, int coords_dtype, int64_t csn, int64_t csd, const void* dout,
+                                  int dout_dtype, int64_t dout_stride_n, float* dtable, int64_t n_points,
+                                  const nf_hash_geom* geom, const int64_t* primes, float scale, int flags,
+                                  void* stream) {
+  DevGeom g;
+  if (int rc = make_dev_geom(geom, &g)) return rc;
+  NF_REQUIRE(dtype_ok(coords_dtype) && dtype_ok(dout_dtype), NF_EINVAL, "unknown dtype code");
+  NF_REQUIRE(n_points >= 0, NF_EINVAL, "n_points negative");
+  NF_REQUIRE(dout_stride_n >= (int64_t)g.levels * g.feat, NF_EINVAL, "dout_stride_n=%lld < levels*feat",
+             (long long)dout_stride_n);
+  NF_REQUIRE(scale > 0.0f, NF_EINVAL, "scale must be positive");
+  if (n_points == 0) return 0;
+  NF_REQUIRE(coords && dout && dtable && primes, NF_EINVAL, "NULL pointer argument");
+  NF_REQUIRE(n_points <= ((int64_t)1 << 31) * 256 - 1, NF_EINVAL, "n_points too large");
+  hipStream_t s = (hipStream_t)stream;
+
+  if (!(flags & NF_HASH_FORCE_GENERIC) && tiled_ok(geom, dout_dtype, dout, dout_stride_n)) {
+    constexpr int PPT = 2;
+    constexpr int P = TILE_THREADS * PPT;
+    const size_t lds = (size_t)g.levels * (P + 2) * sizeof(uint32_t);
+    dim3 grid((unsigned)((n_points + P - 1) / P));
+    if (dout_dtype == NF_F16)
+      hipLaunchKernelGGL((hash_bwd_tiled_k<F16, PPT>), grid, dim3(TILE_THREADS), lds, s, coords, coords_dtype, csn,
+                         csd, (const uint16_t*)dout, dout_stride_n, dtable, n_points, g, primes, scale);
+    else
+      hipLaunchKernelGGL((hash_bwd_tiled_k<BF16, PPT>), grid, dim3(TILE_THREADS), lds, s, coords, coords_dtype, csn,
+                         csd, (const uint16_t*)dout, dout_stride_n, dtable, n_points, g, primes, scale);
+    return check_launch("hash_bwd_tiled");
+  }
+  dim3 grid((unsigned)((n_points + 255) / 256), (unsigned)g.levels);
+  switch (g.dims) {
+    case 1: hipLaunchKernelGGL((hash_bwd_generic_k<1>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, g, primes, scale); break;
+    case 2: hipLaunchKernelGGL((hash_bwd_generic_k<2>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, g, primes, scale); break;
+    case 3: hipLaunchKernelGGL((hash_bwd_generic_k<3>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, g, primes, scale); break;
+    default: hipLaunchKernelGGL((hash_bwd_generic_k<4>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, g, primes, scale); break;
+  }
+  return check_launch("hash_bwd_generic");
+}
+
+extern "C" int nf_hash_encode_indices(const void* coords, int coords_dtype, int64_t csn, int64_t csd,
+                                      int64_t* out_rows, float* out_w, int64_t n_points, const nf_hash_geom* geom,
+                                      const int64_t* primes, float scale, void* stream) {
+  DevGeom g;
+  if (int rc = make_dev_geom(geom, &g)) return rc;
+  NF_REQUIRE(dtype_ok(coords_dtype), NF_EINVAL, "unknown dtype code");
+  NF_REQUIRE(n_points >= 0, NF_EINVAL, "n_points negative");
+  NF_REQUIRE(scale > 0.0f, NF_EINVAL, "scale must be positive");
+  if (n_points == 0) return 0;
+  NF_REQUIRE(coords && out_rows && primes, NF_EINVAL, "NULL pointer argument");
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid((unsigned)((n_points + 255) / 256), (unsigned)g.levels);
+  switch (g.dims) {
+    case 1: hipLaunchKernelGGL((hash_indices_k<1>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, out_rows, out_w, n_points, g, primes, scale); break;
+    case 2: hipLaunchKernelGGL((hash_indices_k<2>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, out_rows, out_w, n_points, g, primes, scale); break;
+    case 3: hipLaunchKernelGGL((hash_indices_k<3>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, out_rows, out_w, n_points, g, primes, scale); break;
+    default: hipLaunchKernelGGL((hash_indices_k<4>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, out_rows, out_w, n_points, g, primes, scale); break;
+  }
+  return check_launch("hash_indices");
+}
