@@ -1,0 +1,197 @@
+"""GPU parity of the fused MLP against the CPU oracle (through the C ABI).
+
+Tolerance: rtol 2e-2 / atol 1e-2 on y, dx and every dw/db for 16-bit storage, against the
+float32 oracle evaluated on the 16-bit-rounded inputs and weights (the way the reference's tests
+compare its kernel with a float32 ``nn.Linear`` chain, tests/test_layers/test_fully_fused_mlp.py:253-289,
+whose own tolerance is 1e-2).  Weight gradients summed over many rows are compared relative to
+their scale (rtol on the tensor's max magnitude).
+"""
+import pytest
+import torch
+import torch.nn as nn
+
+from oracle import mlp as M
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+RTOL, ATOL = 2e-2, 1e-2
+
+
+def _mk():
+    from triton_helpers_amd.layers.fully_fused_mlp import kernel
+
+    return kernel
+
+
+def _params(d_in, d_hidden, d_out, depth, bias, dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+
+    def u(shape, fan_in):
+        return ((torch.rand(*shape, generator=g) * 2 - 1) / fan_in**0.5).to(dtype)
+
+    p = dict(w_in=u((d_hidden, d_in), d_in), w_out=u((d_out, d_hidden), d_hidden))
+    p["b_in"] = u((d_hidden,), d_in) if bias else None
+    p["b_out"] = u((d_out,), d_hidden) if bias else None
+    if depth > 1:
+        p["w_hid"] = u(((depth - 1) * d_hidden, d_hidden), d_hidden)
+        p["b_hid"] = u((depth - 1, d_hidden), d_hidden) if bias else None
+    else:
+        p["w_hid"] = p["b_hid"] = None
+    return p
+
+
+def _dev(t):
+    return None if t is None else t.to(DEV)
+
+
+def _close(got, want, what, scale_rel=False):
+    got, want = got.detach().cpu().float(), want.float()
+    atol = ATOL
+    if scale_rel:
+        atol = max(ATOL, RTOL * float(want.abs().max()))
+    torch.testing.assert_close(got, want, rtol=RTOL, atol=atol, msg=lambda m: f"{what}: {m}")
+
+
+SHAPES = [
+    # rows(B,L), d_in, d_hidden, d_out, depth
+    ((3, 40), 1, 32, 5, 1),     # reference test_forward_shallow
+    ((3, 40), 1, 32, 5, 8),     # reference test_forward_deep
+    ((2, 2), 8, 16, 4, 1),      # reference test_backward_shallow
+    ((2, 2), 8, 16, 4, 3),      # reference test_backward_deep
+    ((2, 2), 8, 16, 4, 8),
+    ((1, 1000), 32, 64, 16, 2),  # BASELINE configs[2] geometry
+    ((1, 4097), 32, 64, 4, 2),   # BASELINE configs[4] geometry, ragged rows
+    ((5, 77), 64, 64, 64, 4),
+    ((2, 33), 17, 32, 33, 2),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("act", ["relu", "silu", "relu2", "none"])
+@pytest.mark.parametrize("bias", [True, False])
+@pytest.mark.parametrize("shape,d_in,d_hidden,d_out,depth", SHAPES)
+def test_forward_backward(shape, d_in, d_hidden, d_out, depth, bias, act, dtype):
+    mk = _mk()
+    torch.manual_seed(0)
+    p = _params(d_in, d_hidden, d_out, depth, bias, dtype)
+    x = torch.randn(*shape, d_in).to(dtype)
+    dy = torch.randn(*shape, d_out).to(dtype)
+    want_y = M.mlp_forward(x.float().view(-1, d_in), p["w_in"], p["b_in"], p["w_out"], p["b_out"], p["w_hid"], p["b_hid"], act)
+    want = M.mlp_backward(x.view(-1, d_in), dy.view(-1, d_out), p["w_in"], p["b_in"], p["w_out"], p["b_out"], p["w_hid"], p["b_hid"], act)
+
+    leaves = {k: (None if v is None else v.to(DEV).requires_grad_(True)) for k, v in p.items()}
+    xd = x.to(DEV).requires_grad_(True)
+    y = mk.fully_fused_mlp(xd, leaves["w_in"], leaves["b_in"], leaves["w_out"], leaves["b_out"], leaves["w_hid"], leaves["b_hid"], act)
+    assert y.shape == (*shape, d_out) and y.dtype == dtype
+    _close(y.view(-1, d_out), want_y, "y")
+    y.backward(dy.to(DEV))
+    _close(xd.grad.view(-1, d_in), want["dx"], "dx")
+    for k in ("w_in", "b_in", "w_out", "b_out", "w_hid", "b_hid"):
+        if leaves[k] is None:
+            continue
+        _close(leaves[k].grad, want["d" + k], "d" + k, scale_rel=True)
+
+
+def test_config2_sample_vs_oracle():
+    """BASELINE configs[2] (32->64->64->16, ReLU, bf16, no bias) on 65536 rows against the oracle."""
+    mk = _mk()
+    torch.manual_seed(0)
+    p = _params(32, 64, 16, 2, False, torch.bfloat16)
+    rows = 65536
+    x = torch.randn(1, rows, 32).bfloat16()
+    dy = torch.randn(1, rows, 16).bfloat16()
+    want_y = M.mlp_forward(x.view(-1, 32), p["w_in"], None, p["w_out"], None, p["w_hid"], None, "relu")
+    want = M.mlp_backward(x.view(-1, 32), dy.view(-1, 16), p["w_in"], None, p["w_out"], None, p["w_hid"], None, "relu")
+    leaves = {k: (None if v is None else v.to(DEV).requires_grad_(True)) for k, v in p.items()}
+    xd = x.to(DEV).requires_grad_(True)
+    y = mk.fully_fused_mlp(xd, leaves["w_in"], None, leaves["w_out"], None, leaves["w_hid"], None)
+    _close(y.view(-1, 16), want_y, "y")
+    y.backward(dy.to(DEV))
+    _close(xd.grad.view(-1, 32), want["dx"], "dx")
+    for k in ("w_in", "w_out", "w_hid"):
+        _close(leaves[k].grad, want["d" + k], "d" + k, scale_rel=True)
+
+
+def test_full_size_properties_config2():
+    """configs[2] at 2^20 rows: linearity of the backward in dy, additivity of dW over row halves,
+    and forward agreement of a 4096-row sample with the oracle."""
+    mk = _mk()
+    torch.manual_seed(0)
+    p = {k: _dev(v) for k, v in _params(32, 64, 16, 2, False, torch.bfloat16).items()}
+    rows = 2**20
+    x = torch.randn(1, rows, 32, device=DEV).bfloat16()
+    dy = torch.randn(1, rows, 16, device=DEV).bfloat16()
+
+    def grads(xx, dd):
+        leaves = {k: (None if v is None else v.detach().clone().requires_grad_(True)) for k, v in p.items()}
+        xr = xx.detach().clone().requires_grad_(True)
+        y = mk.fully_fused_mlp(xr, leaves["w_in"], None, leaves["w_out"], None, leaves["w_hid"], None)
+        y.backward(dd)
+        return y, xr.grad, {k: leaves[k].grad.float() for k in ("w_in", "w_out", "w_hid")}
+
+    y, dx, dw = grads(x, dy)
+    idx = torch.randperm(rows)[:4096]
+    cpu = {k: (None if v is None else v.cpu()) for k, v in p.items()}
+    want = M.mlp_forward(x[0, idx.to(DEV)].cpu(), cpu["w_in"], None, cpu["w_out"], None, cpu["w_hid"], None, "relu")
+    _close(y[0, idx.to(DEV)], want, "y sample")
+    half = rows // 2
+    _, _, dwa = grads(x[:, :half], dy[:, :half])
+    _, _, dwb = grads(x[:, half:], dy[:, half:])
+    for k in dw:
+        s = dwa[k] + dwb[k]
+        torch.testing.assert_close(dw[k], s, rtol=RTOL, atol=RTOL * float(s.abs().max()))
+    _, dx2, _ = grads(x, dy * 2)
+    torch.testing.assert_close(dx2.float(), dx.float() * 2, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("depth", [1, 4, 8])
+def test_module_autocast(depth):
+    # reference test_module (test_fully_fused_mlp.py:372-415): same seed => same init as an nn.Linear chain
+    from triton_helpers_amd.layers.fully_fused_mlp import FullyFusedMLP
+
+    torch.manual_seed(0)
+    x = torch.randn(2, 2, 8, device=DEV, requires_grad=True)
+    torch.manual_seed(0)
+    lin_in = nn.Linear(8, 16)
+    lin_hid = [nn.Linear(16, 16) for _ in range(depth - 1)]
+    lin_out = nn.Linear(16, 4)
+    torch.manual_seed(0)
+    layer = FullyFusedMLP(8, 16, 4, depth=depth).to(DEV)
+    assert torch.equal(layer.w_in.cpu(), lin_in.weight) and torch.equal(layer.b_out.cpu(), lin_out.bias)
+    if depth > 1:
+        assert torch.equal(layer.w_hid.cpu(), torch.cat([l.weight for l in lin_hid], 0))
+    with torch.autocast(device_type="cuda", dtype=torch.float16):
+        y = layer(x)
+    assert y.dtype == torch.float16
+    y.sum().backward()
+    ref_net = nn.Sequential(lin_in, nn.ReLU(), *[m for l in lin_hid for m in (l, nn.ReLU())], lin_out)
+    xc = x.detach().cpu().requires_grad_(True)
+    yr = ref_net(xc)
+    yr.sum().backward()
+    _close(y, yr.detach(), "y")
+    _close(x.grad, xc.grad, "dx")
+    _close(layer.w_in.grad, lin_in.weight.grad, "dw_in", scale_rel=True)
+    _close(layer.b_in.grad, lin_in.bias.grad, "db_in", scale_rel=True)
+    _close(layer.w_out.grad, lin_out.weight.grad, "dw_out", scale_rel=True)
+    _close(layer.b_out.grad, lin_out.bias.grad, "db_out", scale_rel=True)
+    expect = {"w_in", "b_in", "w_out", "b_out"} | ({"w_hid", "b_hid"} if depth > 1 else set())
+    assert set(layer.state_dict().keys()) == expect
+
+
+def test_argument_errors():
+    mk = _mk()
+    p = {k: _dev(v) for k, v in _params(8, 16, 4, 1, True, torch.float16).items()}
+    x = torch.randn(2, 3, 8, device=DEV).half()
+    with pytest.raises(AssertionError):
+        mk.fully_fused_mlp(x[..., :7], p["w_in"], p["b_in"], p["w_out"], p["b_out"])  # input dim mismatch
+    with pytest.raises(AssertionError):
+        mk.fully_fused_mlp(x, p["w_in"], p["b_in"], p["w_out"], p["b_out"], activation="tanh")
+    with pytest.raises(ValueError):
+        mk.fully_fused_mlp(x[0], p["w_in"], p["b_in"], p["w_out"], p["b_out"])  # x must be 3-D
+    with pytest.raises(NotImplementedError):
+        mk.fully_fused_mlp(x.float(), *(p[k].float() for k in ("w_in", "b_in", "w_out", "b_out")))
+    w24 = torch.zeros(24, 8, device=DEV).half()
+    with pytest.raises(AssertionError):
+        mk.fully_fused_mlp(x, w24, None, torch.zeros(4, 24, device=DEV).half(), None)  # hidden not a power of 2
+    y = mk.fully_fused_mlp(x[:, :0], p["w_in"], p["b_in"], p["w_out"], p["b_out"])
+    assert y.shape == (2, 0, 4)

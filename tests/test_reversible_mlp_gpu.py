@@ -1,0 +1,114 @@
+"""GPU parity of the reversible MLP against the CPU oracle (through the C ABI).
+
+The reference holds no reversible MLP, so parity with the reference is UNPINNED for this layer; the
+oracle is pinned by mathematics (tests/test_oracle_mlp.py).  Tolerance: rtol 2e-2 / atol 1e-2 on y,
+dx and (relative to their scale) dw/db, float32 oracle on the 16-bit-rounded inputs.
+"""
+import pytest
+import torch
+
+from oracle import reversible as R
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+RTOL, ATOL = 2e-2, 1e-2
+
+
+def _rk():
+    from triton_helpers_amd.layers.reversible_mlp import kernel
+
+    return kernel
+
+
+def _params(blocks, H, bias, dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    u = lambda *s: ((torch.rand(*s, generator=g) * 2 - 1) / H**0.5).to(dtype)  # noqa: E731
+    return u(blocks * 2 * H, H), (u(blocks * 2, H) if bias else None), u(blocks * 2 * H, H), (u(blocks * 2, H) if bias else None)
+
+
+def _close(got, want, what, scale_rel=False):
+    got, want = got.detach().cpu().float(), want.float()
+    atol = max(ATOL, RTOL * float(want.abs().max())) if scale_rel else ATOL
+    torch.testing.assert_close(got, want, rtol=RTOL, atol=atol, msg=lambda m: f"{what}: {m}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("act", ["gelu", "relu", "silu"])
+@pytest.mark.parametrize("bias", [False, True])
+@pytest.mark.parametrize("rows,H,blocks", [(1000, 64, 4), (37, 64, 1), (300, 32, 2), (129, 16, 3), (513, 64, 6), (64, 20, 2)])
+def test_forward_backward(rows, H, blocks, bias, act, dtype):
+    rk = _rk()
+    torch.manual_seed(0)
+    w1, b1, w2, b2 = _params(blocks, H, bias, dtype)
+    x = torch.randn(rows, 2 * H).to(dtype)
+    dy = torch.randn(rows, 2 * H).to(dtype)
+    want_y = R.rev_forward(x, w1, b1, w2, b2, act)
+    want = R.rev_backward(x, dy, w1, b1, w2, b2, act)
+    leaves = [None if t is None else t.to(DEV).requires_grad_(True) for t in (w1, b1, w2, b2)]
+    xd = x.to(DEV).requires_grad_(True)
+    y = rk.reversible_mlp(xd, *leaves, act)
+    assert y.shape == x.shape and y.dtype == dtype
+    _close(y, want_y, "y")
+    y.backward(dy.to(DEV))
+    _close(xd.grad, want["dx"], "dx")
+    for name, leaf in zip(("dw1", "db1", "dw2", "db2"), leaves):
+        if leaf is not None:
+            _close(leaf.grad, want[name], name, scale_rel=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_inverse_round_trip(dtype):
+    """inverse(forward(x)) == x up to the 16-bit rounding of the stream (the in-kernel reconstruction)."""
+    rk = _rk()
+    torch.manual_seed(0)
+    w1, b1, w2, b2 = (None if t is None else t.to(DEV) for t in _params(4, 64, True, dtype))
+    x = torch.randn(3, 700, 128, device=DEV).to(dtype)
+    y = rk.reversible_mlp(x, w1, b1, w2, b2)
+    xr = rk.reversible_mlp_inverse(y, w1, b1, w2, b2)
+    eps = 2.0**-7 if dtype == torch.bfloat16 else 2.0**-10
+    torch.testing.assert_close(xr.float(), x.float(), rtol=8 * eps, atol=8 * eps)
+
+
+def test_full_size_config3_properties():
+    """BASELINE configs[3] at 2^20 rows: round trip, linearity of dx in dy, and a 2048-row sample against the oracle."""
+    rk = _rk()
+    torch.manual_seed(0)
+    w1, b1, w2, b2 = _params(4, 64, False, torch.bfloat16)
+    dev = [None if t is None else t.to(DEV) for t in (w1, b1, w2, b2)]
+    rows = 2**20
+    x = torch.randn(rows, 128, device=DEV).bfloat16()
+    y = rk.reversible_mlp(x, *dev)
+    idx = torch.randperm(rows)[:2048].to(DEV)
+    _close(y[idx], R.rev_forward(x[idx].cpu(), w1, b1, w2, b2), "y sample")
+    xr = rk.reversible_mlp_inverse(y, *dev)
+    torch.testing.assert_close(xr.float(), x.float(), rtol=2.0**-4, atol=2.0**-4)
+    dy = torch.randn(rows, 128, device=DEV).bfloat16()
+    xg = x.clone().requires_grad_(True)
+    rk.reversible_mlp(xg, *dev).backward(dy)
+    xg2 = x.clone().requires_grad_(True)
+    rk.reversible_mlp(xg2, *dev).backward(dy * 2)
+    torch.testing.assert_close(xg2.grad.float(), xg.grad.float() * 2, rtol=RTOL, atol=ATOL)
+    want = R.rev_backward(x[idx].cpu(), dy[idx].cpu(), w1, b1, w2, b2)
+    _close(xg.grad[idx], want["dx"], "dx sample")
+
+
+def test_module_and_errors():
+    from triton_helpers_amd.layers.reversible_mlp import ReversibleMLP
+
+    rk = _rk()
+    torch.manual_seed(0)
+    layer = ReversibleMLP(128, 4).to(DEV)
+    x = torch.randn(2, 50, 128, device=DEV, requires_grad=True)
+    with torch.autocast(device_type="cuda", dtype=torch.float16):
+        y = layer(x)
+    assert y.dtype == torch.float16 and y.shape == x.shape
+    y.sum().backward()
+    assert layer.w1.grad is not None and layer.b2.grad is not None and x.grad is not None
+    assert set(layer.state_dict().keys()) == {"w1", "w2", "b1", "b2"}
+    w = torch.zeros(256, 64, device=DEV).half()
+    with pytest.raises(AssertionError):
+        rk.reversible_mlp(torch.zeros(4, 127, device=DEV).half(), w, None, w, None)
+    with pytest.raises(AssertionError):
+        rk.reversible_mlp(torch.zeros(4, 128, device=DEV).half(), w[:100], None, w[:100], None)
+    with pytest.raises(NotImplementedError):
+        rk.reversible_mlp(torch.zeros(4, 128, device=DEV), w.float(), None, w.float(), None)

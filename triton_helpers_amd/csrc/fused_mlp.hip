@@ -1,3 +1,714 @@
-#include "nf_common.h"
-extern "C" int nf_mlp_fwd(const void*, int64_t, void*, int64_t, const void*, const void*, const void*, const void*, const void*, const void*, int64_t, int, int, int, int, int, int, void*) { return nf::fail(NF_EUNSUPPORTED, "nf_mlp_fwd not built yet"); }
-extern "C" int nf_mlp_bwd(const void*, int64_t, const void*, int64_t, void*, int64_t, const void*, const void*, const void*, const void*, const void*, const void*, float*, float*, float*, float*, float*, float*, int64_t, int, int, int, int, int, int, void*) { return nf::fail(NF_EUNSUPPORTED, "nf_mlp_bwd not built yet"); }
+// Fully fused MLP for gfx950: forward and backward, 16-bit storage (bf16 / fp16),
+// float32 accumulation on v_mfma_f32_16x16x32.
+//
+// Layer math follows triton_helpers/layers/fully_fused_mlp/kernel.py:17-74 of the reference:
+//   z = x W^T + b (float32 accumulate), h = act(z) rounded to the storage type, no activation
+//   after the output layer; backward dz = act'(z) * dh, dW = dz^T h_prev, dh_prev = dz W.
+//
+// Forward: weights are staged once per workgroup into LDS as MFMA A fragments; each wave
+// walks 32-row chunks and keeps every activation in registers (see mlp_tile.h).
+// Backward: the forward is recomputed once per chunk from x; each layer's input is parked
+// in LDS transposed ([feature][row]) so that dW = dZ^T H can read both operands as
+// K = 32 data rows; act'(z) is parked as a register image.  Weight gradients accumulate in
+// float32 registers over the wave's whole row loop (up to REG_HIDDEN hidden layers), are
+// reduced across the workgroup through LDS and leave with one coalesced atomic add per
+// 64-byte segment; deeper nets add the hidden-layer partials to memory chunk by chunk.
+#include "mlp_tile.h"
+
+namespace nf {
+
+struct MlpArgs {
+  const uint16_t* x;
+  int64_t x_stride;
+  uint16_t* y;
+  int64_t y_stride;
+  const uint16_t* dy;
+  int64_t dy_stride;
+  uint16_t* dx;
+  int64_t dx_stride;
+  const uint16_t *w_in, *b_in, *w_hid, *b_hid, *w_out, *b_out;
+  float *dw_in, *db_in, *dw_hid, *db_hid, *dw_out, *db_out;
+  int64_t rows;
+  int d_in, d_hidden, d_out, depth, act;
+  int x_vec, y_vec, dy_vec, dx_vec;
+  int waves;  // waves per workgroup
+};
+
+constexpr int FRAG_ELEMS = 64 * 8;  // 16-bit elements per fragment (1 KiB)
+constexpr int TPITCH = 40;          // 16-bit elements per feature row of a transposed 32-row panel (80 B)
+
+template <typename T>
+__device__ __forceinline__ void stage_bias(float* dst, const uint16_t* b, int n_valid, int n_pad, int tid, int nthreads) {
+  for (int i = tid; i < n_pad; i += nthreads) dst[i] = (b != nullptr && i < n_valid) ? T::to_f32(b[i]) : 0.0f;
+}
+
+// acc[nt][mt] = bias + W(frags) * in[nt][kc]
+template <typename T, int MT, int KC>
+__device__ __forceinline__ void layer_mma(f32x4_t (&acc)[2][4], const Frag (&in)[2][2], const uint16_t* frags,
+                                          const float* bias, int lane) {
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(bias + 16 * mt + 4 * (lane >> 4));
+    acc[0][mt] = b4;
+    acc[1][mt] = b4;
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc) {
+      const Frag a = lds_frag(frags, mt * KC + kc, lane);
+      acc[0][mt] = mfma16<T>(a, in[0][kc], acc[0][mt]);
+      acc[1][mt] = mfma16<T>(a, in[1][kc], acc[1][mt]);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Forward
+// ---------------------------------------------------------------------------------------
+template <typename T, int KIN, int HP, int OUTP>
+__global__ __launch_bounds__(256) void mlp_fwd_k(MlpArgs a) {
+  constexpr int KC_IN = KIN / 32, KC_H = HP / 32, MT_H = HP / 16, MT_O = OUTP / 16;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n_hid = a.depth - 1;
+
+  uint16_t* f_in = reinterpret_cast<uint16_t*>(smem);
+  uint16_t* f_hid = f_in + MT_H * KC_IN * FRAG_ELEMS;
+  uint16_t* f_out = f_hid + (size_t)n_hid * MT_H * KC_H * FRAG_ELEMS;
+  float* bias_in = reinterpret_cast<float*>(f_out + MT_O * KC_H * FRAG_ELEMS);
+  float* bias_hid = bias_in + HP;
+  float* bias_out = bias_hid + (size_t)n_hid * HP;
+
+  stage_weight_frags<false, false>(f_in, a.w_in, a.d_hidden, a.d_in, MT_H, KC_IN, tid, nthreads);
+  for (int k = 0; k < n_hid; ++k)
+    stage_weight_frags<true, false>(f_hid + (size_t)k * MT_H * KC_H * FRAG_ELEMS,
+                                    a.w_hid + (size_t)k * a.d_hidden * a.d_hidden, a.d_hidden, a.d_hidden, MT_H, KC_H,
+                                    tid, nthreads);
+  stage_weight_frags<true, false>(f_out, a.w_out, a.d_out, a.d_hidden, MT_O, KC_H, tid, nthreads);
+  stage_bias<T>(bias_in, a.b_in, a.d_hidden, HP, tid, nthreads);
+  for (int k = 0; k < n_hid; ++k)
+    stage_bias<T>(bias_hid + k * HP, a.b_hid ? a.b_hid + (size_t)k * a.d_hidden : nullptr, a.d_hidden, HP, tid, nthreads);
+  stage_bias<T>(bias_out, a.b_out, a.d_out, OUTP, tid, nthreads);
+  __syncthreads();
+
+  const int64_t n_chunks = (a.rows + 31) / 32;
+  const int64_t wave_stride = (int64_t)gridDim.x * a.waves;
+  for (int64_t chunk = (int64_t)blockIdx.x * a.waves + wave; chunk < n_chunks; chunk += wave_stride) {
+    const int64_t row0 = chunk * 32;
+    Frag in[2][2];
+    f32x4_t acc[2][4];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int kc = 0; kc < KC_IN; ++kc)
+        in[nt][kc] = load_rows_frag(a.x, a.x_stride, row0 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+
+    layer_mma<T, MT_H, KC_IN>(acc, in, f_in, bias_in, lane);
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int kc = 0; kc < KC_H; ++kc) {
+        const f32x4_t lo = acc[nt][2 * kc], hi = acc[nt][2 * kc + 1];
+        in[nt][kc].w[0] = pack2<T>(act_fwd(lo[0], a.act), act_fwd(lo[1], a.act));
+        in[nt][kc].w[1] = pack2<T>(act_fwd(lo[2], a.act), act_fwd(lo[3], a.act));
+        in[nt][kc].w[2] = pack2<T>(act_fwd(hi[0], a.act), act_fwd(hi[1], a.act));
+        in[nt][kc].w[3] = pack2<T>(act_fwd(hi[2], a.act), act_fwd(hi[3], a.act));
+      }
+    for (int k = 0; k < n_hid; ++k) {
+      layer_mma<T, MT_H, KC_H>(acc, in, f_hid + (size_t)k * MT_H * KC_H * FRAG_ELEMS, bias_hid + k * HP, lane);
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int kc = 0; kc < KC_H; ++kc) {
+          const f32x4_t lo = acc[nt][2 * kc], hi = acc[nt][2 * kc + 1];
+          in[nt][kc].w[0] = pack2<T>(act_fwd(lo[0], a.act), act_fwd(lo[1], a.act));
+          in[nt][kc].w[1] = pack2<T>(act_fwd(lo[2], a.act), act_fwd(lo[3], a.act));
+          in[nt][kc].w[2] = pack2<T>(act_fwd(hi[0], a.act), act_fwd(hi[1], a.act));
+          in[nt][kc].w[3] = pack2<T>(act_fwd(hi[2], a.act), act_fwd(hi[3], a.act));
+        }
+    }
+    layer_mma<T, MT_O, KC_H>(acc, in, f_out, bias_out, lane);
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT_O; ++mt)
+        store_rows_tile<T>(a.y, a.y_stride, row0 + 16 * nt, a.rows, a.d_out, mt, lane, acc[nt][mt], a.y_vec);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Backward
+// ---------------------------------------------------------------------------------------
+// Park an accumulator-layout tile (lane (n,g): features 16*mt + 4*g + r of row 16*nt + n) into a
+// transposed panel panel[feature][row].
+__device__ __forceinline__ void park_tile_T(uint16_t* panel, int mt, int nt, int lane, uint32_t p01, uint32_t p23) {
+  const int n = (lane & 15) + 16 * nt;
+  const int f = 16 * mt + 4 * (lane >> 4);
+  panel[(f + 0) * TPITCH + n] = (uint16_t)(p01 & 0xffffu);
+  panel[(f + 1) * TPITCH + n] = (uint16_t)(p01 >> 16);
+  panel[(f + 2) * TPITCH + n] = (uint16_t)(p23 & 0xffffu);
+  panel[(f + 3) * TPITCH + n] = (uint16_t)(p23 >> 16);
+}
+// Park a natural-order fragment (lane (n,g): features 32*kc + 8*g + j of row 16*nt + n).
+__device__ __forceinline__ void park_frag_T(uint16_t* panel, int kc, int nt, int lane, const Frag& f) {
+  const int n = (lane & 15) + 16 * nt;
+  const int c = 32 * kc + 8 * (lane >> 4);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    panel[(c + 2 * j) * TPITCH + n] = (uint16_t)(f.w[j] & 0xffffu);
+    panel[(c + 2 * j + 1) * TPITCH + n] = (uint16_t)(f.w[j] >> 16);
+  }
+}
+// Operand of a K = 32-rows product: lane (i, g) reads rows 8*g .. 8*g+7 of feature 16*t + i.
+__device__ __forceinline__ Frag panel_frag(const uint16_t* panel, int t, int lane) {
+  Frag f;
+  f.u = *reinterpret_cast<const uint4*>(panel + (16 * t + (lane & 15)) * TPITCH + 8 * (lane >> 4));
+  return f;
+}
+
+// dW tile (mt over output features, nt over input features): lane (n, g) reg r is
+// dW[16*mt + 4*g + r][16*nt + n].
+__device__ __forceinline__ void flush_dw_tile(float* dw, int out_dim, int in_dim, int mt, int nt, int lane, f32x4_t v) {
+  const int c = 16 * nt + (lane & 15);
+  const int r0 = 16 * mt + 4 * (lane >> 4);
+  if (c >= in_dim) return;
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+    if (r0 + r < out_dim) unsafeAtomicAdd(dw + (size_t)(r0 + r) * in_dim + c, v[r]);
+}
+
+template <typename T, int KIN, int HP, int OUTP, int REG_HIDDEN>
+__global__ __launch_bounds__(256) void mlp_bwd_k(MlpArgs a) {
+  constexpr int KC_IN = KIN / 32, KC_H = HP / 32, MT_H = HP / 16, MT_I = KIN / 16, MT_O = OUTP / 16;
+  constexpr int KC_O = (OUTP + 31) / 32;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n_hid = a.depth - 1;
+  const bool regs_hold_hidden = n_hid <= REG_HIDDEN;
+
+  // ---- LDS carve-up: weights (forward + transposed), biases, then per-wave panels ----
+  uint16_t* f_in = reinterpret_cast<uint16_t*>(smem);                            // [MT_H][KC_IN]
+  uint16_t* f_hid = f_in + MT_H * KC_IN * FRAG_ELEMS;                            // [n_hid][MT_H][KC_H]
+  uint16_t* t_in = f_hid + (size_t)n_hid * MT_H * KC_H * FRAG_ELEMS;             // W_in^T  [MT_I][KC_H]
+  uint16_t* t_hid = t_in + MT_I * KC_H * FRAG_ELEMS;                             // W_hid^T [n_hid][MT_H][KC_H]
+  uint16_t* t_out = t_hid + (size_t)n_hid * MT_H * KC_H * FRAG_ELEMS;            // W_out^T [MT_H][KC_O]
+  float* bias_in = reinterpret_cast<float*>(t_out + MT_H * KC_O * FRAG_ELEMS);   // [HP]
+  float* bias_hid = bias_in + HP;                                                // [n_hid][HP]
+  uint16_t* wave_base = reinterpret_cast<uint16_t*>(bias_hid + (size_t)n_hid * HP);
+  // per wave: x^T [KIN], h_k^T [depth][HP], dz^T [max(HP,OUTP32)], act' images [depth][MT_H*2*2*64 dwords]
+  constexpr int DZ_FEATS = HP > 32 * KC_O ? HP : 32 * KC_O;
+  const size_t panel_elems = (size_t)(KIN + (size_t)a.depth * HP + DZ_FEATS) * TPITCH;
+  const size_t image_elems = (size_t)a.depth * MT_H * 2 * 2 * 64 * 2;  // in 16-bit units
+  const size_t per_wave = panel_elems + image_elems;
+  uint16_t* xT = wave_base + (size_t)wave * per_wave;
+  uint16_t* hT = xT + KIN * TPITCH;                   // hT + (k-1)*HP*TPITCH : h_k^T, k = 1..depth
+  uint16_t* dzT = hT + (size_t)a.depth * HP * TPITCH;
+  uint32_t* img = reinterpret_cast<uint32_t*>(dzT + DZ_FEATS * TPITCH);  // [depth][MT_H][2 nt][2][64]
+
+  stage_weight_frags<false, false>(f_in, a.w_in, a.d_hidden, a.d_in, MT_H, KC_IN, tid, nthreads);
+  stage_weight_frags<true, true>(t_in, a.w_in, a.d_hidden, a.d_in, MT_I, KC_H, tid, nthreads);
+  for (int k = 0; k < n_hid; ++k) {
+    const uint16_t* w = a.w_hid + (size_t)k * a.d_hidden * a.d_hidden;
+    stage_weight_frags<true, false>(f_hid + (size_t)k * MT_H * KC_H * FRAG_ELEMS, w, a.d_hidden, a.d_hidden, MT_H, KC_H, tid, nthreads);
+    stage_weight_frags<true, true>(t_hid + (size_t)k * MT_H * KC_H * FRAG_ELEMS, w, a.d_hidden, a.d_hidden, MT_H, KC_H, tid, nthreads);
+  }
+  stage_weight_frags<false, true>(t_out, a.w_out, a.d_out, a.d_hidden, MT_H, KC_O, tid, nthreads);
+  stage_bias<T>(bias_in, a.b_in, a.d_hidden, HP, tid, nthreads);
+  for (int k = 0; k < n_hid; ++k)
+    stage_bias<T>(bias_hid + k * HP, a.b_hid ? a.b_hid + (size_t)k * a.d_hidden : nullptr, a.d_hidden, HP, tid, nthreads);
+  // zero the padding rows of the dz panel once (features >= what a layer writes are read as zero operands)
+  for (int i = lane; i < DZ_FEATS * TPITCH; i += 64) dzT[i] = 0;
+  __syncthreads();
+
+  f32x4_t dw_in[MT_H][MT_I];
+  f32x4_t dw_out[MT_O][MT_H];
+  f32x4_t dw_hid[REG_HIDDEN > 0 ? REG_HIDDEN : 1][MT_H][MT_H];
+  f32x4_t db_acc_in[MT_H], db_acc_hid[REG_HIDDEN > 0 ? REG_HIDDEN : 1][MT_H];
+  const f32x4_t zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int i = 0; i < MT_H; ++i) {
+    db_acc_in[i] = zero4;
+#pragma unroll
+    for (int j = 0; j < MT_I; ++j) dw_in[i][j] = zero4;
+  }
+#pragma unroll
+  for (int i = 0; i < MT_O; ++i)
+#pragma unroll
+    for (int j = 0; j < MT_H; ++j) dw_out[i][j] = zero4;
+#pragma unroll
+  for (int h = 0; h < (REG_HIDDEN > 0 ? REG_HIDDEN : 1); ++h)
+#pragma unroll
+    for (int i = 0; i < MT_H; ++i) {
+      db_acc_hid[h][i] = zero4;
+#pragma unroll
+      for (int j = 0; j < MT_H; ++j) dw_hid[h][i][j] = zero4;
+    }
+  const bool want_db = a.db_in != nullptr || a.db_hid != nullptr;  // db_out is a separate pass over dy
+
+  const int64_t n_chunks = (a.rows + 31) / 32;
+  const int64_t wave_stride = (int64_t)gridDim.x * a.waves;
+  for (int64_t chunk = (int64_t)blockIdx.x * a.waves + wave; chunk < n_chunks; chunk += wave_stride) {
+    const int64_t row0 = chunk * 32;
+    Frag in[2][2];
+    f32x4_t acc[2][4];
+
+    // ---------------- forward recompute; park inputs (transposed) and act'(z) ----------------
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int kc = 0; kc < KC_IN; ++kc) {
+        in[nt][kc] = load_rows_frag(a.x, a.x_stride, row0 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+        park_frag_T(xT, kc, nt, lane, in[nt][kc]);
+      }
+    for (int k = 1; k <= a.depth; ++k) {
+      if (k == 1)
+        layer_mma<T, MT_H, KC_IN>(acc, in, f_in, bias_in, lane);
+      else
+        layer_mma<T, MT_H, KC_H>(acc, in, f_hid + (size_t)(k - 2) * MT_H * KC_H * FRAG_ELEMS, bias_hid + (k - 2) * HP, lane);
+      uint16_t* panel = hT + (size_t)(k - 1) * HP * TPITCH;
+      uint32_t* im = img + (size_t)(k - 1) * MT_H * 2 * 2 * 64;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT_H; ++mt) {
+          const f32x4_t z = acc[nt][mt];
+          const uint32_t h01 = pack2<T>(act_fwd(z[0], a.act), act_fwd(z[1], a.act));
+          const uint32_t h23 = pack2<T>(act_fwd(z[2], a.act), act_fwd(z[3], a.act));
+          in[nt][mt >> 1].w[2 * (mt & 1)] = h01;
+          in[nt][mt >> 1].w[2 * (mt & 1) + 1] = h23;
+          park_tile_T(panel, mt, nt, lane, h01, h23);
+          im[((mt * 2 + nt) * 2 + 0) * 64 + lane] = pack2<T>(act_grad(z[0], a.act), act_grad(z[1], a.act));
+          im[((mt * 2 + nt) * 2 + 1) * 64 + lane] = pack2<T>(act_grad(z[2], a.act), act_grad(z[3], a.act));
+        }
+    }
+
+    // ---------------- output layer: dz_out = dy ----------------
+    Frag dz[2][2];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int kc = 0; kc < KC_O; ++kc) {
+        dz[nt][kc] = load_rows_frag(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
+        park_frag_T(dzT, kc, nt, lane, dz[nt][kc]);
+      }
+    {
+      const uint16_t* hprev = hT + (size_t)(a.depth - 1) * HP * TPITCH;
+      Frag hb[MT_H];
+#pragma unroll
+      for (int j = 0; j < MT_H; ++j) hb[j] = panel_frag(hprev, j, lane);
+#pragma unroll
+      for (int i = 0; i < MT_O; ++i) {
+        const Frag da = panel_frag(dzT, i, lane);
+#pragma unroll
+        for (int j = 0; j < MT_H; ++j) dw_out[i][j] = mfma16<T>(da, hb[j], dw_out[i][j]);
+      }
+      // dh_depth = W_out^T dy
+#pragma unroll
+      for (int mt = 0; mt < MT_H; ++mt) {
+        acc[0][mt] = zero4;
+        acc[1][mt] = zero4;
+#pragma unroll
+        for (int kc = 0; kc < KC_O; ++kc) {
+          const Frag wa = lds_frag(t_out, mt * KC_O + kc, lane);
+          acc[0][mt] = mfma16<T>(wa, dz[0][kc], acc[0][mt]);
+          acc[1][mt] = mfma16<T>(wa, dz[1][kc], acc[1][mt]);
+        }
+      }
+    }
+
+    // ---------------- hidden layers (k = depth .. 2) and the input layer (k = 1) ----------------
+    for (int k = a.depth; k >= 1; --k) {
+      // dz_k = dh_k * act'(z_k), rounded to the storage type; park transposed
+      const uint32_t* im = img + (size_t)(k - 1) * MT_H * 2 * 2 * 64;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT_H; ++mt) {
+          const uint32_t g01 = im[((mt * 2 + nt) * 2 + 0) * 64 + lane];
+          const uint32_t g23 = im[((mt * 2 + nt) * 2 + 1) * 64 + lane];
+          const f32x4_t dh = acc[nt][mt];
+          const float d0 = dh[0] * unpack_lo<T>(g01), d1 = dh[1] * unpack_hi<T>(g01);
+          const float d2 = dh[2] * unpack_lo<T>(g23), d3 = dh[3] * unpack_hi<T>(g23);
+          const uint32_t p01 = pack2<T>(d0, d1), p23 = pack2<T>(d2, d3);
+          dz[nt][mt >> 1].w[2 * (mt & 1)] = p01;
+          dz[nt][mt >> 1].w[2 * (mt & 1) + 1] = p23;
+          park_tile_T(dzT, mt, nt, lane, p01, p23);
+          if (want_db) {
+            const f32x4_t dzv = {unpack_lo<T>(p01), unpack_hi<T>(p01), unpack_lo<T>(p23), unpack_hi<T>(p23)};
+            if (k == 1) {
+              db_acc_in[mt] += dzv;
+            } else if (regs_hold_hidden) {
+#pragma unroll
+              for (int h = 0; h < REG_HIDDEN; ++h)
+                if (h == k - 2) db_acc_hid[h][mt] += dzv;
+            } else if (a.db_hid != nullptr) {
+              // deep nets: fold the 16 rows of this tile now and add to memory
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                float t = dzv[r];
+                t += __shfl_xor(t, 1);
+                t += __shfl_xor(t, 2);
+                t += __shfl_xor(t, 4);
+                t += __shfl_xor(t, 8);
+                const int f = 16 * mt + 4 * (lane >> 4) + r;
+                if ((lane & 15) == 0 && f < a.d_hidden) unsafeAtomicAdd(a.db_hid + (size_t)(k - 2) * a.d_hidden + f, t);
+              }
+            }
+          }
+        }
+      if (k == 1) {
+        // dW_in += dz_1^T x ; dx = W_in^T dz_1
+        Frag xb[MT_I];
+#pragma unroll
+        for (int j = 0; j < MT_I; ++j) xb[j] = panel_frag(xT, j, lane);
+#pragma unroll
+        for (int i = 0; i < MT_H; ++i) {
+          const Frag da = panel_frag(dzT, i, lane);
+#pragma unroll
+          for (int j = 0; j < MT_I; ++j) dw_in[i][j] = mfma16<T>(da, xb[j], dw_in[i][j]);
+        }
+        if (a.dx != nullptr) {
+#pragma unroll
+          for (int mt = 0; mt < MT_I; ++mt) {
+            f32x4_t o0 = zero4, o1 = zero4;
+#pragma unroll
+            for (int kc = 0; kc < KC_H; ++kc) {
+              const Frag wa = lds_frag(t_in, mt * KC_H + kc, lane);
+              o0 = mfma16<T>(wa, dz[0][kc], o0);
+              o1 = mfma16<T>(wa, dz[1][kc], o1);
+            }
+            store_rows_tile<T>(a.dx, a.dx_stride, row0, a.rows, a.d_in, mt, lane, o0, a.dx_vec);
+            store_rows_tile<T>(a.dx, a.dx_stride, row0 + 16, a.rows, a.d_in, mt, lane, o1, a.dx_vec);
+          }
+        }
+      } else {
+        // hidden layer k-2: dW += dz_k^T h_{k-1} ; dh_{k-1} = W^T dz_k
+        const uint16_t* hprev = hT + (size_t)(k - 2) * HP * TPITCH;
+        Frag hb[MT_H];
+#pragma unroll
+        for (int j = 0; j < MT_H; ++j) hb[j] = panel_frag(hprev, j, lane);
+        if (regs_hold_hidden) {
+#pragma unroll
+          for (int h = 0; h < REG_HIDDEN; ++h)
+            if (h == k - 2) {
+#pragma unroll
+              for (int i = 0; i < MT_H; ++i) {
+                const Frag da = panel_frag(dzT, i, lane);
+#pragma unroll
+                for (int j = 0; j < MT_H; ++j) dw_hid[h][i][j] = mfma16<T>(da, hb[j], dw_hid[h][i][j]);
+              }
+            }
+        } else {
+          float* dst = a.dw_hid + (size_t)(k - 2) * a.d_hidden * a.d_hidden;
+#pragma unroll
+          for (int i = 0; i < MT_H; ++i) {
+            const Frag da = panel_frag(dzT, i, lane);
+#pragma unroll
+            for (int j = 0; j < MT_H; ++j)
+              flush_dw_tile(dst, a.d_hidden, a.d_hidden, i, j, lane, mfma16<T>(da, hb[j], zero4));
+          }
+        }
+        const uint16_t* wt = t_hid + (size_t)(k - 2) * MT_H * KC_H * FRAG_ELEMS;
+#pragma unroll
+        for (int mt = 0; mt < MT_H; ++mt) {
+          f32x4_t o0 = zero4, o1 = zero4;
+#pragma unroll
+          for (int kc = 0; kc < KC_H; ++kc) {
+            const Frag wa = lds_frag(wt, mt * KC_H + kc, lane);
+            o0 = mfma16<T>(wa, dz[0][kc], o0);
+            o1 = mfma16<T>(wa, dz[1][kc], o1);
+          }
+          acc[0][mt] = o0;
+          acc[1][mt] = o1;
+        }
+      }
+    }
+  }
+
+  // ---------------- reduce the weight gradients over the workgroup, then one atomic pass ----------------
+  // Reuse the (now idle) per-wave region as a float staging buffer, one wave at a time.
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(wave_base);
+  for (int w = 1; w < a.waves; ++w) {
+    if (wave == w) {
+      int t = 0;
+#pragma unroll
+      for (int i = 0; i < MT_H; ++i)
+#pragma unroll
+        for (int j = 0; j < MT_I; ++j) *reinterpret_cast<f32x4_t*>(red + ((t++) * 64 + lane) * 4) = dw_in[i][j];
+#pragma unroll
+      for (int i = 0; i < MT_O; ++i)
+#pragma unroll
+        for (int j = 0; j < MT_H; ++j) *reinterpret_cast<f32x4_t*>(red + ((t++) * 64 + lane) * 4) = dw_out[i][j];
+#pragma unroll
+      for (int h = 0; h < (REG_HIDDEN > 0 ? REG_HIDDEN : 1); ++h)
+#pragma unroll
+        for (int i = 0; i < MT_H; ++i)
+#pragma unroll
+          for (int j = 0; j < MT_H; ++j) *reinterpret_cast<f32x4_t*>(red + ((t++) * 64 + lane) * 4) = dw_hid[h][i][j];
+#pragma unroll
+      for (int i = 0; i < MT_H; ++i) *reinterpret_cast<f32x4_t*>(red + ((t++) * 64 + lane) * 4) = db_acc_in[i];
+#pragma unroll
+      for (int h = 0; h < (REG_HIDDEN > 0 ? REG_HIDDEN : 1); ++h)
+#pragma unroll
+        for (int i = 0; i < MT_H; ++i) *reinterpret_cast<f32x4_t*>(red + ((t++) * 64 + lane) * 4) = db_acc_hid[h][i];
+    }
+    __syncthreads();
+    if (wave == 0) {
+      int t = 0;
+#pragma unroll
+      for (int i = 0; i < MT_H; ++i)
+#pragma unroll
+        for (int j = 0; j < MT_I; ++j) dw_in[i][j] += *reinterpret_cast<const f32x4_t*>(red + ((t++) * 64 + lane) * 4);
+#pragma unroll
+      for (int i = 0; i < MT_O; ++i)
+#pragma unroll
+        for (int j = 0; j < MT_H; ++j) dw_out[i][j] += *reinterpret_cast<const f32x4_t*>(red + ((t++) * 64 + lane) * 4);
+#pragma unroll
+      for (int h = 0; h < (REG_HIDDEN > 0 ? REG_HIDDEN : 1); ++h)
+#pragma unroll
+        for (int i = 0; i < MT_H; ++i)
+#pragma unroll
+          for (int j = 0; j < MT_H; ++j) dw_hid[h][i][j] += *reinterpret_cast<const f32x4_t*>(red + ((t++) * 64 + lane) * 4);
+#pragma unroll
+      for (int i = 0; i < MT_H; ++i) db_acc_in[i] += *reinterpret_cast<const f32x4_t*>(red + ((t++) * 64 + lane) * 4);
+#pragma unroll
+      for (int h = 0; h < (REG_HIDDEN > 0 ? REG_HIDDEN : 1); ++h)
+#pragma unroll
+        for (int i = 0; i < MT_H; ++i) db_acc_hid[h][i] += *reinterpret_cast<const f32x4_t*>(red + ((t++) * 64 + lane) * 4);
+    }
+    __syncthreads();
+  }
+  if (wave != 0) return;
+
+#pragma unroll
+  for (int i = 0; i < MT_H; ++i)
+#pragma unroll
+    for (int j = 0; j < MT_I; ++j) flush_dw_tile(a.dw_in, a.d_hidden, a.d_in, i, j, lane, dw_in[i][j]);
+#pragma unroll
+  for (int i = 0; i < MT_O; ++i)
+#pragma unroll
+    for (int j = 0; j < MT_H; ++j) flush_dw_tile(a.dw_out, a.d_out, a.d_hidden, i, j, lane, dw_out[i][j]);
+  if (regs_hold_hidden) {
+#pragma unroll
+    for (int h = 0; h < REG_HIDDEN; ++h)
+      if (h < n_hid) {
+        float* dst = a.dw_hid + (size_t)h * a.d_hidden * a.d_hidden;
+#pragma unroll
+        for (int i = 0; i < MT_H; ++i)
+#pragma unroll
+          for (int j = 0; j < MT_H; ++j) flush_dw_tile(dst, a.d_hidden, a.d_hidden, i, j, lane, dw_hid[h][i][j]);
+      }
+  }
+  if (want_db) {
+    // hidden / input biases: lane (n,g) reg r holds the partial sum of feature 16*mt + 4*g + r over its rows n
+    auto fold_store = [&](f32x4_t s, int mt, float* dst, int width) {
+      if (dst == nullptr) return;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float t = s[r];
+        t += __shfl_xor(t, 1);
+        t += __shfl_xor(t, 2);
+        t += __shfl_xor(t, 4);
+        t += __shfl_xor(t, 8);
+        const int f = 16 * mt + 4 * (lane >> 4) + r;
+        if ((lane & 15) == 0 && f < width) unsafeAtomicAdd(dst + f, t);
+      }
+    };
+#pragma unroll
+    for (int mt = 0; mt < MT_H; ++mt) fold_store(db_acc_in[mt], mt, a.db_in, a.d_hidden);
+    if (regs_hold_hidden) {
+#pragma unroll
+      for (int h = 0; h < REG_HIDDEN; ++h)
+        if (h < n_hid && a.db_hid != nullptr) {
+#pragma unroll
+          for (int mt = 0; mt < MT_H; ++mt) fold_store(db_acc_hid[h][mt], mt, a.db_hid + (size_t)h * a.d_hidden, a.d_hidden);
+        }
+    }
+  }
+}
+
+// db_out = column sums of dy; tiny and memory-bound, done apart from the fused kernel.
+template <typename T>
+__global__ __launch_bounds__(256) void db_out_k(const uint16_t* dy, int64_t stride, int64_t rows, int d_out, float* db_out) {
+  __shared__ float part[256];
+  const int c = threadIdx.x % 64;  // column handled (d_out <= 64)
+  const int rl = threadIdx.x / 64;
+  float s = 0.0f;
+  if (c < d_out)
+    for (int64_t r = (int64_t)blockIdx.x * 4 + rl; r < rows; r += (int64_t)gridDim.x * 4) s += T::to_f32(dy[r * stride + c]);
+  part[threadIdx.x] = s;
+  __syncthreads();
+  if (rl == 0 && c < d_out) unsafeAtomicAdd(db_out + c, part[c] + part[64 + c] + part[128 + c] + part[192 + c]);
+}
+
+// ---------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------
+static int pad_to(int v, int m) { return (v + m - 1) / m * m; }
+
+static int validate(int64_t rows, int d_in, int d_hidden, int d_out, int depth, int act, int dtype) {
+  NF_REQUIRE(rows >= 0, NF_EINVAL, "rows negative");
+  NF_REQUIRE(d_in >= 1 && d_in <= 64, NF_EINVAL, "d_in=%d outside 1..64", d_in);
+  NF_REQUIRE(d_out >= 1 && d_out <= 64, NF_EINVAL, "d_out=%d outside 1..64", d_out);
+  NF_REQUIRE(d_hidden >= 16 && d_hidden <= 64 && (d_hidden & (d_hidden - 1)) == 0, NF_EINVAL,
+             "d_hidden=%d must be 16, 32 or 64", d_hidden);
+  NF_REQUIRE(depth >= 1, NF_EINVAL, "depth=%d must be >= 1", depth);
+  NF_REQUIRE(act >= NF_ACT_NONE && act <= NF_ACT_GELU, NF_EINVAL, "unknown activation %d", act);
+  NF_REQUIRE(dtype == NF_F16 || dtype == NF_BF16, NF_EUNSUPPORTED,
+             "dtype code %d: the fused MLP kernels take float16 or bfloat16 storage", dtype);
+  return 0;
+}
+
+static int device_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) cus = p.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+constexpr size_t LDS_LIMIT = 160 * 1024;
+
+template <typename T, int KIN, int HP, int OUTP>
+static int launch_fwd(const MlpArgs& a0, hipStream_t s) {
+  MlpArgs a = a0;
+  const int n_hid = a.depth - 1;
+  const size_t lds = ((size_t)(HP / 16) * (KIN / 32) + (size_t)n_hid * (HP / 16) * (HP / 32) + (size_t)(OUTP / 16) * (HP / 32)) * 1024 +
+                     ((size_t)HP + (size_t)n_hid * HP + OUTP) * 4;
+  NF_REQUIRE(lds <= LDS_LIMIT, NF_EUNSUPPORTED, "weights of depth %d need %zu B of LDS (limit %zu)", a.depth, lds, LDS_LIMIT);
+  a.waves = 4;
+  const int64_t chunks = (a.rows + 31) / 32;
+  int64_t blocks = (chunks + a.waves - 1) / a.waves;
+  const int64_t cap = (int64_t)device_cus() * (lds > 64 * 1024 ? 1 : 2);
+  if (blocks > cap) blocks = cap;
+  auto kern = mlp_fwd_k<T, KIN, HP, OUTP>;
+  if (lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(64 * a.waves), lds, s, a);
+  return check_launch("mlp_fwd");
+}
+
+template <typename T, int KIN, int HP, int OUTP, int REG_HIDDEN>
+static int launch_bwd(const MlpArgs& a0, hipStream_t s) {
+  MlpArgs a = a0;
+  constexpr int KC_O = (OUTP + 31) / 32;
+  constexpr int DZ_FEATS = HP > 32 * KC_O ? HP : 32 * KC_O;
+  const int n_hid = a.depth - 1;
+  const size_t w_bytes = ((size_t)(HP / 16) * (KIN / 32) + (size_t)(KIN / 16) * (HP / 32) + 2 * (size_t)n_hid * (HP / 16) * (HP / 32) +
+                          (size_t)(HP / 16) * KC_O) * 1024 + ((size_t)HP + (size_t)n_hid * HP) * 4;
+  const size_t per_wave = ((size_t)(KIN + (size_t)a.depth * HP + DZ_FEATS) * TPITCH + (size_t)a.depth * (HP / 16) * 2 * 2 * 64 * 2) * 2;
+  // staging area for the cross-wave reduction (one wave's accumulators)
+  const size_t red_bytes = ((size_t)(HP / 16) * (KIN / 16) + (size_t)(OUTP / 16) * (HP / 16) +
+                            (size_t)(REG_HIDDEN > 0 ? REG_HIDDEN : 1) * (HP / 16) * (HP / 16) + (HP / 16) + (OUTP / 16) +
+                            (size_t)(REG_HIDDEN > 0 ? REG_HIDDEN : 1) * (HP / 16)) * 64 * 16;
+  int waves = 4;
+  while (waves > 1 && w_bytes + waves * per_wave > LDS_LIMIT) waves >>= 1;
+  size_t lds = w_bytes + waves * per_wave;
+  if (waves > 1 && lds < w_bytes + red_bytes) lds = w_bytes + red_bytes;
+  NF_REQUIRE(lds <= LDS_LIMIT, NF_EUNSUPPORTED, "backward of depth %d needs %zu B of LDS (limit %zu)", a.depth, lds, LDS_LIMIT);
+  a.waves = waves;
+  const int64_t chunks = (a.rows + 31) / 32;
+  int64_t blocks = (chunks + waves - 1) / waves;
+  const int64_t cap = (int64_t)device_cus() * (lds > 80 * 1024 ? 1 : 2);
+  if (blocks > cap) blocks = cap;
+  auto kern = mlp_bwd_k<T, KIN, HP, OUTP, REG_HIDDEN>;
+  if (lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(64 * waves), lds, s, a);
+  if (int rc = check_launch("mlp_bwd")) return rc;
+  if (a.db_out != nullptr) {
+    int64_t b = (a.rows + 1023) / 1024;
+    if (b > 1024) b = 1024;
+    hipLaunchKernelGGL((db_out_k<T>), dim3((unsigned)b), dim3(256), 0, s, a.dy, a.dy_stride, a.rows, a.d_out, a.db_out);
+    return check_launch("db_out");
+  }
+  return 0;
+}
+
+template <typename T>
+static int dispatch_fwd(const MlpArgs& a, hipStream_t s) {
+  const int kin = pad_to(a.d_in, 32), hp = a.d_hidden <= 32 ? 32 : 64, outp = a.d_out <= 16 ? 16 : 64;
+  if (kin == 32 && hp == 64 && outp == 16) return launch_fwd<T, 32, 64, 16>(a, s);
+  if (kin == 32 && hp == 64) return launch_fwd<T, 32, 64, 64>(a, s);
+  if (kin == 64 && hp == 64 && outp == 16) return launch_fwd<T, 64, 64, 16>(a, s);
+  if (kin == 64 && hp == 64) return launch_fwd<T, 64, 64, 64>(a, s);
+  if (kin == 32 && outp == 16) return launch_fwd<T, 32, 32, 16>(a, s);
+  if (kin == 32) return launch_fwd<T, 32, 32, 64>(a, s);
+  if (outp == 16) return launch_fwd<T, 64, 32, 16>(a, s);
+  return launch_fwd<T, 64, 32, 64>(a, s);
+}
+
+template <typename T, int REG_HIDDEN>
+static int dispatch_bwd2(const MlpArgs& a, hipStream_t s) {
+  const int kin = pad_to(a.d_in, 32), hp = a.d_hidden <= 32 ? 32 : 64, outp = a.d_out <= 16 ? 16 : 64;
+  if (kin == 32 && hp == 64 && outp == 16) return launch_bwd<T, 32, 64, 16, REG_HIDDEN>(a, s);
+  if (kin == 32 && hp == 64) return launch_bwd<T, 32, 64, 64, REG_HIDDEN>(a, s);
+  if (kin == 64 && hp == 64 && outp == 16) return launch_bwd<T, 64, 64, 16, REG_HIDDEN>(a, s);
+  if (kin == 64 && hp == 64) return launch_bwd<T, 64, 64, 64, REG_HIDDEN>(a, s);
+  if (kin == 32 && outp == 16) return launch_bwd<T, 32, 32, 16, REG_HIDDEN>(a, s);
+  if (kin == 32) return launch_bwd<T, 32, 32, 64, REG_HIDDEN>(a, s);
+  if (outp == 16) return launch_bwd<T, 64, 32, 16, REG_HIDDEN>(a, s);
+  return launch_bwd<T, 64, 32, 64, REG_HIDDEN>(a, s);
+}
+
+template <typename T>
+static int dispatch_bwd(const MlpArgs& a, hipStream_t s) {
+  // one hidden layer's dW fits in registers next to dW_in / dW_out; deeper nets use the memory path
+  return a.depth - 1 <= 1 ? dispatch_bwd2<T, 1>(a, s) : dispatch_bwd2<T, 0>(a, s);
+}
+
+}  // namespace nf
+
+using namespace nf;
+
+extern "C" int nf_mlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_stride, const void* w_in, const void* b_in,
+                          const void* w_hid, const void* b_hid, const void* w_out, const void* b_out, int64_t rows,
+                          int d_in, int d_hidden, int d_out, int depth, int act, int dtype, void* stream) {
+  if (int rc = validate(rows, d_in, d_hidden, d_out, depth, act, dtype)) return rc;
+  if (rows == 0) return 0;
+  NF_REQUIRE(x && y && w_in && w_out, NF_EINVAL, "NULL pointer argument");
+  NF_REQUIRE(depth == 1 || w_hid, NF_EINVAL, "w_hid is NULL but depth=%d", depth);
+  NF_REQUIRE(x_stride >= d_in && y_stride >= d_out, NF_EINVAL, "row stride smaller than row width");
+  MlpArgs a = {};
+  a.x = (const uint16_t*)x; a.x_stride = x_stride; a.y = (uint16_t*)y; a.y_stride = y_stride;
+  a.w_in = (const uint16_t*)w_in; a.b_in = (const uint16_t*)b_in; a.w_hid = (const uint16_t*)w_hid;
+  a.b_hid = (const uint16_t*)b_hid; a.w_out = (const uint16_t*)w_out; a.b_out = (const uint16_t*)b_out;
+  a.rows = rows; a.d_in = d_in; a.d_hidden = d_hidden; a.d_out = d_out; a.depth = depth; a.act = act;
+  a.x_vec = vec_load_ok(x, x_stride, d_in);
+  a.y_vec = vec_store_ok(y, y_stride, d_out);
+  hipStream_t s = (hipStream_t)stream;
+  return dtype == NF_BF16 ? dispatch_fwd<BF16>(a, s) : dispatch_fwd<F16>(a, s);
+}
+
+extern "C" int nf_mlp_bwd(const void* x, int64_t x_stride, const void* dy, int64_t dy_stride, void* dx, int64_t dx_stride,
+                          const void* w_in, const void* b_in, const void* w_hid, const void* b_hid, const void* w_out,
+                          const void* b_out, float* dw_in, float* db_in, float* dw_hid, float* db_hid, float* dw_out,
+                          float* db_out, int64_t rows, int d_in, int d_hidden, int d_out, int depth, int act, int dtype,
+                          void* stream) {
+  if (int rc = validate(rows, d_in, d_hidden, d_out, depth, act, dtype)) return rc;
+  if (rows == 0) return 0;
+  NF_REQUIRE(x && dy && w_in && w_out && dw_in && dw_out, NF_EINVAL, "NULL pointer argument");
+  NF_REQUIRE(depth == 1 || (w_hid && dw_hid), NF_EINVAL, "w_hid / dw_hid is NULL but depth=%d", depth);
+  NF_REQUIRE(x_stride >= d_in && dy_stride >= d_out && (dx == nullptr || dx_stride >= d_in), NF_EINVAL,
+             "row stride smaller than row width");
+  MlpArgs a = {};
+  a.x = (const uint16_t*)x; a.x_stride = x_stride; a.dy = (const uint16_t*)dy; a.dy_stride = dy_stride;
+  a.dx = (uint16_t*)dx; a.dx_stride = dx_stride;
+  a.w_in = (const uint16_t*)w_in; a.b_in = (const uint16_t*)b_in; a.w_hid = (const uint16_t*)w_hid;
+  a.b_hid = (const uint16_t*)b_hid; a.w_out = (const uint16_t*)w_out; a.b_out = (const uint16_t*)b_out;
+  a.dw_in = dw_in; a.db_in = db_in; a.dw_hid = dw_hid; a.db_hid = db_hid; a.dw_out = dw_out; a.db_out = db_out;
+  a.rows = rows; a.d_in = d_in; a.d_hidden = d_hidden; a.d_out = d_out; a.depth = depth; a.act = act;
+  a.x_vec = vec_load_ok(x, x_stride, d_in);
+  a.dy_vec = vec_load_ok(dy, dy_stride, d_out);
+  a.dx_vec = dx ? vec_store_ok(dx, dx_stride, d_in) : 0;
+  hipStream_t s = (hipStream_t)stream;
+  return dtype == NF_BF16 ? dispatch_bwd<BF16>(a, s) : dispatch_bwd<F16>(a, s);
+}

@@ -1,0 +1,167 @@
+// Building blocks shared by the fused-MLP and reversible-MLP kernels (gfx950, wave64).
+//
+// All matmuls run on v_mfma_f32_16x16x32_{bf16,f16}.  Activations are kept
+// "row-per-lane":   for a tile of 16 data rows, lane l = (n, g) with n = l % 16 the
+// data row and g = l / 16 one of four lane groups.
+//
+//   * A layer computes  D^T = W * X^T :  A operand = weights (M = output feature),
+//     B operand = activations (N = data row), so an accumulator tile `mt` leaves
+//     lane (n, g) holding output features 16*mt + 4*g + r, r = 0..3, of row n.
+//   * Packing those four values to 16 bit gives two dwords; the tiles 2*kc and
+//     2*kc+1 together are exactly the B operand of K-chunk kc of the next layer,
+//     provided the next layer's weights are laid out with the same K order
+//     ("chain order", k_chain()).  No cross-lane traffic between layers.
+//   * Operands that come straight from global memory use the natural K order
+//     (k_nat()): lane (n, g) loads 8 consecutive features 32*kc + 8*g .. +7.
+//
+// Weights live in LDS as ready-made A fragments: fragment (mt, kc) is 64 lanes x
+// 16 bytes, lane (m, g) holding W[16*mt + m][k(kc, g, 0..7)].
+#pragma once
+
+#include "nf_common.h"
+
+namespace nf {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+union Frag {
+  uint4 u;
+  uint32_t w[4];
+  bf16x8_t b;
+  f16x8_t h;
+};
+
+template <typename T>
+__device__ __forceinline__ f32x4_t mfma16(const Frag& a, const Frag& b, f32x4_t c);
+template <>
+__device__ __forceinline__ f32x4_t mfma16<BF16>(const Frag& a, const Frag& b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b.b, c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x4_t mfma16<F16>(const Frag& a, const Frag& b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, c, 0, 0, 0);
+}
+
+// K-slot -> feature maps (kc = 32-wide chunk, g = lane group, j = element 0..7)
+__host__ __device__ __forceinline__ int k_nat(int kc, int g, int j) { return 32 * kc + 8 * g + j; }
+__host__ __device__ __forceinline__ int k_chain(int kc, int g, int j) { return 32 * kc + 16 * (j >> 2) + 4 * g + (j & 3); }
+
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  return (uint32_t)T::from_f32(lo) | ((uint32_t)T::from_f32(hi) << 16);
+}
+template <typename T>
+__device__ __forceinline__ float unpack_lo(uint32_t v) { return T::to_f32((uint16_t)(v & 0xffffu)); }
+template <typename T>
+__device__ __forceinline__ float unpack_hi(uint32_t v) { return T::to_f32((uint16_t)(v >> 16)); }
+
+// ---- activations (triton_helpers/ops.py:37-66 of the reference; gelu = exact erf form) ----
+__device__ __forceinline__ float act_fwd(float z, int act) {
+  switch (act) {
+    case NF_ACT_RELU: return z < 0.0f ? 0.0f : z;
+    case NF_ACT_SILU: return z / (1.0f + __expf(-z));
+    case NF_ACT_RELU2: return fmaxf(z, 0.0f) * z;
+    case NF_ACT_GELU: return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
+    default: return z;
+  }
+}
+// derivative d act / d z
+__device__ __forceinline__ float act_grad(float z, int act) {
+  switch (act) {
+    case NF_ACT_RELU: return z > 0.0f ? 1.0f : 0.0f;
+    case NF_ACT_SILU: {
+      const float s = 1.0f / (1.0f + __expf(-z));
+      return s * (z * (1.0f - s) + 1.0f);
+    }
+    case NF_ACT_RELU2: return z > 0.0f ? 2.0f * z : 0.0f;
+    case NF_ACT_GELU: {
+      const float cdf = 0.5f * (1.0f + erff(z * 0.70710678118654752f));
+      const float pdf = 0.3989422804014327f * __expf(-0.5f * z * z);
+      return cdf + z * pdf;
+    }
+    default: return 1.0f;
+  }
+}
+
+// ---- staging weights into LDS as A fragments ------------------------------------------
+// dst: fragment array [MT][KC][64 lanes][8 elements]; element (mt, kc, lane(m,g), j) =
+//   transposed ? W[kmap(kc,g,j)][16*mt+m] : W[16*mt+m][kmap(kc,g,j)]
+// where W is [w_rows][w_cols] row-major; out-of-range entries are zero.
+template <bool CHAIN, bool TRANSPOSED>
+__device__ __forceinline__ void stage_weight_frags(uint16_t* dst, const uint16_t* w, int w_rows, int w_cols, int MT,
+                                                   int KC, int tid, int nthreads) {
+  const int total = MT * KC * 64 * 8;
+  for (int e = tid; e < total; e += nthreads) {
+    const int j = e & 7;
+    const int lane = (e >> 3) & 63;
+    const int frag = e >> 9;
+    const int kc = frag % KC, mt = frag / KC;
+    const int m = 16 * mt + (lane & 15);
+    const int g = lane >> 4;
+    const int k = CHAIN ? k_chain(kc, g, j) : k_nat(kc, g, j);
+    const int r = TRANSPOSED ? k : m;
+    const int c = TRANSPOSED ? m : k;
+    dst[e] = (r < w_rows && c < w_cols) ? w[(size_t)r * w_cols + c] : (uint16_t)0;
+  }
+}
+
+__device__ __forceinline__ Frag lds_frag(const uint16_t* frags, int frag_index, int lane) {
+  Frag f;
+  f.u = *reinterpret_cast<const uint4*>(frags + ((size_t)frag_index * 64 + lane) * 8);
+  return f;
+}
+
+// ---- global <-> row-per-lane fragments ---------------------------------------------------
+// B fragment of K-chunk kc for 16 rows starting at row0: lane (n, g) gets features
+// 32*kc + 8*g .. +7 of row row0 + n; zero beyond `rows` / `width`.
+__device__ __forceinline__ Frag load_rows_frag(const uint16_t* base, int64_t stride, int64_t row0, int64_t rows,
+                                               int width, int kc, int lane, bool vec_ok) {
+  Frag f;
+  f.u = make_uint4(0u, 0u, 0u, 0u);
+  const int64_t r = row0 + (lane & 15);
+  const int c0 = 32 * kc + 8 * (lane >> 4);
+  if (r < rows && c0 < width) {
+    const uint16_t* p = base + r * stride + c0;
+    if (vec_ok && c0 + 8 <= width) {
+      f.u = *reinterpret_cast<const uint4*>(p);
+    } else {
+      uint16_t tmp[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) tmp[j] = (c0 + j < width) ? p[j] : (uint16_t)0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) f.w[j] = (uint32_t)tmp[2 * j] | ((uint32_t)tmp[2 * j + 1] << 16);
+    }
+  }
+  return f;
+}
+
+// Store accumulator tile mt (lane (n,g): features 16*mt + 4*g + r) of 16 rows as 16-bit values.
+template <typename T>
+__device__ __forceinline__ void store_rows_tile(uint16_t* base, int64_t stride, int64_t row0, int64_t rows, int width,
+                                                int mt, int lane, f32x4_t v, bool vec_ok) {
+  const int64_t r = row0 + (lane & 15);
+  const int c0 = 16 * mt + 4 * (lane >> 4);
+  if (r >= rows || c0 >= width) return;
+  uint16_t* p = base + r * stride + c0;
+  if (vec_ok && c0 + 4 <= width) {
+    uint2 o;
+    o.x = pack2<T>(v[0], v[1]);
+    o.y = pack2<T>(v[2], v[3]);
+    *reinterpret_cast<uint2*>(p) = o;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (c0 + i < width) p[i] = T::from_f32(v[i]);
+  }
+}
+
+inline bool vec_load_ok(const void* p, int64_t stride_elems, int width) {
+  return ((uintptr_t)p % 16 == 0) && (stride_elems % 8 == 0) && (width % 8 == 0);
+}
+inline bool vec_store_ok(const void* p, int64_t stride_elems, int width) {
+  return ((uintptr_t)p % 8 == 0) && (stride_elems % 4 == 0) && (width % 4 == 0);
+}
+
+}  // namespace nf

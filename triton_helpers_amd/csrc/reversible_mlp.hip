@@ -1,3 +1,569 @@
-#include "nf_common.h"
-extern "C" int nf_revmlp_fwd(const void*, int64_t, void*, int64_t, const void*, const void*, const void*, const void*, int64_t, int, int, int, int, void*) { return nf::fail(NF_EUNSUPPORTED, "nf_revmlp_fwd not built yet"); }
-extern "C" int nf_revmlp_bwd(const void*, int64_t, const void*, int64_t, void*, int64_t, void*, int64_t, const void*, const void*, const void*, const void*, float*, float*, float*, float*, int64_t, int, int, int, int, void*) { return nf::fail(NF_EUNSUPPORTED, "nf_revmlp_bwd not built yet"); }
+// Reversible (additive-coupling) fused MLP for gfx950, 16-bit storage, MFMA 16x16x32.
+//
+//   block k:  y1 = x1 + F_k(x2),  y2 = x2 + G_k(y1),   F/G(u) = act(u W1^T + b1) W2^T + b2
+//
+// Forward: one launch runs up to FWD_GROUP coupling blocks with all their weights resident
+// in LDS; the two halves of the residual stream stay in float32 registers between blocks.
+// Backward: one launch per coupling block, last block first.  It takes the block's OUTPUT
+// (y, dy), rebuilds the block's input in-kernel (x2 = y2 - G(y1), x1 = y1 - F(x2)) while it
+// back-propagates, and writes (x, dx), which the next launch reads in place.  No activation
+// of the forward pass is ever stored.  The four weight gradients of a block accumulate in
+// float32 registers over the wave's whole row loop.
+//
+// There is no counterpart in the reference; the layer math is that of its fused MLP
+// (triton_helpers/layers/fully_fused_mlp/kernel.py:17-74).
+#include "mlp_tile.h"
+
+namespace nf {
+
+constexpr int RFRAG = 64 * 8;
+constexpr int RPITCH = 40;     // 16-bit elements per feature row of a transposed 32-row panel
+constexpr int FWD_GROUP = 4;   // coupling blocks per forward launch (LDS: 32 KiB of weights per block at H = 64)
+
+struct RevArgs {
+  const uint16_t* in;   // fwd: x ; bwd: y of this block
+  int64_t in_stride;
+  uint16_t* out;        // fwd: y ; bwd: reconstructed x
+  int64_t out_stride;
+  const uint16_t* dy;
+  int64_t dy_stride;
+  uint16_t* dx;
+  int64_t dx_stride;
+  const uint16_t *w1, *b1, *w2, *b2;  // already offset to the first block of this launch
+  float *dw1, *db1, *dw2, *db2;       // already offset to this block (backward)
+  int64_t rows;
+  int half, nblocks, act;
+  int vec_in, vec_out, vec_dy, vec_dx;
+};
+
+// accumulator-layout load: lane (n,g) gets features 16*mt + 4*g + r of row row0 + n as two packed dwords
+__device__ __forceinline__ uint2 load_tile_packed(const uint16_t* base, int64_t stride, int64_t row0, int64_t rows, int col0,
+                                                  int width, int mt, int lane, bool vec_ok) {
+  uint2 v = make_uint2(0u, 0u);
+  const int64_t r = row0 + (lane & 15);
+  const int c = 16 * mt + 4 * (lane >> 4);
+  if (r < rows && c < width) {
+    const uint16_t* p = base + r * stride + col0 + c;
+    if (vec_ok && c + 4 <= width) {
+      v = *reinterpret_cast<const uint2*>(p);
+    } else {
+      uint16_t t[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) t[i] = (c + i < width) ? p[i] : (uint16_t)0;
+      v.x = (uint32_t)t[0] | ((uint32_t)t[1] << 16);
+      v.y = (uint32_t)t[2] | ((uint32_t)t[3] << 16);
+    }
+  }
+  return v;
+}
+__device__ __forceinline__ void store_tile_packed(uint16_t* base, int64_t stride, int64_t row0, int64_t rows, int col0,
+                                                  int width, int mt, int lane, uint2 v, bool vec_ok) {
+  const int64_t r = row0 + (lane & 15);
+  const int c = 16 * mt + 4 * (lane >> 4);
+  if (r >= rows || c >= width) return;
+  uint16_t* p = base + r * stride + col0 + c;
+  if (vec_ok && c + 4 <= width) {
+    *reinterpret_cast<uint2*>(p) = v;
+  } else {
+    const uint16_t t[4] = {(uint16_t)(v.x & 0xffffu), (uint16_t)(v.x >> 16), (uint16_t)(v.y & 0xffffu), (uint16_t)(v.y >> 16)};
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (c + i < width) p[i] = t[i];
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ f32x4_t unpack4(uint2 v) {
+  f32x4_t o = {unpack_lo<T>(v.x), unpack_hi<T>(v.x), unpack_lo<T>(v.y), unpack_hi<T>(v.y)};
+  return o;
+}
+template <typename T>
+__device__ __forceinline__ uint2 pack4(f32x4_t v) {
+  return make_uint2(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]));
+}
+
+// packed accumulator-layout tiles P[nt][mt] -> B fragments (chain order) F[nt][kc]
+template <int MT>
+__device__ __forceinline__ void tiles_to_frags(const uint2 (&p)[2][4], Frag (&f)[2][2]) {
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      f[nt][mt >> 1].w[2 * (mt & 1)] = p[nt][mt].x;
+      f[nt][mt >> 1].w[2 * (mt & 1) + 1] = p[nt][mt].y;
+    }
+}
+
+template <typename T, int MT, int KC>
+__device__ __forceinline__ void rev_layer(f32x4_t (&acc)[2][4], const Frag (&in)[2][2], const uint16_t* frags, const float* bias,
+                                          int lane) {
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    f32x4_t b4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (bias != nullptr) b4 = *reinterpret_cast<const f32x4_t*>(bias + 16 * mt + 4 * (lane >> 4));
+    acc[0][mt] = b4;
+    acc[1][mt] = b4;
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc) {
+      const Frag a = lds_frag(frags, mt * KC + kc, lane);
+      acc[0][mt] = mfma16<T>(a, in[0][kc], acc[0][mt]);
+      acc[1][mt] = mfma16<T>(a, in[1][kc], acc[1][mt]);
+    }
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ void stage_bias_row(float* dst, const uint16_t* b, int n_valid, int n_pad, int tid, int nthreads) {
+  for (int i = tid; i < n_pad; i += nthreads) dst[i] = (b != nullptr && i < n_valid) ? T::to_f32(b[i]) : 0.0f;
+}
+
+// ---------------------------------------------------------------------------------------
+// Forward: up to FWD_GROUP blocks per launch
+// ---------------------------------------------------------------------------------------
+template <typename T, int HP>
+__global__ __launch_bounds__(256) void rev_fwd_k(RevArgs a) {
+  constexpr int MT = HP / 16, KC = HP / 32, LAYER = MT * KC * RFRAG;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, nthreads = blockDim.x, lane = tid & 63, wave = tid >> 6;
+  uint16_t* frags = reinterpret_cast<uint16_t*>(smem);  // [nblocks][F.w1, F.w2, G.w1, G.w2][LAYER]
+  float* bias = reinterpret_cast<float*>(frags + (size_t)a.nblocks * 4 * LAYER);  // [nblocks][4][HP]
+  const int H = a.half;
+  for (int k = 0; k < a.nblocks; ++k)
+    for (int s = 0; s < 2; ++s) {
+      const size_t sub = (size_t)(2 * k + s);
+      stage_weight_frags<true, false>(frags + ((size_t)k * 4 + 2 * s) * LAYER, a.w1 + sub * H * H, H, H, MT, KC, tid, nthreads);
+      stage_weight_frags<true, false>(frags + ((size_t)k * 4 + 2 * s + 1) * LAYER, a.w2 + sub * H * H, H, H, MT, KC, tid, nthreads);
+      stage_bias_row<T>(bias + ((size_t)k * 4 + 2 * s) * HP, a.b1 ? a.b1 + sub * H : nullptr, H, HP, tid, nthreads);
+      stage_bias_row<T>(bias + ((size_t)k * 4 + 2 * s + 1) * HP, a.b2 ? a.b2 + sub * H : nullptr, H, HP, tid, nthreads);
+    }
+  __syncthreads();
+
+  const int64_t n_chunks = (a.rows + 31) / 32;
+  for (int64_t chunk = (int64_t)blockIdx.x * 4 + wave; chunk < n_chunks; chunk += (int64_t)gridDim.x * 4) {
+    const int64_t row0 = chunk * 32;
+    f32x4_t s1[2][4], s2[2][4];  // the two halves of the residual stream, float32
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        s1[nt][mt] = unpack4<T>(load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in));
+        s2[nt][mt] = unpack4<T>(load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_in));
+      }
+    for (int k = 0; k < a.nblocks; ++k) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        // s == 0: s1 += F(s2) ; s == 1: s2 += G(s1)
+        f32x4_t(&src)[2][4] = s == 0 ? s2 : s1;
+        f32x4_t(&dst)[2][4] = s == 0 ? s1 : s2;
+        const uint16_t* fw1 = frags + ((size_t)k * 4 + 2 * s) * LAYER;
+        const float* bb1 = bias + ((size_t)k * 4 + 2 * s) * HP;
+        uint2 p[2][4];
+        Frag u[2][2], t[2][2];
+        f32x4_t acc[2][4];
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) p[nt][mt] = pack4<T>(src[nt][mt]);
+        tiles_to_frags<MT>(p, u);
+        rev_layer<T, MT, KC>(acc, u, fw1, bb1, lane);
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            f32x4_t z = acc[nt][mt];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) z[r] = act_fwd(z[r], a.act);
+            p[nt][mt] = pack4<T>(z);
+          }
+        tiles_to_frags<MT>(p, t);
+        rev_layer<T, MT, KC>(acc, t, fw1 + LAYER, bb1 + HP, lane);
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) dst[nt][mt] += acc[nt][mt];
+      }
+    }
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        store_tile_packed(a.out, a.out_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, pack4<T>(s1[nt][mt]), a.vec_out);
+        store_tile_packed(a.out, a.out_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, pack4<T>(s2[nt][mt]), a.vec_out);
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Backward of one coupling block
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ void park_packed_T(uint16_t* panel, int mt, int nt, int lane, uint2 v) {
+  const int n = (lane & 15) + 16 * nt;
+  const int f = 16 * mt + 4 * (lane >> 4);
+  panel[(f + 0) * RPITCH + n] = (uint16_t)(v.x & 0xffffu);
+  panel[(f + 1) * RPITCH + n] = (uint16_t)(v.x >> 16);
+  panel[(f + 2) * RPITCH + n] = (uint16_t)(v.y & 0xffffu);
+  panel[(f + 3) * RPITCH + n] = (uint16_t)(v.y >> 16);
+}
+__device__ __forceinline__ Frag rpanel_frag(const uint16_t* panel, int t, int lane) {
+  Frag f;
+  f.u = *reinterpret_cast<const uint4*>(panel + (16 * t + (lane & 15)) * RPITCH + 8 * (lane >> 4));
+  return f;
+}
+
+// Sum over the 32 rows of feature `lane` of a transposed panel (lanes >= feats return 0).
+template <typename T>
+__device__ __forceinline__ float panel_rowsum(const uint16_t* panel, int feats, int lane) {
+  float s = 0.0f;
+  if (lane < feats) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint4 v = *reinterpret_cast<const uint4*>(panel + lane * RPITCH + 8 * q);
+      s += unpack_lo<T>(v.x) + unpack_hi<T>(v.x) + unpack_lo<T>(v.y) + unpack_hi<T>(v.y) + unpack_lo<T>(v.z) +
+           unpack_hi<T>(v.z) + unpack_lo<T>(v.w) + unpack_hi<T>(v.w);
+    }
+  }
+  return s;
+}
+
+// Back-propagate through one sub-MLP  out = in_other + S(u):
+//   given u (packed tiles), the incoming gradient d (packed tiles) w.r.t. S's output, computes
+//   s_out = S(u) (float32, returned in `sout`), accumulates dW1, dW2 (and db), and returns du = W1^T dz.
+template <typename T, int MT, int KC>
+__device__ __forceinline__ void sub_backward(const uint2 (&u)[2][4], const uint2 (&d)[2][4], f32x4_t (&sout)[2][4],
+                                             f32x4_t (&du)[2][4], f32x4_t (&dw1)[4][4], f32x4_t (&dw2)[4][4],
+                                             float& db1, float& db2, bool want_db, const uint16_t* fw1,
+                                             const uint16_t* fw2, const uint16_t* tw1, const uint16_t* tw2, const float* b1,
+                                             const float* b2, uint16_t* p_in, uint16_t* p_t, uint16_t* p_d, uint16_t* p_dz,
+                                             int act, int lane) {
+  Frag uf[2][2], tf[2][2], df[2][2], dzf[2][2];
+  uint2 tp[2][4], gp[2][4];
+  f32x4_t acc[2][4];
+  tiles_to_frags<MT>(u, uf);
+  tiles_to_frags<MT>(d, df);
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      park_packed_T(p_in, mt, nt, lane, u[nt][mt]);
+      park_packed_T(p_d, mt, nt, lane, d[nt][mt]);
+    }
+  // recompute hidden activation t = act(W1 u + b1) and act'(z)
+  rev_layer<T, MT, KC>(acc, uf, fw1, b1, lane);
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      f32x4_t h, g;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        h[r] = act_fwd(acc[nt][mt][r], act);
+        g[r] = act_grad(acc[nt][mt][r], act);
+      }
+      tp[nt][mt] = pack4<T>(h);
+      gp[nt][mt] = pack4<T>(g);
+      park_packed_T(p_t, mt, nt, lane, tp[nt][mt]);
+    }
+  tiles_to_frags<MT>(tp, tf);
+  // S(u) = W2 t + b2
+  rev_layer<T, MT, KC>(sout, tf, fw2, b2, lane);
+  // dW2 += d^T t
+  {
+    Frag tb[MT];
+#pragma unroll
+    for (int j = 0; j < MT; ++j) tb[j] = rpanel_frag(p_t, j, lane);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const Frag da = rpanel_frag(p_d, i, lane);
+#pragma unroll
+      for (int j = 0; j < MT; ++j) dw2[i][j] = mfma16<T>(da, tb[j], dw2[i][j]);
+    }
+  }
+  // dt = W2^T d ; dz = dt * act'(z)
+  rev_layer<T, MT, KC>(acc, df, tw2, nullptr, lane);
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const f32x4_t g = unpack4<T>(gp[nt][mt]);
+      f32x4_t dz;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) dz[r] = acc[nt][mt][r] * g[r];
+      tp[nt][mt] = pack4<T>(dz);
+      park_packed_T(p_dz, mt, nt, lane, tp[nt][mt]);
+    }
+  tiles_to_frags<MT>(tp, dzf);
+  if (want_db) {
+    // lane f sums the 32 parked rows of feature f: db1 from dz, db2 from the incoming gradient
+    db1 += panel_rowsum<T>(p_dz, 16 * MT, lane);
+    db2 += panel_rowsum<T>(p_d, 16 * MT, lane);
+  }
+  // dW1 += dz^T u
+  {
+    Frag ub[MT];
+#pragma unroll
+    for (int j = 0; j < MT; ++j) ub[j] = rpanel_frag(p_in, j, lane);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const Frag da = rpanel_frag(p_dz, i, lane);
+#pragma unroll
+      for (int j = 0; j < MT; ++j) dw1[i][j] = mfma16<T>(da, ub[j], dw1[i][j]);
+    }
+  }
+  // du = W1^T dz
+  rev_layer<T, MT, KC>(du, dzf, tw1, nullptr, lane);
+}
+
+__device__ __forceinline__ void flush_tile(float* dw, int dim, int mt, int nt, int lane, f32x4_t v) {
+  const int c = 16 * nt + (lane & 15);
+  const int r0 = 16 * mt + 4 * (lane >> 4);
+  if (c >= dim) return;
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+    if (r0 + r < dim) unsafeAtomicAdd(dw + (size_t)(r0 + r) * dim + c, v[r]);
+}
+
+template <typename T, int HP>
+__global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
+  constexpr int MT = HP / 16, KC = HP / 32, LAYER = MT * KC * RFRAG;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, nthreads = blockDim.x, lane = tid & 63, wave = tid >> 6;
+  const int H = a.half;
+  // weights: forward-form [F.w1, F.w2, G.w1, G.w2], transposed-form the same order
+  uint16_t* fw = reinterpret_cast<uint16_t*>(smem);
+  uint16_t* tw = fw + 4 * LAYER;
+  float* bias = reinterpret_cast<float*>(tw + 4 * LAYER);  // [4][HP]
+  uint16_t* panels = reinterpret_cast<uint16_t*>(bias + 4 * HP) + (size_t)wave * 4 * HP * RPITCH;
+  uint16_t *p_in = panels, *p_t = panels + HP * RPITCH, *p_d = panels + 2 * HP * RPITCH, *p_dz = panels + 3 * HP * RPITCH;
+  for (int s = 0; s < 2; ++s) {
+    stage_weight_frags<true, false>(fw + (2 * s) * LAYER, a.w1 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
+    stage_weight_frags<true, false>(fw + (2 * s + 1) * LAYER, a.w2 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
+    stage_weight_frags<true, true>(tw + (2 * s) * LAYER, a.w1 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
+    stage_weight_frags<true, true>(tw + (2 * s + 1) * LAYER, a.w2 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
+    stage_bias_row<T>(bias + (2 * s) * HP, a.b1 ? a.b1 + (size_t)s * H : nullptr, H, HP, tid, nthreads);
+    stage_bias_row<T>(bias + (2 * s + 1) * HP, a.b2 ? a.b2 + (size_t)s * H : nullptr, H, HP, tid, nthreads);
+  }
+  __syncthreads();
+
+  f32x4_t dwF1[4][4], dwF2[4][4], dwG1[4][4], dwG2[4][4];
+  float dbF1 = 0.0f, dbF2 = 0.0f, dbG1 = 0.0f, dbG2 = 0.0f;  // lane f: bias gradient of feature f
+  const f32x4_t zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dwF1[i][j] = dwF2[i][j] = dwG1[i][j] = dwG2[i][j] = zero4;
+  const bool want_db = a.db1 != nullptr || a.db2 != nullptr;
+
+  const int64_t n_chunks = (a.rows + 31) / 32;
+  for (int64_t chunk = (int64_t)blockIdx.x * 4 + wave; chunk < n_chunks; chunk += (int64_t)gridDim.x * 4) {
+    const int64_t row0 = chunk * 32;
+    uint2 y1[2][4], y2[2][4], d1[2][4], d2[2][4];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        y1[nt][mt] = load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in);
+        y2[nt][mt] = load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_in);
+        d1[nt][mt] = load_tile_packed(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_dy);
+        d2[nt][mt] = load_tile_packed(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_dy);
+      }
+    f32x4_t sout[2][4], du[2][4];
+    // ---- G:  y2 = x2 + G(y1)  =>  x2 = y2 - G(y1),  dy1 += (dG/dy1)^T dy2
+    sub_backward<T, MT, KC>(y1, d2, sout, du, dwG1, dwG2, dbG1, dbG2, want_db, fw + 2 * LAYER, fw + 3 * LAYER,
+                            tw + 2 * LAYER, tw + 3 * LAYER, bias + 2 * HP, bias + 3 * HP, p_in, p_t, p_d, p_dz, a.act, lane);
+    uint2 x2[2][4];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        x2[nt][mt] = pack4<T>(unpack4<T>(y2[nt][mt]) - sout[nt][mt]);
+        d1[nt][mt] = pack4<T>(unpack4<T>(d1[nt][mt]) + du[nt][mt]);
+      }
+    // ---- F:  y1 = x1 + F(x2)  =>  x1 = y1 - F(x2),  dx2 = dy2 + (dF/dx2)^T dy1
+    sub_backward<T, MT, KC>(x2, d1, sout, du, dwF1, dwF2, dbF1, dbF2, want_db, fw, fw + LAYER, tw, tw + LAYER, bias,
+                            bias + HP, p_in, p_t, p_d, p_dz, a.act, lane);
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const uint2 x1 = pack4<T>(unpack4<T>(y1[nt][mt]) - sout[nt][mt]);
+        const uint2 dx2 = pack4<T>(unpack4<T>(d2[nt][mt]) + du[nt][mt]);
+        store_tile_packed(a.out, a.out_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, x1, a.vec_out);
+        store_tile_packed(a.out, a.out_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, x2[nt][mt], a.vec_out);
+        store_tile_packed(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, d1[nt][mt], a.vec_dx);
+        store_tile_packed(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, dx2, a.vec_dx);
+      }
+  }
+
+  // ---- weight gradients: every wave adds its float32 accumulators (64-byte coalesced atomics) ----
+  // layer order in dw1 / dw2: sub-MLP F is row block 0, G is row block 1 of this coupling block
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      flush_tile(a.dw1, H, i, j, lane, dwF1[i][j]);
+      flush_tile(a.dw2, H, i, j, lane, dwF2[i][j]);
+      flush_tile(a.dw1 + (size_t)H * H, H, i, j, lane, dwG1[i][j]);
+      flush_tile(a.dw2 + (size_t)H * H, H, i, j, lane, dwG2[i][j]);
+    }
+  if (want_db && lane < H) {
+    if (a.db1 != nullptr) {
+      unsafeAtomicAdd(a.db1 + lane, dbF1);
+      unsafeAtomicAdd(a.db1 + H + lane, dbG1);
+    }
+    if (a.db2 != nullptr) {
+      unsafeAtomicAdd(a.db2 + lane, dbF2);
+      unsafeAtomicAdd(a.db2 + H + lane, dbG2);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------
+static int rev_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) cus = p.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+static int rev_validate(int64_t rows, int half, int blocks, int act, int dtype) {
+  NF_REQUIRE(rows >= 0, NF_EINVAL, "rows negative");
+  NF_REQUIRE(half >= 1 && half <= 64, NF_EINVAL, "half=%d outside 1..64", half);
+  NF_REQUIRE(blocks >= 1, NF_EINVAL, "blocks=%d must be >= 1", blocks);
+  NF_REQUIRE(act >= NF_ACT_NONE && act <= NF_ACT_GELU, NF_EINVAL, "unknown activation %d", act);
+  NF_REQUIRE(dtype == NF_F16 || dtype == NF_BF16, NF_EUNSUPPORTED,
+             "dtype code %d: the reversible MLP kernels take float16 or bfloat16 storage", dtype);
+  return 0;
+}
+
+static bool vec8_ok(const void* p, int64_t stride, int half) {
+  return ((uintptr_t)p % 8 == 0) && (stride % 4 == 0) && (half % 4 == 0);
+}
+
+template <typename T, int HP>
+static int launch_rev_fwd(RevArgs a, hipStream_t s) {
+  constexpr int LAYER = (HP / 16) * (HP / 32) * RFRAG;
+  const size_t lds = (size_t)a.nblocks * 4 * LAYER * 2 + (size_t)a.nblocks * 4 * HP * 4;
+  const int64_t chunks = (a.rows + 31) / 32;
+  int64_t blocks = (chunks + 3) / 4;
+  const int64_t cap = (int64_t)rev_cus() * (lds > 80 * 1024 ? 1 : 2);
+  if (blocks > cap) blocks = cap;
+  auto kern = rev_fwd_k<T, HP>;
+  if (lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), lds, s, a);
+  return check_launch("rev_fwd");
+}
+
+template <typename T, int HP>
+static int launch_rev_bwd(RevArgs a, hipStream_t s) {
+  constexpr int LAYER = (HP / 16) * (HP / 32) * RFRAG;
+  const size_t lds = (size_t)8 * LAYER * 2 + (size_t)4 * HP * 4 + (size_t)4 * 4 * HP * RPITCH * 2;
+  const int64_t chunks = (a.rows + 31) / 32;
+  int64_t blocks = (chunks + 3) / 4;
+  const int64_t cap = (int64_t)rev_cus() * (lds > 80 * 1024 ? 1 : 2);
+  if (blocks > cap) blocks = cap;
+  auto kern = rev_bwd_block_k<T, HP>;
+  if (lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), lds, s, a);
+  return check_launch("rev_bwd_block");
+}
+
+}  // namespace nf
+
+using namespace nf;
+
+extern "C" int nf_revmlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_stride, const void* w1, const void* b1,
+                             const void* w2, const void* b2, int64_t rows, int half, int blocks, int act, int dtype,
+                             void* stream) {
+  if (int rc = rev_validate(rows, half, blocks, act, dtype)) return rc;
+  if (rows == 0) return 0;
+  NF_REQUIRE(x && y && w1 && w2, NF_EINVAL, "NULL pointer argument");
+  NF_REQUIRE(x_stride >= 2 * half && y_stride >= 2 * half, NF_EINVAL, "row stride smaller than 2*half");
+  hipStream_t s = (hipStream_t)stream;
+  const int es = 2;
+  for (int k0 = 0; k0 < blocks; k0 += FWD_GROUP) {
+    RevArgs a = {};
+    // the first group reads x; later groups continue in place on y (a wave reads its rows before it writes them)
+    a.in = (const uint16_t*)(k0 == 0 ? x : y);
+    a.in_stride = k0 == 0 ? x_stride : y_stride;
+    a.out = (uint16_t*)y;
+    a.out_stride = y_stride;
+    a.w1 = (const uint16_t*)w1 + (size_t)2 * k0 * half * half;
+    a.w2 = (const uint16_t*)w2 + (size_t)2 * k0 * half * half;
+    a.b1 = b1 ? (const uint16_t*)b1 + (size_t)2 * k0 * half : nullptr;
+    a.b2 = b2 ? (const uint16_t*)b2 + (size_t)2 * k0 * half : nullptr;
+    a.rows = rows;
+    a.half = half;
+    a.nblocks = blocks - k0 < FWD_GROUP ? blocks - k0 : FWD_GROUP;
+    a.act = act;
+    a.vec_in = vec8_ok(a.in, a.in_stride, half);
+    a.vec_out = vec8_ok(a.out, a.out_stride, half);
+    (void)es;
+    int rc;
+    if (half <= 32)
+      rc = dtype == NF_BF16 ? launch_rev_fwd<BF16, 32>(a, s) : launch_rev_fwd<F16, 32>(a, s);
+    else
+      rc = dtype == NF_BF16 ? launch_rev_fwd<BF16, 64>(a, s) : launch_rev_fwd<F16, 64>(a, s);
+    if (rc) return rc;
+  }
+  return 0;
+}
+
+extern "C" int nf_revmlp_bwd(const void* y, int64_t y_stride, const void* dy, int64_t dy_stride, void* dx, int64_t dx_stride,
+                             void* x_rec, int64_t x_rec_stride, const void* w1, const void* b1, const void* w2,
+                             const void* b2, float* dw1, float* db1, float* dw2, float* db2, int64_t rows, int half,
+                             int blocks, int act, int dtype, void* stream) {
+  if (int rc = rev_validate(rows, half, blocks, act, dtype)) return rc;
+  if (rows == 0) return 0;
+  NF_REQUIRE(y && dy && dx && x_rec && w1 && w2 && dw1 && dw2, NF_EINVAL,
+             "NULL pointer argument (x_rec is required: it carries the reconstructed input between blocks)");
+  NF_REQUIRE(y_stride >= 2 * half && dy_stride >= 2 * half && dx_stride >= 2 * half && x_rec_stride >= 2 * half, NF_EINVAL,
+             "row stride smaller than 2*half");
+  hipStream_t s = (hipStream_t)stream;
+  for (int k = blocks - 1; k >= 0; --k) {
+    RevArgs a = {};
+    const bool first = k == blocks - 1;
+    a.in = (const uint16_t*)(first ? y : x_rec);
+    a.in_stride = first ? y_stride : x_rec_stride;
+    a.out = (uint16_t*)x_rec;
+    a.out_stride = x_rec_stride;
+    a.dy = (const uint16_t*)(first ? dy : dx);
+    a.dy_stride = first ? dy_stride : dx_stride;
+    a.dx = (uint16_t*)dx;
+    a.dx_stride = dx_stride;
+    a.w1 = (const uint16_t*)w1 + (size_t)2 * k * half * half;
+    a.w2 = (const uint16_t*)w2 + (size_t)2 * k * half * half;
+    a.b1 = b1 ? (const uint16_t*)b1 + (size_t)2 * k * half : nullptr;
+    a.b2 = b2 ? (const uint16_t*)b2 + (size_t)2 * k * half : nullptr;
+    a.dw1 = dw1 + (size_t)2 * k * half * half;
+    a.dw2 = dw2 + (size_t)2 * k * half * half;
+    a.db1 = db1 ? db1 + (size_t)2 * k * half : nullptr;
+    a.db2 = db2 ? db2 + (size_t)2 * k * half : nullptr;
+    a.rows = rows;
+    a.half = half;
+    a.nblocks = 1;
+    a.act = act;
+    a.vec_in = vec8_ok(a.in, a.in_stride, half);
+    a.vec_out = vec8_ok(a.out, a.out_stride, half);
+    a.vec_dy = vec8_ok(a.dy, a.dy_stride, half);
+    a.vec_dx = vec8_ok(a.dx, a.dx_stride, half);
+    int rc;
+    if (half <= 32)
+      rc = dtype == NF_BF16 ? launch_rev_bwd<BF16, 32>(a, s) : launch_rev_bwd<F16, 32>(a, s);
+    else
+      rc = dtype == NF_BF16 ? launch_rev_bwd<BF16, 64>(a, s) : launch_rev_bwd<F16, 64>(a, s);
+    if (rc) return rc;
+  }
+  return 0;
+}

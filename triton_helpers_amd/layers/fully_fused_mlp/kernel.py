@@ -1,0 +1,218 @@
+"""Fully fused small MLP on MI355X.
+
+Drop-in for ``triton_helpers/layers/fully_fused_mlp/kernel.py`` of the reference:
+same ``fully_fused_mlp(...)`` functional and ``_fully_fused_mlp`` autograd Function
+(argument order, 9-tuple returned by ``backward``), same assertions and the same
+weight layout (``w_hid`` = hidden layers stacked along rows, ``b_hid [depth-1, H]``).
+The Triton launches are replaced by ``nf_mlp_fwd`` / ``nf_mlp_bwd`` of ``libnf_cdna4.so``.
+
+Supersets / differences:
+  * any bias may be ``None`` (the reference always has biases);
+  * weight gradients are accumulated in float32 inside the kernel and rounded once
+    (the reference sums per-program partials in the storage dtype, kernel.py:599-633);
+  * ``fp16_acc`` is accepted and ignored: accumulation is always float32 (MFMA);
+  * storage dtypes are float16 and bfloat16 (what autocast produces); float32 tensors
+    raise ``NotImplementedError`` -- cast them, or run the module under autocast.
+"""
+from __future__ import annotations
+
+from typing import Final, Optional
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor
+from torch.autograd import Function
+
+from ... import _lib
+
+# Above this size the weights do not stay on chip (reference kernel.py:13-14)
+FULLY_FUSED_MAX_DIM: Final = 64
+
+_ACTIVATIONS = ("relu", "relu2", "silu", "none")
+
+
+# ---------------------------------------------------------------------------
+# Per-layer math with the reference's names (kernel.py:17-74).  In the reference these
+# are Triton device functions; here they are plain torch functions for users' tests.
+# No operator of this package calls them.
+# ---------------------------------------------------------------------------
+def _activate(z: Tensor, activation: str) -> Tensor:
+    if activation == "relu":
+        return torch.where(z < 0, torch.zeros_like(z), z)
+    if activation == "silu":
+        return z * torch.sigmoid(z)
+    if activation == "relu2":
+        return torch.clamp_min(z, 0) * z
+    if activation == "none":
+        return z
+    raise ValueError(f"Invalid activation function: {activation}")
+
+
+def feedforward(x: Tensor, w: Tensor, b: Optional[Tensor], HAS_BIAS: bool = True, ACTIVATION: str = "relu",
+                DTYPE: torch.dtype = torch.float32) -> Tensor:
+    z = x.to(DTYPE) @ w.to(DTYPE).t()
+    if HAS_BIAS and b is not None:
+        z = z + b.to(DTYPE)
+    return _activate(z, ACTIVATION).to(x.dtype)
+
+
+def feedforward_bwd_dz(z: Tensor, do: Tensor, ACTIVATION: str) -> Tensor:
+    zf, g = z.float(), do.float()
+    if ACTIVATION == "relu":
+        dz = torch.where(zf > 0, g, torch.zeros_like(g))
+    elif ACTIVATION == "silu":
+        s = torch.sigmoid(zf)
+        dz = g * s * (zf * (1 - s) + 1)
+    elif ACTIVATION == "relu2":
+        dz = torch.where(zf > 0, g * (2 * zf), torch.zeros_like(g))
+    elif ACTIVATION == "none":
+        dz = g
+    else:
+        raise ValueError(f"Invalid activation function: {ACTIVATION}")
+    return dz.to(do.dtype)
+
+
+def feedforward_bwd_dw(x: Tensor, dz: Tensor, DTYPE: torch.dtype = torch.float32) -> Tensor:
+    return (dz.to(DTYPE).t() @ x.to(DTYPE)).to(dz.dtype)
+
+
+def feedforward_bwd_dx(w: Tensor, dz: Tensor, DTYPE: torch.dtype = torch.float32) -> Tensor:
+    return (dz.to(DTYPE) @ w.to(DTYPE)).to(dz.dtype)
+
+
+# ---------------------------------------------------------------------------
+def _check_storage(x: Tensor, *others: Optional[Tensor]) -> None:
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise NotImplementedError(
+            f"fully_fused_mlp runs on float16 / bfloat16 storage, got {x.dtype}; cast the tensors or use autocast"
+        )
+    for t in others:
+        assert t is None or t.dtype == x.dtype, f"All tensors must share one dtype, got {x.dtype} and {t.dtype}"
+        assert t is None or t.device == x.device, "All tensors must be on the same device"
+    assert x.device.type == "cuda", "All tensors must be on a GPU device"
+
+
+def _rows2d(t: Tensor, width: int) -> Tensor:
+    t2 = t.reshape(-1, width)
+    if t2.stride(1) != 1:
+        t2 = t2.contiguous()
+    return t2
+
+
+def _c(t: Optional[Tensor]) -> Optional[Tensor]:
+    return None if t is None else (t if t.is_contiguous() else t.contiguous())
+
+
+class _fully_fused_mlp(Function):
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.float16)
+    @torch.no_grad()
+    def forward(
+        ctx,
+        x: Tensor,
+        w_in: Tensor, b_in: Optional[Tensor],
+        w_out: Tensor, b_out: Optional[Tensor],
+        w_hid: Optional[Tensor], b_hid: Optional[Tensor],
+        activation: str = "relu",
+        fp16_acc: bool = False,
+    ) -> Tensor:
+        B, L, D = x.shape
+        D_hidden, D_in = w_in.shape
+        D_out, _ = w_out.shape
+        assert D_in == D, "Input dimension mismatch"
+        assert D_hidden == w_out.shape[-1], "Hidden dimension mismatch"
+
+        assert D_in <= FULLY_FUSED_MAX_DIM, f"Input dimension {D_in} too large for full fusion"
+        assert D_hidden <= FULLY_FUSED_MAX_DIM, f"Hidden dimension {D_hidden} too large for full fusion"
+        assert D_out <= FULLY_FUSED_MAX_DIM, f"Output dimension {D_out} too large for full fusion"
+
+        assert D_hidden & (D_hidden - 1) == 0, "Hidden dimension must be a power of 2"
+        assert D_hidden >= 16, "Hidden dimension must be at least 16"
+
+        if w_hid is not None and w_hid.numel() > 0:
+            n_hid = w_hid.shape[0] // D_hidden
+            assert w_hid.shape == (n_hid * D_hidden, D_hidden), "Hidden weight shape mismatch"
+            assert b_hid is None or b_hid.shape == (n_hid, D_hidden), "Hidden bias shape mismatch"
+            depth = n_hid + 1
+        else:
+            depth = 1
+            w_hid = b_hid = None
+        assert b_in is None or b_in.shape == (D_hidden,), "Input bias shape mismatch"
+        assert b_out is None or b_out.shape == (D_out,), "Output bias shape mismatch"
+
+        assert activation in _ACTIVATIONS, f"Invalid activation function: {activation}"
+        _check_storage(x, w_in, b_in, w_out, b_out, w_hid, b_hid)
+
+        w_in, b_in, w_out, b_out, w_hid, b_hid = (_c(t) for t in (w_in, b_in, w_out, b_out, w_hid, b_hid))
+        x2 = _rows2d(x, D_in)
+        o = x.new_empty((B, L, D_out))
+        o2 = o.view(-1, D_out)
+        lib = _lib.load()
+        rc = lib.nf_mlp_fwd(
+            x2.data_ptr(), x2.stride(0), o2.data_ptr(), o2.stride(0),
+            w_in.data_ptr(), _lib.ptr(b_in), _lib.ptr(w_hid), _lib.ptr(b_hid), w_out.data_ptr(), _lib.ptr(b_out),
+            x2.shape[0], D_in, D_hidden, D_out, depth, _lib.NF_ACT[activation], _lib.dtype_code(x.dtype),
+            _lib.current_stream(x.device),
+        )
+        _lib.check(rc, "nf_mlp_fwd")
+
+        ctx.save_for_backward(x, w_in, b_in, w_out, b_out, w_hid, b_hid)
+        ctx.activation = activation
+        ctx.fp16_acc = fp16_acc
+        ctx.depth = depth
+        return o
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    @torch.no_grad()
+    def backward(ctx, do: Tensor):
+        x, w_in, b_in, w_out, b_out, w_hid, b_hid = ctx.saved_tensors
+        B, L, D_in = x.shape
+        D_hidden = w_in.shape[0]
+        D_out = w_out.shape[0]
+        if do.dtype != x.dtype:
+            do = do.to(x.dtype)
+        x2 = _rows2d(x, D_in)
+        do2 = _rows2d(do, D_out)
+        need_dx = ctx.needs_input_grad[0]
+        dx = x.new_empty(x.shape) if need_dx else None
+
+        def acc(t: Optional[Tensor]) -> Optional[Tensor]:
+            return None if t is None else torch.zeros(t.shape, dtype=torch.float32, device=t.device)
+
+        dw_in, db_in, dw_out, db_out, dw_hid, db_hid = (acc(t) for t in (w_in, b_in, w_out, b_out, w_hid, b_hid))
+        lib = _lib.load()
+        rc = lib.nf_mlp_bwd(
+            x2.data_ptr(), x2.stride(0), do2.data_ptr(), do2.stride(0),
+            _lib.ptr(dx), D_in,
+            w_in.data_ptr(), _lib.ptr(b_in), _lib.ptr(w_hid), _lib.ptr(b_hid), w_out.data_ptr(), _lib.ptr(b_out),
+            dw_in.data_ptr(), _lib.ptr(db_in), _lib.ptr(dw_hid), _lib.ptr(db_hid), dw_out.data_ptr(), _lib.ptr(db_out),
+            x2.shape[0], D_in, D_hidden, D_out, ctx.depth, _lib.NF_ACT[ctx.activation], _lib.dtype_code(x.dtype),
+            _lib.current_stream(x.device),
+        )
+        _lib.check(rc, "nf_mlp_bwd")
+        # float32 accumulators; autograd rounds them once to each parameter's dtype
+        return dx, dw_in, db_in, dw_out, db_out, dw_hid, db_hid, None, None
+
+
+def fully_fused_mlp(
+    x: Tensor,
+    w_in: Tensor, b_in: Optional[Tensor],
+    w_out: Tensor, b_out: Optional[Tensor],
+    w_hid: Optional[Tensor] = None, b_hid: Optional[Tensor] = None,
+    activation: str = "relu",
+    fp16_acc: bool = False,
+) -> Tensor:
+    r"""Fully fused forward pass of a small MLP (reference kernel.py:640-686).
+
+    Shapes:
+        - x: :math:`(B, L, D_{in})`
+        - w_in: :math:`(D_{hidden}, D_{in})`, b_in: :math:`(D_{hidden},)` or ``None``
+        - w_out: :math:`(D_{out}, D_{hidden})`, b_out: :math:`(D_{out},)` or ``None``
+        - w_hid: :math:`((depth-1) \cdot D_{hidden}, D_{hidden})`, b_hid: :math:`(depth-1, D_{hidden})` or ``None``
+        - Output: :math:`(B, L, D_{out})`
+
+    ``activation`` is one of ``"relu"``, ``"relu2"``, ``"silu"``, ``"none"`` and is applied after every
+    layer but the last.
+    """
+    return _fully_fused_mlp.apply(x, w_in, b_in, w_out, b_out, w_hid, b_hid, activation, fp16_acc)
