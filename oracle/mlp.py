@@ -35,6 +35,15 @@ def activation(z: Tensor, name: str) -> Tensor:
     raise ValueError(name)
 
 
+def ste_round(t: Tensor, dtype: Optional[torch.dtype]) -> Tensor:
+    """Round to ``dtype`` (back in float32) with a straight-through gradient, so that autograd
+    sees the rounded values -- and therefore the same activation gates as a kernel that stores
+    ``dtype`` between layers -- while the derivative of the rounding itself is taken as one."""
+    if dtype is None:
+        return t
+    return t + (t.detach().to(dtype).to(torch.float32) - t.detach())
+
+
 def split_hidden(w_hid: Optional[Tensor], b_hid: Optional[Tensor], hidden: int):
     """Un-stack ``w_hid``/``b_hid`` into per-layer lists (kernel.py:534-542)."""
     if w_hid is None or w_hid.numel() == 0:
@@ -63,7 +72,7 @@ def mlp_forward(
     """
 
     def rnd(t: Tensor) -> Tensor:
-        return t if round_to is None else t.to(round_to).to(torch.float32)
+        return ste_round(t, round_to)
 
     f32 = lambda t: None if t is None else t.to(torch.float32)  # noqa: E731
     h = rnd(activation(F.linear(f32(x), f32(w_in), f32(b_in)), act))
@@ -83,9 +92,11 @@ def mlp_backward(
     w_hid: Optional[Tensor] = None,
     b_hid: Optional[Tensor] = None,
     act: str = "relu",
+    round_to: Optional[torch.dtype] = None,
 ) -> Dict[str, Optional[Tensor]]:
     """Float32 gradients of ``mlp_forward`` via autograd (the reference tests'
-    baseline, test_fully_fused_mlp.py:253-260)."""
+    baseline, test_fully_fused_mlp.py:253-260).  ``round_to`` evaluates the forward
+    with storage-dtype rounding between layers (what a 16-bit ``nn.Linear`` chain does)."""
     leaves = {}
 
     def leaf(name, t):
@@ -98,6 +109,6 @@ def mlp_backward(
 
     xx = leaf("x", x)
     args = [leaf(n, t) for n, t in (("w_in", w_in), ("b_in", b_in), ("w_out", w_out), ("b_out", b_out), ("w_hid", w_hid), ("b_hid", b_hid))]
-    y = mlp_forward(xx, *args, act=act)
+    y = mlp_forward(xx, *args, act=act, round_to=round_to)
     y.backward(dy.to(torch.float32))
     return {("d" + k): (None if v is None else v.grad) for k, v in leaves.items()}

@@ -25,13 +25,13 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor
 
-from .mlp import activation
+from .mlp import activation, ste_round
 
 
 def _sub(u: Tensor, w1: Tensor, b1, w2: Tensor, b2, i: int, h: int, act: str, rnd) -> Tensor:
     bb1 = None if b1 is None else b1[i]
     bb2 = None if b2 is None else b2[i]
-    t = rnd(activation(F.linear(u, w1[i * h : (i + 1) * h], bb1), act))
+    t = rnd(activation(F.linear(rnd(u), w1[i * h : (i + 1) * h], bb1), act))
     return F.linear(t, w2[i * h : (i + 1) * h], bb2)
 
 
@@ -43,19 +43,23 @@ def rev_forward(
     b2: Optional[Tensor],
     act: str = "gelu",
     round_to: Optional[torch.dtype] = None,
+    stream_round_every: int = 1,
 ) -> Tensor:
-    """Float32 forward over all coupling blocks.  With ``round_to`` the hidden
-    activation and each block's output halves are rounded to that dtype, the
-    points at which a storage-dtype kernel rounds."""
-    rnd = (lambda t: t) if round_to is None else (lambda t: t.to(round_to).to(torch.float32))
+    """Float32 forward over all coupling blocks.  With ``round_to`` every matmul operand
+    (sub-MLP input and hidden activation) is rounded to that dtype, and the residual stream
+    itself after every ``stream_round_every``-th block (0: never) -- the points at which a
+    storage-dtype kernel that runs that many blocks per launch rounds."""
+    rnd = lambda t: ste_round(t, round_to)  # noqa: E731
     f32 = lambda t: None if t is None else t.to(torch.float32)  # noqa: E731
     x, w1, b1, w2, b2 = f32(x), f32(w1), f32(b1), f32(w2), f32(b2)
     h = x.shape[-1] // 2
     blocks = w1.shape[0] // (2 * h)
     x1, x2 = x[..., :h], x[..., h:]
     for k in range(blocks):
-        y1 = rnd(x1 + _sub(x2, w1, b1, w2, b2, 2 * k, h, act, rnd))
-        y2 = rnd(x2 + _sub(y1, w1, b1, w2, b2, 2 * k + 1, h, act, rnd))
+        y1 = x1 + _sub(x2, w1, b1, w2, b2, 2 * k, h, act, rnd)
+        y2 = x2 + _sub(y1, w1, b1, w2, b2, 2 * k + 1, h, act, rnd)
+        if stream_round_every and (k + 1) % stream_round_every == 0:
+            y1, y2 = rnd(y1), rnd(y2)
         x1, x2 = y1, y2
     return torch.cat([x1, x2], -1)
 
@@ -78,7 +82,8 @@ def rev_inverse(
 
 
 def rev_backward(
-    x: Tensor, dy: Tensor, w1: Tensor, b1: Optional[Tensor], w2: Tensor, b2: Optional[Tensor], act: str = "gelu"
+    x: Tensor, dy: Tensor, w1: Tensor, b1: Optional[Tensor], w2: Tensor, b2: Optional[Tensor], act: str = "gelu",
+    round_to: Optional[torch.dtype] = None,
 ) -> Dict[str, Optional[Tensor]]:
     """Float32 gradients via autograd through ``rev_forward`` (stored activations)."""
     leaves = {}
@@ -92,6 +97,6 @@ def rev_backward(
         return v
 
     args = [leaf(n, t) for n, t in (("x", x), ("w1", w1), ("b1", b1), ("w2", w2), ("b2", b2))]
-    y = rev_forward(*args, act=act)
+    y = rev_forward(*args, act=act, round_to=round_to)
     y.backward(dy.to(torch.float32))
     return {("d" + k): (None if v is None else v.grad) for k, v in leaves.items()}
