@@ -1,0 +1,297 @@
+#!/usr/bin/env python3
+"""Benchmark of the neural-field hot paths on one MI355X.
+
+``python bench.py [--gpus 1] [--steps K] [--warmup W]`` prints ONE JSON line.
+
+The headline workload is BASELINE.json ``configs[1]``: multiresolution hash encoding,
+forward + backward, N = 2^20 points, L = 16, F = 2, T = 2^19, fp16 tables, fp16 upstream
+gradient, float32 table gradient.  One step = forward launch + clearing the float32
+gradient table + backward launch(es), inputs resident in HBM.  ``value`` is Mpoints/s.
+
+Extra objects in the same line:
+  roofline      the dominant kernel of the step (longest average launch), algorithmic bytes
+                per launch / measured launch time against the 8 TB/s HBM peak;
+  cpu_baseline  the CPU oracle (a port of the reference's PyTorch path) timed on this host
+                on a 65536-point sample of the same workload;
+  workloads     the other BASELINE configs (fused MLP, reversible MLP, end-to-end step) with
+                their own throughput and MFMA roofline fraction.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16
+
+# geometry of BASELINE configs[1] ("base 16, growth 1.5, L=16" == min_res 16, max_res 7006)
+T, L, F, D, MIN_RES, MAX_RES = 2**19, 16, 2, 3, 16, 7006
+N_POINTS = 2**20
+# algorithmic bytes per point: fwd = 4D + L*2^D*F*2 + L*F*2 ; bwd = 4D + L*F*2 + L*2^D*F*4
+FWD_BYTES_PER_POINT = 4 * D + L * 8 * F * 2 + L * F * 2  # 588
+BWD_BYTES_PER_POINT = 4 * D + L * F * 2 + L * 8 * F * 4  # 1100
+
+
+def event_times(fn, reps):
+    """Per-call GPU duration (ms) of ``fn`` measured with events on the current stream."""
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return [a.elapsed_time(b) for a, b in evs]
+
+
+def wall_time(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e3  # ms per step
+
+
+def bench_hash(steps, warmup):
+    from triton_helpers_amd.layers.hash_encoding import kernel as hk
+    from triton_helpers_amd.layers.hash_encoding.helpers import total_rows
+
+    dev = torch.device("cuda", 0)
+    E = total_rows(T, L, D, MIN_RES, MAX_RES)
+    torch.manual_seed(0)
+    x = torch.rand(N_POINTS, D).to(dev)
+    table = ((torch.rand(E, F) * 2 - 1) * 1e-4).half().to(dev)
+    do = torch.randn(N_POINTS, L * F).half().to(dev)
+    grad = torch.zeros(E, F, dtype=torch.float32, device=dev)
+    pi = torch.tensor([hk.PI_1, hk.PI_2, hk.PI_3], dtype=torch.int64, device=dev)
+
+    def fwd():
+        with torch.no_grad():
+            return hk.hash_encoding(x, table, None, pi, T, MIN_RES, MAX_RES, L)
+
+    def zero():
+        grad.zero_()
+
+    def bwd():
+        hk.hash_encoding_table_grad(x, do, E, F, pi, T, MIN_RES, MAX_RES, L, out=grad)
+
+    def step():
+        fwd()
+        zero()
+        bwd()
+
+    ms = wall_time(step, steps, warmup)
+    reps = max(10, min(steps, 50))
+    t_fwd = statistics.mean(event_times(fwd, reps))
+    t_zero = statistics.mean(event_times(zero, reps))
+    t_bwd = statistics.mean(event_times(bwd, reps))
+
+    # the same step through autograd (table grad rounded to fp16 by the engine), for information
+    e = table.clone().requires_grad_(True)
+
+    def step_autograd():
+        e.grad = None
+        hk.hash_encoding(x, e, None, pi, T, MIN_RES, MAX_RES, L).backward(do)
+
+    ms_autograd = wall_time(step_autograd, max(5, steps // 5), 3)
+    return dict(ms=ms, t_fwd=t_fwd, t_zero=t_zero, t_bwd=t_bwd, ms_autograd=ms_autograd, E=E)
+
+
+def cpu_baseline_hash():
+    """CPU oracle (port of the reference's PyTorch path) on a 65536-point sample of the workload."""
+    from oracle import hash_encoding as O
+
+    n = 65536
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    torch.manual_seed(0)
+    E = O.level_row_offsets(L, T, D, MIN_RES, MAX_RES)[-1]
+    x = torch.rand(n, D)
+    table = ((torch.rand(E, F) * 2 - 1) * 1e-4).half()
+    do = torch.randn(n, L * F).half()
+
+    def run():
+        O.encode_forward(x, table, None, T, L, MIN_RES, MAX_RES)
+        O.encode_backward(x, do, E, F, None, T, L, MIN_RES, MAX_RES)
+
+    run()
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < 10 and len(times) < 20):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    med = statistics.median(times)
+    return {
+        "value": n / med / 1e6,
+        "unit": "Mpoints/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"fwd+bwd of {n} points, same geometry (L=16,F=2,T=2^19), fp16 table, fp32 grad; median of {len(times)} runs",
+    }
+
+
+def bench_mlp(steps, warmup, d_out=16, rows=2**20):
+    from triton_helpers_amd.layers.fully_fused_mlp import kernel as mk
+
+    dev = torch.device("cuda", 0)
+    torch.manual_seed(0)
+
+    def u(shape, fan_in):
+        return ((torch.rand(*shape) * 2 - 1) / fan_in**0.5).bfloat16().to(dev).requires_grad_(True)
+
+    w_in, w_hid, w_out = u((64, 32), 32), u((64, 64), 64), u((d_out, 64), 64)
+    x = torch.randn(1, rows, 32).bfloat16().to(dev).requires_grad_(True)
+    dy = torch.randn(1, rows, d_out).bfloat16().to(dev)
+
+    def step():
+        x.grad = w_in.grad = w_hid.grad = w_out.grad = None
+        mk.fully_fused_mlp(x, w_in, None, w_out, None, w_hid, None, "relu").backward(dy)
+
+    ms = wall_time(step, steps, warmup)
+    flop_row = 3 * 2 * (32 * 64 + 64 * 64 + 64 * d_out)
+    tflops = rows * flop_row / (ms * 1e-3) / 1e12
+    return {
+        "workload": f"fused MLP 32->64->64->{d_out} ReLU bf16 fwd+bwd, {rows} rows (through autograd)",
+        "value": rows / ms / 1e3, "unit": "Mrows/s", "ms_per_step": ms,
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None},
+        "hbm_GBs": rows * 256 / (ms * 1e-3) / 1e9,
+    }
+
+
+def bench_rev(steps, warmup, rows=2**20):
+    from triton_helpers_amd.layers.reversible_mlp import kernel as rk
+
+    dev = torch.device("cuda", 0)
+    torch.manual_seed(0)
+    H, blocks = 64, 4
+    w1 = ((torch.rand(blocks * 2 * H, H) * 2 - 1) / 8).bfloat16().to(dev).requires_grad_(True)
+    w2 = ((torch.rand(blocks * 2 * H, H) * 2 - 1) / 8).bfloat16().to(dev).requires_grad_(True)
+    x = torch.randn(rows, 2 * H).bfloat16().to(dev).requires_grad_(True)
+    dy = torch.randn(rows, 2 * H).bfloat16().to(dev)
+
+    def step():
+        x.grad = w1.grad = w2.grad = None
+        rk.reversible_mlp(x, w1, None, w2, None, "gelu").backward(dy)
+
+    ms = wall_time(step, steps, warmup)
+    flop_row = 3 * 2 * blocks * 4 * H * H
+    tflops = rows * flop_row / (ms * 1e-3) / 1e12
+    return {
+        "workload": f"reversible MLP width 128, 4 couplings, GELU bf16 fwd+bwd, {rows} rows (through autograd)",
+        "value": rows / ms / 1e3, "unit": "Mrows/s", "ms_per_step": ms,
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None},
+    }
+
+
+def bench_e2e(steps, warmup, n=2**21):
+    """BASELINE configs[4]: encode -> MLP 32->64->64->4 -> MSE, forward + backward through autograd."""
+    from triton_helpers_amd.layers.fully_fused_mlp import kernel as mk
+    from triton_helpers_amd.layers.hash_encoding import kernel as hk
+    from triton_helpers_amd.layers.hash_encoding.helpers import total_rows
+
+    dev = torch.device("cuda", 0)
+    torch.manual_seed(0)
+    E = total_rows(T, L, D, MIN_RES, MAX_RES)
+    table = ((torch.rand(E, F) * 2 - 1) * 1e-4).half().to(dev).requires_grad_(True)
+    x = torch.rand(n, D).to(dev)
+    target = torch.rand(n, 4).to(dev)
+
+    def u(shape, fan_in):
+        return ((torch.rand(*shape) * 2 - 1) / fan_in**0.5).bfloat16().to(dev).requires_grad_(True)
+
+    w_in, w_hid, w_out = u((64, 32), 32), u((64, 64), 64), u((4, 64), 64)
+
+    def step():
+        table.grad = w_in.grad = w_hid.grad = w_out.grad = None
+        enc = hk.hash_encoding(x, table, None, None, T, MIN_RES, MAX_RES, L)
+        y = mk.fully_fused_mlp(enc.to(torch.bfloat16).unsqueeze(0), w_in, None, w_out, None, w_hid, None, "relu")
+        loss = torch.nn.functional.mse_loss(y.float().squeeze(0), target)
+        loss.backward()
+
+    ms = wall_time(step, steps, warmup)
+    return {"workload": f"end-to-end step: {n} points -> hash encoding -> MLP 32->64->64->4 -> MSE, fwd+bwd",
+            "value": n / ms / 1e3, "unit": "Mpoints/s", "ms_per_step": ms}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-extras", action="store_true", help="skip the MLP / end-to-end workloads")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (points are independent, so the work "
+              "would shard over points with one gradient all-reduce). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+
+    h = bench_hash(args.steps, args.warmup)
+    kernels = {
+        "hash_fwd": (h["t_fwd"], FWD_BYTES_PER_POINT * N_POINTS),
+        "hash_bwd": (h["t_bwd"], BWD_BYTES_PER_POINT * N_POINTS),
+    }
+    dom = max(kernels, key=lambda k: kernels[k][0])
+    dom_ms, dom_bytes = kernels[dom]
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    step_bytes = (FWD_BYTES_PER_POINT + BWD_BYTES_PER_POINT) * N_POINTS + h["E"] * F * 4
+    out = {
+        "metric": "Mpoints/s fwd+bwd: hash-enc+fused MLP @2^20 pts; % HBM / MFMA peak",
+        "value": N_POINTS / h["ms"] / 1e3,
+        "unit": "Mpoints/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": h["ms"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[1]: hash encoding fwd+bwd, N=2^20 3-D points, L=16, F=2, T=2^19, res 16..7006, "
+                        "fp16 tables and upstream grad, float32 table gradient (zero-fill included in the step)",
+            "points": N_POINTS, "levels": L, "features": F, "table_rows_per_level": T,
+        },
+        "roofline": {
+            "bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "launch_ms": dom_ms, "algorithmic_bytes_per_launch": dom_bytes,
+        },
+        "kernels_ms": {"hash_fwd": h["t_fwd"], "grad_zero_fill": h["t_zero"], "hash_bwd": h["t_bwd"]},
+        "step_roofline_frac": step_bytes / (h["ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "autograd_ms_per_step": h["ms_autograd"],
+    }
+    if not args.no_extras:
+        s, w = max(5, args.steps // 2), max(3, args.warmup // 2)
+        out["workloads"] = {
+            "configs[2]": bench_mlp(s, w, 16),
+            "configs[3]": bench_rev(max(3, s // 2), 2),
+            "configs[4]": bench_e2e(max(3, s // 2), 2),
+        }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline_hash()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
