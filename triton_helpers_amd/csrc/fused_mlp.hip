@@ -60,6 +60,18 @@ __device__ __forceinline__ void layer_mma(f32x4_t (&acc)[2][4], const Frag (&in)
   }
 }
 
+// activation + rounding of a hidden layer; the packed tiles become the next layer's B fragments
+template <typename T, int KC_H, bool RELU>
+__device__ __forceinline__ void hidden_epilogue(const f32x4_t (&acc)[2][4], Frag (&in)[2][2], int act) {
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int kc = 0; kc < KC_H; ++kc) {
+      act_pack<T, RELU>(acc[nt][2 * kc], act, in[nt][kc].w[0], in[nt][kc].w[1]);
+      act_pack<T, RELU>(acc[nt][2 * kc + 1], act, in[nt][kc].w[2], in[nt][kc].w[3]);
+    }
+}
+
 // ---------------------------------------------------------------------------------------
 // Forward
 // ---------------------------------------------------------------------------------------
@@ -90,41 +102,40 @@ __global__ __launch_bounds__(256) void mlp_fwd_k(MlpArgs a) {
   stage_bias<T>(bias_out, a.b_out, a.d_out, OUTP, tid, nthreads);
   __syncthreads();
 
+  const bool relu = a.act == NF_ACT_RELU;
   const int64_t n_chunks = (a.rows + 31) / 32;
   const int64_t wave_stride = (int64_t)gridDim.x * a.waves;
-  for (int64_t chunk = (int64_t)blockIdx.x * a.waves + wave; chunk < n_chunks; chunk += wave_stride) {
+  // the next chunk's rows are requested before the current chunk is computed (loads past the end return zeros)
+  Frag nxt[2][2];
+  const int64_t first_chunk = (int64_t)blockIdx.x * a.waves + wave;
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int kc = 0; kc < KC_IN; ++kc)
+      nxt[nt][kc] = load_rows_frag(a.x, a.x_stride, first_chunk * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+  for (int64_t chunk = first_chunk; chunk < n_chunks; chunk += wave_stride) {
     const int64_t row0 = chunk * 32;
     Frag in[2][2];
     f32x4_t acc[2][4];
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-      for (int kc = 0; kc < KC_IN; ++kc)
-        in[nt][kc] = load_rows_frag(a.x, a.x_stride, row0 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+      for (int kc = 0; kc < KC_IN; ++kc) {
+        in[nt][kc] = nxt[nt][kc];
+        nxt[nt][kc] = load_rows_frag(a.x, a.x_stride, (chunk + wave_stride) * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+      }
 
     layer_mma<T, MT_H, KC_IN>(acc, in, f_in, bias_in, lane);
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int kc = 0; kc < KC_H; ++kc) {
-        const f32x4_t lo = acc[nt][2 * kc], hi = acc[nt][2 * kc + 1];
-        in[nt][kc].w[0] = pack2<T>(act_fwd(lo[0], a.act), act_fwd(lo[1], a.act));
-        in[nt][kc].w[1] = pack2<T>(act_fwd(lo[2], a.act), act_fwd(lo[3], a.act));
-        in[nt][kc].w[2] = pack2<T>(act_fwd(hi[0], a.act), act_fwd(hi[1], a.act));
-        in[nt][kc].w[3] = pack2<T>(act_fwd(hi[2], a.act), act_fwd(hi[3], a.act));
-      }
+    if (relu)
+      hidden_epilogue<T, KC_H, true>(acc, in, a.act);
+    else
+      hidden_epilogue<T, KC_H, false>(acc, in, a.act);
     for (int k = 0; k < n_hid; ++k) {
       layer_mma<T, MT_H, KC_H>(acc, in, f_hid + (size_t)k * MT_H * KC_H * FRAG_ELEMS, bias_hid + k * HP, lane);
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int kc = 0; kc < KC_H; ++kc) {
-          const f32x4_t lo = acc[nt][2 * kc], hi = acc[nt][2 * kc + 1];
-          in[nt][kc].w[0] = pack2<T>(act_fwd(lo[0], a.act), act_fwd(lo[1], a.act));
-          in[nt][kc].w[1] = pack2<T>(act_fwd(lo[2], a.act), act_fwd(lo[3], a.act));
-          in[nt][kc].w[2] = pack2<T>(act_fwd(hi[0], a.act), act_fwd(hi[1], a.act));
-          in[nt][kc].w[3] = pack2<T>(act_fwd(hi[2], a.act), act_fwd(hi[3], a.act));
-        }
+      if (relu)
+        hidden_epilogue<T, KC_H, true>(acc, in, a.act);
+      else
+        hidden_epilogue<T, KC_H, false>(acc, in, a.act);
     }
     layer_mma<T, MT_O, KC_H>(acc, in, f_out, bias_out, lane);
 #pragma unroll
@@ -163,6 +174,25 @@ __device__ __forceinline__ Frag panel_frag(const uint16_t* panel, int t, int lan
   Frag f;
   f.u = *reinterpret_cast<const uint4*>(panel + (16 * t + (lane & 15)) * TPITCH + 8 * (lane >> 4));
   return f;
+}
+
+// forward recompute of one layer inside the backward: activation, park h^T, park the gate image
+template <typename T, int MT_H, bool RELU>
+__device__ __forceinline__ void recompute_epilogue(const f32x4_t (&acc)[2][4], Frag (&in)[2][2], uint16_t* panel, uint32_t* im,
+                                                   int act, int lane) {
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < MT_H; ++mt) {
+      uint32_t h01, h23, g01, g23;
+      act_pack<T, RELU>(acc[nt][mt], act, h01, h23);
+      gate_pack<T, RELU>(acc[nt][mt], act, h01, h23, g01, g23);
+      in[nt][mt >> 1].w[2 * (mt & 1)] = h01;
+      in[nt][mt >> 1].w[2 * (mt & 1) + 1] = h23;
+      park_tile_T(panel, mt, nt, lane, h01, h23);
+      im[((mt * 2 + nt) * 2 + 0) * 64 + lane] = g01;
+      im[((mt * 2 + nt) * 2 + 1) * 64 + lane] = g23;
+    }
 }
 
 // dW tile (mt over output features, nt over input features): lane (n, g) reg r is
@@ -244,22 +274,43 @@ __global__ __launch_bounds__(256) void mlp_bwd_k(MlpArgs a) {
       for (int j = 0; j < MT_H; ++j) dw_hid[h][i][j] = zero4;
     }
   const bool want_db = a.db_in != nullptr || a.db_hid != nullptr;  // db_out is a separate pass over dy
+  const bool relu = a.act == NF_ACT_RELU;
 
   const int64_t n_chunks = (a.rows + 31) / 32;
   const int64_t wave_stride = (int64_t)gridDim.x * a.waves;
-  for (int64_t chunk = (int64_t)blockIdx.x * a.waves + wave; chunk < n_chunks; chunk += wave_stride) {
+  // the next chunk's x and dy rows are requested before the current chunk is computed
+  Frag nx[2][2], ndy[2][2];
+  const int64_t first_chunk = (int64_t)blockIdx.x * a.waves + wave;
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+    for (int kc = 0; kc < KC_IN; ++kc)
+      nx[nt][kc] = load_rows_frag(a.x, a.x_stride, first_chunk * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+#pragma unroll
+    for (int kc = 0; kc < KC_O; ++kc)
+      ndy[nt][kc] = load_rows_frag(a.dy, a.dy_stride, first_chunk * 32 + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
+  }
+  for (int64_t chunk = first_chunk; chunk < n_chunks; chunk += wave_stride) {
     const int64_t row0 = chunk * 32;
     Frag in[2][2];
     f32x4_t acc[2][4];
+    Frag dz[2][2];
 
     // ---------------- forward recompute; park inputs (transposed) and act'(z) ----------------
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+    for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
       for (int kc = 0; kc < KC_IN; ++kc) {
-        in[nt][kc] = load_rows_frag(a.x, a.x_stride, row0 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+        in[nt][kc] = nx[nt][kc];
+        nx[nt][kc] = load_rows_frag(a.x, a.x_stride, (chunk + wave_stride) * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
         park_frag_T(xT, kc, nt, lane, in[nt][kc]);
       }
+#pragma unroll
+      for (int kc = 0; kc < KC_O; ++kc) {
+        dz[nt][kc] = ndy[nt][kc];
+        ndy[nt][kc] = load_rows_frag(a.dy, a.dy_stride, (chunk + wave_stride) * 32 + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
+      }
+    }
     for (int k = 1; k <= a.depth; ++k) {
       if (k == 1)
         layer_mma<T, MT_H, KC_IN>(acc, in, f_in, bias_in, lane);
@@ -267,30 +318,17 @@ __global__ __launch_bounds__(256) void mlp_bwd_k(MlpArgs a) {
         layer_mma<T, MT_H, KC_H>(acc, in, f_hid + (size_t)(k - 2) * MT_H * KC_H * FRAG_ELEMS, bias_hid + (k - 2) * HP, lane);
       uint16_t* panel = hT + (size_t)(k - 1) * HP * TPITCH;
       uint32_t* im = img + (size_t)(k - 1) * MT_H * 2 * 2 * 64;
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < MT_H; ++mt) {
-          const f32x4_t z = acc[nt][mt];
-          const uint32_t h01 = pack2<T>(act_fwd(z[0], a.act), act_fwd(z[1], a.act));
-          const uint32_t h23 = pack2<T>(act_fwd(z[2], a.act), act_fwd(z[3], a.act));
-          in[nt][mt >> 1].w[2 * (mt & 1)] = h01;
-          in[nt][mt >> 1].w[2 * (mt & 1) + 1] = h23;
-          park_tile_T(panel, mt, nt, lane, h01, h23);
-          im[((mt * 2 + nt) * 2 + 0) * 64 + lane] = pack2<T>(act_grad(z[0], a.act), act_grad(z[1], a.act));
-          im[((mt * 2 + nt) * 2 + 1) * 64 + lane] = pack2<T>(act_grad(z[2], a.act), act_grad(z[3], a.act));
-        }
+      if (relu)
+        recompute_epilogue<T, MT_H, true>(acc, in, panel, im, a.act, lane);
+      else
+        recompute_epilogue<T, MT_H, false>(acc, in, panel, im, a.act, lane);
     }
 
     // ---------------- output layer: dz_out = dy ----------------
-    Frag dz[2][2];
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-      for (int kc = 0; kc < KC_O; ++kc) {
-        dz[nt][kc] = load_rows_frag(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
-        park_frag_T(dzT, kc, nt, lane, dz[nt][kc]);
-      }
+      for (int kc = 0; kc < KC_O; ++kc) park_frag_T(dzT, kc, nt, lane, dz[nt][kc]);
     {
       const uint16_t* hprev = hT + (size_t)(a.depth - 1) * HP * TPITCH;
       Frag hb[MT_H];
@@ -326,10 +364,11 @@ __global__ __launch_bounds__(256) void mlp_bwd_k(MlpArgs a) {
         for (int mt = 0; mt < MT_H; ++mt) {
           const uint32_t g01 = im[((mt * 2 + nt) * 2 + 0) * 64 + lane];
           const uint32_t g23 = im[((mt * 2 + nt) * 2 + 1) * 64 + lane];
-          const f32x4_t dh = acc[nt][mt];
-          const float d0 = dh[0] * unpack_lo<T>(g01), d1 = dh[1] * unpack_hi<T>(g01);
-          const float d2 = dh[2] * unpack_lo<T>(g23), d3 = dh[3] * unpack_hi<T>(g23);
-          const uint32_t p01 = pack2<T>(d0, d1), p23 = pack2<T>(d2, d3);
+          uint32_t p01, p23;
+          if (relu)
+            gate_apply<T, true>(acc[nt][mt], g01, g23, p01, p23);
+          else
+            gate_apply<T, false>(acc[nt][mt], g01, g23, p01, p23);
           dz[nt][mt >> 1].w[2 * (mt & 1)] = p01;
           dz[nt][mt >> 1].w[2 * (mt & 1) + 1] = p23;
           park_tile_T(dzT, mt, nt, lane, p01, p23);
@@ -583,7 +622,7 @@ static int launch_fwd(const MlpArgs& a0, hipStream_t s) {
   a.waves = 4;
   const int64_t chunks = (a.rows + 31) / 32;
   int64_t blocks = (chunks + a.waves - 1) / a.waves;
-  const int64_t cap = (int64_t)device_cus() * (lds > 64 * 1024 ? 1 : 2);
+  const int64_t cap = (int64_t)device_cus() * (lds > 64 * 1024 ? 1 : (lds > 40 * 1024 ? 2 : 3));
   if (blocks > cap) blocks = cap;
   auto kern = mlp_fwd_k<T, KIN, HP, OUTP>;
   if (lds > 64 * 1024) {

@@ -48,14 +48,35 @@ __device__ __forceinline__ f32x4_t mfma16<F16>(const Frag& a, const Frag& b, f32
 __host__ __device__ __forceinline__ int k_nat(int kc, int g, int j) { return 32 * kc + 8 * g + j; }
 __host__ __device__ __forceinline__ int k_chain(int kc, int g, int j) { return 32 * kc + 16 * (j >> 2) + 4 * g + (j & 3); }
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+// Two floats -> one dword of 16-bit values, round-to-nearest-even, one v_cvt_pk_* instruction on gfx950.
 template <typename T>
-__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-  return (uint32_t)T::from_f32(lo) | ((uint32_t)T::from_f32(hi) << 16);
+__device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <>
+__device__ __forceinline__ uint32_t pack2<BF16>(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+template <>
+__device__ __forceinline__ uint32_t pack2<F16>(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
 }
 template <typename T>
-__device__ __forceinline__ float unpack_lo(uint32_t v) { return T::to_f32((uint16_t)(v & 0xffffu)); }
+__device__ __forceinline__ float unpack_lo(uint32_t v);
 template <typename T>
-__device__ __forceinline__ float unpack_hi(uint32_t v) { return T::to_f32((uint16_t)(v >> 16)); }
+__device__ __forceinline__ float unpack_hi(uint32_t v);
+template <>
+__device__ __forceinline__ float unpack_lo<BF16>(uint32_t v) { return __uint_as_float(v << 16); }
+template <>
+__device__ __forceinline__ float unpack_hi<BF16>(uint32_t v) { return __uint_as_float(v & 0xffff0000u); }
+template <>
+__device__ __forceinline__ float unpack_lo<F16>(uint32_t v) { return (float)__builtin_bit_cast(f16x2_t, v)[0]; }
+template <>
+__device__ __forceinline__ float unpack_hi<F16>(uint32_t v) { return (float)__builtin_bit_cast(f16x2_t, v)[1]; }
 
 // ---- activations (triton_helpers/ops.py:37-66 of the reference; gelu = exact erf form) ----
 __device__ __forceinline__ float act_fwd(float z, int act) {
@@ -85,6 +106,41 @@ __device__ __forceinline__ float act_grad(float z, int act) {
   }
 }
 
+// h = act(z) packed to 16 bit.  RELU = true is the branch-free fast path; otherwise `act` selects at run time.
+template <typename T, bool RELU>
+__device__ __forceinline__ void act_pack(const f32x4_t z, int act, uint32_t& p01, uint32_t& p23) {
+  if (RELU) {
+    p01 = pack2<T>(fmaxf(z[0], 0.0f), fmaxf(z[1], 0.0f));
+    p23 = pack2<T>(fmaxf(z[2], 0.0f), fmaxf(z[3], 0.0f));
+  } else {
+    p01 = pack2<T>(act_fwd(z[0], act), act_fwd(z[1], act));
+    p23 = pack2<T>(act_fwd(z[2], act), act_fwd(z[3], act));
+  }
+}
+// What the backward keeps per pre-activation: for ReLU the activation itself (its sign bit pattern
+// tells the gate: h != 0  <=>  z > 0); otherwise act'(z) rounded to 16 bit.
+template <typename T, bool RELU>
+__device__ __forceinline__ void gate_pack(const f32x4_t z, int act, uint32_t h01, uint32_t h23, uint32_t& g01, uint32_t& g23) {
+  if (RELU) {
+    g01 = h01;
+    g23 = h23;
+  } else {
+    g01 = pack2<T>(act_grad(z[0], act), act_grad(z[1], act));
+    g23 = pack2<T>(act_grad(z[2], act), act_grad(z[3], act));
+  }
+}
+// dz = dh * act'(z) from the parked gate image, packed to 16 bit.
+template <typename T, bool RELU>
+__device__ __forceinline__ void gate_apply(const f32x4_t dh, uint32_t g01, uint32_t g23, uint32_t& p01, uint32_t& p23) {
+  if (RELU) {
+    p01 = pack2<T>((g01 & 0xffffu) ? dh[0] : 0.0f, (g01 >> 16) ? dh[1] : 0.0f);
+    p23 = pack2<T>((g23 & 0xffffu) ? dh[2] : 0.0f, (g23 >> 16) ? dh[3] : 0.0f);
+  } else {
+    p01 = pack2<T>(dh[0] * unpack_lo<T>(g01), dh[1] * unpack_hi<T>(g01));
+    p23 = pack2<T>(dh[2] * unpack_lo<T>(g23), dh[3] * unpack_hi<T>(g23));
+  }
+}
+
 // ---- staging weights into LDS as A fragments ------------------------------------------
 // dst: fragment array [MT][KC][64 lanes][8 elements]; element (mt, kc, lane(m,g), j) =
 //   transposed ? W[kmap(kc,g,j)][16*mt+m] : W[16*mt+m][kmap(kc,g,j)]
@@ -92,18 +148,45 @@ __device__ __forceinline__ float act_grad(float z, int act) {
 template <bool CHAIN, bool TRANSPOSED>
 __device__ __forceinline__ void stage_weight_frags(uint16_t* dst, const uint16_t* w, int w_rows, int w_cols, int MT,
                                                    int KC, int tid, int nthreads) {
-  const int total = MT * KC * 64 * 8;
-  for (int e = tid; e < total; e += nthreads) {
-    const int j = e & 7;
-    const int lane = (e >> 3) & 63;
-    const int frag = e >> 9;
+  // one unit = the 8 elements of one lane of one fragment; the 8 loads of a unit are independent
+  const int units = MT * KC * 64;
+  const bool vec_ok = !TRANSPOSED && (w_cols % 4 == 0) && ((uintptr_t)w % 8 == 0);
+  for (int u = tid; u < units; u += nthreads) {
+    const int lane = u & 63;
+    const int frag = u >> 6;
     const int kc = frag % KC, mt = frag / KC;
     const int m = 16 * mt + (lane & 15);
     const int g = lane >> 4;
-    const int k = CHAIN ? k_chain(kc, g, j) : k_nat(kc, g, j);
-    const int r = TRANSPOSED ? k : m;
-    const int c = TRANSPOSED ? m : k;
-    dst[e] = (r < w_rows && c < w_cols) ? w[(size_t)r * w_cols + c] : (uint16_t)0;
+    uint16_t v[8];
+    if (vec_ok && m < w_rows) {
+      // non-transposed rows are contiguous in k: two 8-byte pieces (chain order) or one 16-byte run (natural)
+      const int k0 = CHAIN ? k_chain(kc, g, 0) : k_nat(kc, g, 0);
+      const int k1 = CHAIN ? k_chain(kc, g, 4) : k_nat(kc, g, 4);
+      uint2 lo = make_uint2(0u, 0u), hi = make_uint2(0u, 0u);
+      if (k0 + 4 <= w_cols) lo = *reinterpret_cast<const uint2*>(w + (size_t)m * w_cols + k0);
+      else
+        for (int j = 0; j < 4; ++j)
+          if (k0 + j < w_cols) reinterpret_cast<uint16_t*>(&lo)[j] = w[(size_t)m * w_cols + k0 + j];
+      if (k1 + 4 <= w_cols) hi = *reinterpret_cast<const uint2*>(w + (size_t)m * w_cols + k1);
+      else
+        for (int j = 0; j < 4; ++j)
+          if (k1 + j < w_cols) reinterpret_cast<uint16_t*>(&hi)[j] = w[(size_t)m * w_cols + k1 + j];
+      *reinterpret_cast<uint4*>(dst + (size_t)u * 8) = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      continue;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k = CHAIN ? k_chain(kc, g, j) : k_nat(kc, g, j);
+      const int r = TRANSPOSED ? k : m;
+      const int c = TRANSPOSED ? m : k;
+      v[j] = (r < w_rows && c < w_cols) ? w[(size_t)r * w_cols + c] : (uint16_t)0;
+    }
+    uint4 o;
+    o.x = (uint32_t)v[0] | ((uint32_t)v[1] << 16);
+    o.y = (uint32_t)v[2] | ((uint32_t)v[3] << 16);
+    o.z = (uint32_t)v[4] | ((uint32_t)v[5] << 16);
+    o.w = (uint32_t)v[6] | ((uint32_t)v[7] << 16);
+    *reinterpret_cast<uint4*>(dst + (size_t)u * 8) = o;
   }
 }
 
