@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define NF_ABI_VERSION 1
+#define NF_ABI_VERSION 2
 
 /* element types */
 enum { NF_F32 = 0, NF_F16 = 1, NF_BF16 = 2 };
@@ -65,7 +65,8 @@ typedef struct nf_hash_geom {
 
 /* flags for the hash-encoding entry points */
 enum {
-  NF_HASH_FORCE_GENERIC = 1    /* use the one-thread-per-(point,level) kernel even where the tiled kernel applies */
+  NF_HASH_FORCE_GENERIC = 1,   /* use the one-thread-per-(point,level) kernel even where a faster kernel applies */
+  NF_HASH_FORCE_ATOMIC = 2     /* backward: scatter with global atomics even where the LDS-tile kernels apply */
 };
 
 int nf_abi_version(void);
@@ -81,10 +82,19 @@ int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t coords_stri
                        const nf_hash_geom* geom, const int64_t* primes, float scale, int flags, void* stream);
 
 /* dtable[row_offset[l] + row_j, f] += w_j * dout[n, l*F + f]   (float32 accumulators,
- * NOT cleared by the call).  dout rows of dout_dtype with row stride dout_stride_n. */
+ * NOT cleared by the call).  dout rows of dout_dtype with row stride dout_stride_n.
+ * workspace: optional device scratch of at least nf_hash_encode_bwd_workspace_bytes() bytes (4-byte
+ * aligned); with it, large batches accumulate in LDS tiles instead of scattering global atomics.
+ * NULL / too small selects the atomic kernels.  Its contents are undefined afterwards. */
 int nf_hash_encode_bwd(const void* coords, int coords_dtype, int64_t coords_stride_n, int64_t coords_stride_d,
                        const void* dout, int dout_dtype, int64_t dout_stride_n, float* dtable, int64_t n_points,
-                       const nf_hash_geom* geom, const int64_t* primes, float scale, int flags, void* stream);
+                       const nf_hash_geom* geom, const int64_t* primes, float scale, void* workspace,
+                       int64_t workspace_bytes, int flags, void* stream);
+
+/* Scratch bytes nf_hash_encode_bwd can use for this call shape; 0 when the workspace would not be used.
+ * (No counterpart in the reference: its backward allocates nothing besides the gradient table,
+ * triton_helpers/layers/hash_encoding/kernel.py:636.) */
+int64_t nf_hash_encode_bwd_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype);
 
 /* Level-local table rows of all 2^D corners: out_rows [n_points, L, 2^D] int64, and
  * (optional, may be NULL) the interpolation weights out_w [n_points, L, 2^D] float32. */

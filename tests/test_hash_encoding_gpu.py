@@ -135,10 +135,11 @@ def test_forward_config0_full_size():
 
 
 @pytest.mark.parametrize("N,D,F,T,L,lo,hi,scale", CASES + [(65536, 3, 2, 2**20, 16, 16, 512, 1.0), (131072, 3, 2, 2**14, 16, 16, 512, 1.0)])
-@pytest.mark.parametrize("do_dtype,force_generic", [(torch.float32, True), (torch.float16, False), (torch.float16, True)])
-def test_backward_vs_oracle(N, D, F, T, L, lo, hi, scale, do_dtype, force_generic, monkeypatch):
+@pytest.mark.parametrize("do_dtype,flags", [(torch.float32, 1), (torch.float16, 0), (torch.float16, 1), (torch.float16, 2)])
+def test_backward_vs_oracle(N, D, F, T, L, lo, hi, scale, do_dtype, flags, monkeypatch):
+    """flags: 0 = default dispatch (LDS-tile kernels from 32768 points), 1 = generic, 2 = scattered atomics."""
     hk = _hk()
-    monkeypatch.setattr(hk, "_FLAGS", 1 if force_generic else 0)
+    monkeypatch.setattr(hk, "_FLAGS", flags)
     torch.manual_seed(0)
     x = torch.rand(N, D)
     E = O.level_row_offsets(L, T, D, lo, hi)[-1]
@@ -147,6 +148,39 @@ def test_backward_vs_oracle(N, D, F, T, L, lo, hi, scale, do_dtype, force_generi
     got = hk.hash_encoding_table_grad(x.to(DEV) * scale, do.to(DEV), E, F, None, T, lo, hi, L, scale)
     assert got.dtype == torch.float32
     torch.testing.assert_close(got.cpu(), want, rtol=1e-3, atol=1e-4)
+
+
+@pytest.mark.parametrize("do_dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize(
+    "N,T,L,lo,hi",
+    [
+        (40000, 2**14, 16, 16, 512),    # every hashed level is exactly one LDS tile
+        (33000, 2**19, 16, 16, 7006),   # bench geometry: 32 tiles per hashed level, dense levels of 1, 1, 4 and 11 tiles
+        (50001, 2**16, 8, 16, 2048),    # 4 tiles per hashed level, ragged point count
+        (40000, 2**19, 4, 4096, 30000), # resolutions above the tile size: the x corner moves the tile id
+        (45000, 2**12, 4, 8, 64),       # hashed levels smaller than a tile
+    ],
+)
+def test_backward_lds_tile_path(N, T, L, lo, hi, do_dtype):
+    """The LDS-tile backward (plan + scan kernels) against the oracle and against the scattered-atomic kernel."""
+    hk = _hk()
+    torch.manual_seed(3)
+    x = torch.rand(N, 3)
+    x[:7] = torch.tensor([[0.0, 0.0, 0.0], [1.0, 1.0, 1.0], [1.0, 0.0, 0.5], [0.999999, 0.5, 0.25], [0.5, 1.0, 0.0],
+                          [0.25, 0.25, 1.0], [1.0, 1.0, 0.0]])
+    E = O.level_row_offsets(L, T, 3, lo, hi)[-1]
+    do = torch.randn(N, L * 2).to(do_dtype)
+    do[100:200] = 0  # rows with no upstream gradient are skipped
+    want = O.encode_backward(x, do, E, 2, None, T, L, lo, hi)
+    hk._FLAGS = 0
+    got = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, 2, None, T, lo, hi, L)
+    hk._FLAGS = 2
+    try:
+        ref = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, 2, None, T, lo, hi, L)
+    finally:
+        hk._FLAGS = 0
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-3, atol=1e-4)
+    torch.testing.assert_close(got, ref, rtol=1e-3, atol=1e-4)
 
 
 def test_autograd_round_trip_fp16_table():

@@ -14,12 +14,13 @@ import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "libnf_cdna4.so"
 
-NF_ABI_VERSION = 1
+NF_ABI_VERSION = 2
 NF_F32, NF_F16, NF_BF16 = 0, 1, 2
 NF_ACT = {"none": 0, "relu": 1, "silu": 2, "relu2": 3, "gelu": 4}
 NF_MAX_LEVELS = 32
 NF_MAX_DIMS = 4
 NF_HASH_FORCE_GENERIC = 1
+NF_HASH_FORCE_ATOMIC = 2
 
 _DTYPE_CODE = {torch.float32: NF_F32, torch.float16: NF_F16, torch.bfloat16: NF_BF16}
 
@@ -28,6 +29,7 @@ EXPORTS = (
     "nf_last_error",
     "nf_hash_encode_fwd",
     "nf_hash_encode_bwd",
+    "nf_hash_encode_bwd_workspace_bytes",
     "nf_hash_encode_indices",
     "nf_mlp_fwd",
     "nf_mlp_bwd",
@@ -74,7 +76,9 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.nf_hash_encode_fwd.restype = c_int
     lib.nf_hash_encode_fwd.argtypes = [P, I, I64, I64, P, I, P, I64, I64, POINTER(HashGeom), P, c_float, I, P]
     lib.nf_hash_encode_bwd.restype = c_int
-    lib.nf_hash_encode_bwd.argtypes = [P, I, I64, I64, P, I, I64, P, I64, POINTER(HashGeom), P, c_float, I, P]
+    lib.nf_hash_encode_bwd.argtypes = [P, I, I64, I64, P, I, I64, P, I64, POINTER(HashGeom), P, c_float, P, I64, I, P]
+    lib.nf_hash_encode_bwd_workspace_bytes.restype = c_int64
+    lib.nf_hash_encode_bwd_workspace_bytes.argtypes = [I64, POINTER(HashGeom), I]
     lib.nf_hash_encode_indices.restype = c_int
     lib.nf_hash_encode_indices.argtypes = [P, I, I64, I64, P, P, I64, POINTER(HashGeom), P, c_float, P]
     lib.nf_mlp_fwd.restype = c_int

@@ -33,7 +33,7 @@ COMMON_FLAGS = [
     f"-I{CSRC}",
 ]
 # Files whose float arithmetic must not be contracted into FMAs (bit-exact cell / weight math).
-NO_CONTRACT = {"hash_encoding.hip"}
+NO_CONTRACT = {"hash_encoding.hip", "hash_encoding_bwd_scan.hip"}
 
 
 def _hipcc() -> str:

@@ -9,17 +9,9 @@
 //   hashed level:                   row = (xor_d (cell_d + bit_d) * pi_d) mod T_l   (64-bit products)
 //   weight_j = prod_d (bit_d ? frac_d : 1 - frac_d),   out = sum_j weight_j * table[row_j]
 // The file is compiled with -ffp-contract=off so that none of this is fused.
-#include "nf_common.h"
+#include "hash_common.h"
 
 namespace nf {
-
-struct DevGeom {
-  int dims, feat, levels, first_hash;
-  uint64_t max_rows;
-  int res[NF_MAX_LEVELS];
-  uint32_t rows[NF_MAX_LEVELS];
-  int64_t row_offset[NF_MAX_LEVELS];
-};
 
 // ---------------------------------------------------------------------------
 // Generic path: one thread per (point, level); any D <= 4, any F, any dtype mix.
@@ -160,56 +152,6 @@ __global__ __launch_bounds__(256) void hash_indices_k(const void* coords, int cd
 // as full 16-byte pieces of contiguous output rows; the backward stages the
 // incoming gradient rows the same way before scattering.
 // ---------------------------------------------------------------------------
-constexpr int TILE_THREADS = 256;
-
-struct Corner8 {
-  uint32_t row[8];
-};
-
-__device__ __forceinline__ Corner8 rows_d3(const uint32_t c[3], bool hashed, uint32_t res, uint32_t mask,
-                                           const uint32_t pi[3]) {
-  Corner8 r;
-  if (hashed) {
-    // (c+1)*pi == c*pi + pi in 32-bit wrap-around arithmetic; the low 32 bits of the
-    // 64-bit products are all a power-of-two modulus keeps.
-    const uint32_t x0 = c[0] * pi[0], x1 = x0 + pi[0];
-    const uint32_t y0 = c[1] * pi[1], y1 = y0 + pi[1];
-    const uint32_t z0 = c[2] * pi[2], z1 = z0 + pi[2];
-    r.row[0] = (x0 ^ y0 ^ z0) & mask;
-    r.row[1] = (x1 ^ y0 ^ z0) & mask;
-    r.row[2] = (x0 ^ y1 ^ z0) & mask;
-    r.row[3] = (x1 ^ y1 ^ z0) & mask;
-    r.row[4] = (x0 ^ y0 ^ z1) & mask;
-    r.row[5] = (x1 ^ y0 ^ z1) & mask;
-    r.row[6] = (x0 ^ y1 ^ z1) & mask;
-    r.row[7] = (x1 ^ y1 ^ z1) & mask;
-  } else {
-    const uint32_t r2 = res * res;
-    const uint32_t b = c[0] + c[1] * res + c[2] * r2;
-    r.row[0] = b;
-    r.row[1] = b + 1;
-    r.row[2] = b + res;
-    r.row[3] = b + res + 1;
-    r.row[4] = b + r2;
-    r.row[5] = b + r2 + 1;
-    r.row[6] = b + r2 + res;
-    r.row[7] = b + r2 + res + 1;
-  }
-  return r;
-}
-
-__device__ __forceinline__ void weights_d3(const float f[3], float w[8]) {
-  const float gx = 1.0f - f[0], gy = 1.0f - f[1], gz = 1.0f - f[2];
-  w[0] = (gx * gy) * gz;
-  w[1] = (f[0] * gy) * gz;
-  w[2] = (gx * f[1]) * gz;
-  w[3] = (f[0] * f[1]) * gz;
-  w[4] = (gx * gy) * f[2];
-  w[5] = (f[0] * gy) * f[2];
-  w[6] = (gx * f[1]) * f[2];
-  w[7] = (f[0] * f[1]) * f[2];
-}
-
 template <typename TT, int PPT>
 __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_tiled_k(const void* coords, int cdt, int64_t csn, int64_t csd,
                                                                  const uint32_t* table, uint16_t* out,
@@ -369,35 +311,8 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_bwd_tiled_k(const void* coo
 // ---------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------
-static int make_dev_geom(const nf_hash_geom* geom, DevGeom* d) {
-  NF_REQUIRE(geom != nullptr, NF_EINVAL, "geom is NULL");
-  NF_REQUIRE(geom->dims >= 1 && geom->dims <= NF_MAX_DIMS, NF_EINVAL, "dims=%d outside 1..%d", geom->dims,
-             NF_MAX_DIMS);
-  NF_REQUIRE(geom->feat >= 1, NF_EINVAL, "feat=%d must be positive", geom->feat);
-  NF_REQUIRE(geom->levels >= 1 && geom->levels <= NF_MAX_LEVELS, NF_EINVAL, "levels=%d outside 1..%d", geom->levels,
-             NF_MAX_LEVELS);
-  d->dims = geom->dims;
-  d->feat = geom->feat;
-  d->levels = geom->levels;
-  d->first_hash = geom->first_hash_level;
-  d->max_rows = (uint64_t)geom->max_rows;
-  for (int l = 0; l < geom->levels; ++l) {
-    NF_REQUIRE(geom->res[l] >= 1, NF_EINVAL, "res[%d]=%d must be positive", l, geom->res[l]);
-    NF_REQUIRE(geom->rows[l] >= 1 && geom->rows[l] < (int64_t)1 << 32, NF_EINVAL, "rows[%d]=%lld outside 1..2^32-1", l,
-               (long long)geom->rows[l]);
-    NF_REQUIRE(geom->row_offset[l] >= 0, NF_EINVAL, "row_offset[%d] negative", l);
-    // a dense level must be able to hold every corner the stride-N_l indexing can produce
-    if (l < geom->first_hash_level) {
-      double need = 1.0;
-      for (int k = 0; k < geom->dims; ++k) need *= (double)geom->res[l] + 1.0;
-      NF_REQUIRE(need <= (double)geom->rows[l], NF_EINVAL, "level %d marked dense but (res+1)^D > rows", l);
-    }
-    d->res[l] = geom->res[l];
-    d->rows[l] = (uint32_t)geom->rows[l];
-    d->row_offset[l] = geom->row_offset[l];
-  }
-  return 0;
-}
+// below this many points the scattered-atomic kernels are faster than planning + scanning
+constexpr int64_t SCAN_MIN_POINTS = 32768;
 
 static bool tiled_ok(const nf_hash_geom* g, int table_dt, const void* rows_ptr, int64_t row_stride) {
   if (g->dims != 3 || g->feat != 2 || table_dt == NF_F32) return false;
@@ -473,10 +388,15 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
   }
 }
 
+extern "C" int64_t nf_hash_encode_bwd_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype) {
+  if (geom == nullptr || n_points < SCAN_MIN_POINTS) return 0;
+  return bwd_scan_workspace_bytes(n_points, geom, dout_dtype);
+}
+
 extern "C" int nf_hash_encode_bwd(const void* coords, int coords_dtype, int64_t csn, int64_t csd, const void* dout,
                                   int dout_dtype, int64_t dout_stride_n, float* dtable, int64_t n_points,
-                                  const nf_hash_geom* geom, const int64_t* primes, float scale, int flags,
-                                  void* stream) {
+                                  const nf_hash_geom* geom, const int64_t* primes, float scale, void* workspace,
+                                  int64_t workspace_bytes, int flags, void* stream) {
   DevGeom g;
   if (int rc = make_dev_geom(geom, &g)) return rc;
   NF_REQUIRE(dtype_ok(coords_dtype) && dtype_ok(dout_dtype), NF_EINVAL, "unknown dtype code");
@@ -489,6 +409,14 @@ extern "C" int nf_hash_encode_bwd(const void* coords, int coords_dtype, int64_t 
   NF_REQUIRE(n_points <= ((int64_t)1 << 31) * 256 - 1, NF_EINVAL, "n_points too large");
   hipStream_t s = (hipStream_t)stream;
 
+  // large batches: accumulate in LDS tiles (needs the caller's workspace for the bit-planes)
+  if (!(flags & (NF_HASH_FORCE_GENERIC | NF_HASH_FORCE_ATOMIC)) && n_points >= SCAN_MIN_POINTS && workspace != nullptr &&
+      ((uintptr_t)dout % 4 == 0) && (dout_stride_n % 2 == 0) && ((uintptr_t)workspace % 4 == 0)) {
+    const int64_t need = bwd_scan_workspace_bytes(n_points, geom, dout_dtype);
+    if (need > 0 && workspace_bytes >= need)
+      return launch_bwd_scan(coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, geom, g,
+                             primes, scale, workspace, s);
+  }
   if (!(flags & NF_HASH_FORCE_GENERIC) && tiled_ok(geom, dout_dtype, dout, dout_stride_n)) {
     constexpr int PPT = 2;
     constexpr int P = TILE_THREADS * PPT;

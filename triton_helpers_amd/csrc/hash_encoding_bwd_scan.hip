@@ -1,0 +1,335 @@
+// Hash-encoding backward without scattered global atomics (D = 3, F = 2, 16-bit upstream gradient).
+//
+// Measured on MI355X: a global float atomic costs one request slot per 64-byte segment at about
+// 21 G requests/s for the whole chip, whatever the table size or scope, so 2^20 points x 16 levels
+// x 8 corners x 2 features scattered one by one take ~13 ms.  LDS integer atomics and LDS
+// compare-and-swap are two orders of magnitude faster, so the gradient of every level is
+// accumulated in LDS instead:
+//
+//   * A level's gradient table is cut into tiles of TILE_ROWS rows (128 KiB of float2).  One
+//     workgroup owns one (level, tile, slice of the points), accumulates into its LDS tile with a
+//     64-bit compare-and-swap add (both features of a row at once), and finally adds the tile to
+//     the global table with coalesced atomics (16 floats per request).
+//   * A workgroup must only look at the points that touch its tile.  A first kernel (plan) writes,
+//     per (level, tile), one bit per point -- "some corner of this point falls into this tile" --
+//     so an owner reads N/8 bytes of bit-plane instead of all N points, expands the set bits into a
+//     per-wave queue of point indices and processes them 64 at a time with all lanes busy.
+//   * Levels that fit one tile need no bit-plane: every point hits.
+//
+// Arithmetic (cell, corner rows, weights) is the forward's, see hash_encoding.hip.
+#include "hash_common.h"
+
+namespace nf {
+
+constexpr int TILE_ROWS_LOG2 = 14;
+constexpr int TILE_ROWS = 1 << TILE_ROWS_LOG2;  // rows per LDS tile (float2 each: 128 KiB)
+constexpr int SCAN_THREADS = 1024;
+constexpr int SCAN_WAVES = SCAN_THREADS / 64;
+constexpr int QUEUE_CAP = 128;     // per-wave queue entries (< 64 pending + <= 64 appended per round)
+constexpr int PLAN_POINTS = 1024;  // points per plan workgroup == 32 bit-plane words
+constexpr int64_t HITS_PER_TASK = 65536;
+
+struct ScanPlan {
+  int n_levels;
+  int planes_pad;                 // planes rounded up to an odd number (LDS bank spread in the plan kernel)
+  int64_t words;                  // 32-bit words per bit-plane
+  int tiles[NF_MAX_LEVELS];       // tiles of the level
+  int plane0[NF_MAX_LEVELS];      // first bit-plane of the level, -1: single tile, no planes
+  int slices[NF_MAX_LEVELS];      // point slices per tile
+  int task0[NF_MAX_LEVELS + 1];   // first task of the level; task = task0[l] + tile * slices[l] + slice
+  int xfree[NF_MAX_LEVELS];       // hashed level whose tile id does not depend on the x corner (res + 1 <= TILE_ROWS)
+};
+
+struct Located {
+  uint32_t c[3];
+  float fr[3];
+};
+
+__device__ __forceinline__ Located locate3(const void* coords, int cdt, int64_t csn, int64_t csd, int64_t n, float scale,
+                                           float fres) {
+  Located r;
+#pragma unroll
+  for (int d = 0; d < 3; ++d) {
+    float v = load_as_f32(coords, n * csn + d * csd, cdt);
+    if (scale != 1.0f) v = v / scale;
+    const float pos = v * fres;
+    const float fl = floorf(pos);
+    r.c[d] = (uint32_t)(int)fl;
+    r.fr[d] = pos - fl;
+  }
+  return r;
+}
+
+// ---------------------------------------------------------------------------------------
+// Plan: one bit per (level, tile, point)
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(PLAN_POINTS) void hash_bwd_plan_k(const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                               uint32_t* planes, int64_t N, DevGeom g, ScanPlan sp,
+                                                               const int64_t* primes, float scale) {
+  extern __shared__ uint32_t bm[];  // [32 words][planes_pad]
+  const int tid = threadIdx.x;
+  const int P = sp.planes_pad;
+  for (int i = tid; i < 32 * P; i += PLAN_POINTS) bm[i] = 0u;
+  __syncthreads();
+  const int64_t n = (int64_t)blockIdx.x * PLAN_POINTS + tid;
+  if (n < N) {
+    const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], (uint32_t)primes[2]};
+    uint32_t* row = bm + (tid >> 5) * P;
+    const uint32_t bit = 1u << (tid & 31);
+    for (int l = 0; l < sp.n_levels; ++l) {
+      if (sp.plane0[l] < 0) continue;
+      const Located q = locate3(coords, cdt, csn, csd, n, scale, (float)g.res[l]);
+      uint32_t* lrow = row + sp.plane0[l];
+      if (l >= g.first_hash) {
+        const uint32_t mask = g.rows[l] - 1;
+        const uint32_t y0 = q.c[1] * pi[1], y1 = y0 + pi[1];
+        const uint32_t z0 = q.c[2] * pi[2], z1 = z0 + pi[2];
+        const uint32_t x0 = q.c[0] * pi[0], x1 = x0 + pi[0];
+        if (sp.xfree[l]) {
+          atomicOr(lrow + (((x0 ^ y0 ^ z0) & mask) >> TILE_ROWS_LOG2), bit);
+          atomicOr(lrow + (((x0 ^ y1 ^ z0) & mask) >> TILE_ROWS_LOG2), bit);
+          atomicOr(lrow + (((x0 ^ y0 ^ z1) & mask) >> TILE_ROWS_LOG2), bit);
+          atomicOr(lrow + (((x0 ^ y1 ^ z1) & mask) >> TILE_ROWS_LOG2), bit);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const uint32_t h = ((j & 1 ? x1 : x0) ^ (j & 2 ? y1 : y0) ^ (j & 4 ? z1 : z0)) & mask;
+            atomicOr(lrow + (h >> TILE_ROWS_LOG2), bit);
+          }
+        }
+      } else {
+        // dense: the 8 corner rows span [b, b + res^2 + res + 1]
+        const uint32_t res = (uint32_t)g.res[l], r2 = res * res;
+        const uint32_t b = q.c[0] + q.c[1] * res + q.c[2] * r2;
+        const uint32_t t_lo = b >> TILE_ROWS_LOG2, t_hi = (b + r2 + res + 1) >> TILE_ROWS_LOG2;
+        for (uint32_t t = t_lo; t <= t_hi && (int)t < sp.tiles[l]; ++t) atomicOr(lrow + t, bit);
+      }
+    }
+  }
+  __syncthreads();
+  // planes[plane][word]: every plane gets this workgroup's 32 consecutive words
+  int n_planes = 0;
+  for (int l = 0; l < sp.n_levels; ++l)
+    if (sp.plane0[l] >= 0) n_planes = sp.plane0[l] + sp.tiles[l];
+  for (int i = tid; i < n_planes * 32; i += PLAN_POINTS) {
+    const int plane = i >> 5, w = i & 31;
+    planes[(int64_t)plane * sp.words + (int64_t)blockIdx.x * 32 + w] = bm[w * P + plane];
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Scan: one workgroup per (level, tile, slice)
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ void lds_add2(float2* slot, float v0, float v1) {
+  unsigned long long* p = reinterpret_cast<unsigned long long*>(slot);
+  unsigned long long old = *p, assumed;
+  do {
+    assumed = old;
+    const float a = __uint_as_float((uint32_t)assumed) + v0;
+    const float b = __uint_as_float((uint32_t)(assumed >> 32)) + v1;
+    old = atomicCAS(p, assumed, (unsigned long long)__float_as_uint(a) | ((unsigned long long)__float_as_uint(b) << 32));
+  } while (old != assumed);
+}
+
+template <typename GT>
+__device__ __forceinline__ void scatter_point(float2* tile, uint32_t tile_id, int64_t n, int l, bool hashed, bool xfree,
+                                              const void* coords, int cdt, int64_t csn, int64_t csd, const uint16_t* dout,
+                                              int64_t dout_stride, const DevGeom& g, const uint32_t (&pi)[3], float scale) {
+  const uint32_t packed = *reinterpret_cast<const uint32_t*>(dout + n * dout_stride + 2 * l);
+  if ((packed & 0x7fff7fffu) == 0u) return;  // zero upstream gradient for both features
+  const float g0 = GT::to_f32((uint16_t)(packed & 0xffffu));
+  const float g1 = GT::to_f32((uint16_t)(packed >> 16));
+  const uint32_t res = (uint32_t)g.res[l];
+  const Located q = locate3(coords, cdt, csn, csd, n, scale, (float)g.res[l]);
+  float w[8];
+  weights_d3(q.fr, w);
+  const Corner8 r = rows_d3(q.c, hashed, res, g.rows[l] - 1, pi);
+  if (hashed && xfree) {
+    // both x corners of a (y, z) pair share the tile
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) {
+      if ((r.row[j] >> TILE_ROWS_LOG2) == tile_id) {
+        lds_add2(tile + (r.row[j] & (TILE_ROWS - 1)), w[j] * g0, w[j] * g1);
+        lds_add2(tile + (r.row[j + 1] & (TILE_ROWS - 1)), w[j + 1] * g0, w[j + 1] * g1);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if ((r.row[j] >> TILE_ROWS_LOG2) == tile_id) lds_add2(tile + (r.row[j] & (TILE_ROWS - 1)), w[j] * g0, w[j] * g1);
+  }
+}
+
+template <typename GT>
+__global__ __launch_bounds__(SCAN_THREADS) void hash_bwd_scan_k(const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                                const uint16_t* dout, int64_t dout_stride, float* dtable,
+                                                                const uint32_t* planes, int64_t N, DevGeom g, ScanPlan sp,
+                                                                const int64_t* primes, float scale) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  float2* tile = reinterpret_cast<float2*>(smem);
+  uint32_t* queues = reinterpret_cast<uint32_t*>(smem + (size_t)TILE_ROWS * sizeof(float2));
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  // ---- which (level, tile, slice) is this workgroup
+  int l = 0;
+  while (l + 1 < sp.n_levels && (int)blockIdx.x >= sp.task0[l + 1]) ++l;
+  const int local = (int)blockIdx.x - sp.task0[l];
+  const int n_slices = sp.slices[l];
+  const uint32_t tile_id = (uint32_t)(local / n_slices);
+  const int slice = local - (int)tile_id * n_slices;
+  const bool hashed = l >= g.first_hash;
+  const bool xfree = sp.xfree[l] != 0;
+  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], (uint32_t)primes[2]};
+
+  for (int i = tid; i < TILE_ROWS; i += SCAN_THREADS) tile[i] = make_float2(0.0f, 0.0f);
+  __syncthreads();
+
+  // ---- this slice's range of 32-point words
+  const int64_t w_begin = sp.words * slice / n_slices;
+  const int64_t w_end = sp.words * (slice + 1) / n_slices;
+  const uint32_t* plane = sp.plane0[l] >= 0 ? planes + (int64_t)(sp.plane0[l] + (int)tile_id) * sp.words : nullptr;
+  uint32_t* q = queues + wave * QUEUE_CAP;
+  int qn = 0;  // wave-uniform number of queued point indices
+
+  for (int64_t wb = w_begin + (int64_t)wave * 64; wb < w_end; wb += (int64_t)SCAN_WAVES * 64) {
+    const int64_t wi = wb + lane;
+    uint32_t word = 0u;
+    if (wi < w_end) {
+      if (plane != nullptr) {
+        word = plane[wi];
+      } else {
+        // single-tile level: every existing point hits
+        const int64_t left = N - wi * 32;
+        word = left >= 32 ? 0xffffffffu : (left > 0 ? ((1u << left) - 1u) : 0u);
+      }
+    }
+    // each round every lane with bits left queues the point of its lowest set bit
+    while (true) {
+      const bool has = word != 0u;
+      const unsigned long long vote = __ballot(has);
+      if (vote == 0ull) break;
+      if (has) {
+        const int b = __ffs((int)word) - 1;
+        word &= word - 1u;
+        const int pos = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(vote >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)vote, 0u));
+        q[qn + pos] = (uint32_t)(wi * 32 + b);
+      }
+      qn += __popcll(vote);
+      __builtin_amdgcn_wave_barrier();
+      if (qn >= 64) {
+        const int64_t n = (int64_t)q[qn - 64 + lane];
+        qn -= 64;
+        __builtin_amdgcn_wave_barrier();
+        scatter_point<GT>(tile, tile_id, n, l, hashed, xfree, coords, cdt, csn, csd, dout, dout_stride, g, pi, scale);
+      }
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+  if (lane < qn)
+    scatter_point<GT>(tile, tile_id, (int64_t)q[lane], l, hashed, xfree, coords, cdt, csn, csd, dout, dout_stride, g, pi, scale);
+  __syncthreads();
+
+  // ---- add the tile to the global table: consecutive lanes -> consecutive floats (16 per atomic request)
+  const int64_t row0 = (int64_t)tile_id * TILE_ROWS;
+  const int64_t rows_here = (int64_t)g.rows[l] - row0 < TILE_ROWS ? (int64_t)g.rows[l] - row0 : TILE_ROWS;
+  float* dst = dtable + (g.row_offset[l] + row0) * 2;
+  const float* src = reinterpret_cast<const float*>(tile);
+  for (int64_t i = tid; i < rows_here * 2; i += SCAN_THREADS) {
+    const float v = src[i];
+    if (v != 0.0f) unsafeAtomicAdd(dst + i, v);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------
+static bool scan_applicable(const nf_hash_geom* geom, int dout_dtype) {
+  if (geom->dims != 3 || geom->feat != 2 || dout_dtype == NF_F32) return false;
+  for (int l = 0; l < geom->levels; ++l) {
+    const int64_t r = geom->rows[l];
+    if (l >= geom->first_hash_level && (r & (r - 1)) != 0) return false;  // hashed levels: power-of-two sizes
+  }
+  return true;
+}
+
+static void make_plan(int64_t N, const nf_hash_geom* geom, ScanPlan* sp) {
+  sp->n_levels = geom->levels;
+  const int64_t plan_blocks = (N + PLAN_POINTS - 1) / PLAN_POINTS;
+  sp->words = plan_blocks * 32;
+  int planes = 0, task = 0;
+  for (int l = 0; l < geom->levels; ++l) {
+    const int tiles = (int)((geom->rows[l] + TILE_ROWS - 1) / TILE_ROWS);
+    sp->tiles[l] = tiles;
+    const bool hashed = l >= geom->first_hash_level;
+    sp->xfree[l] = hashed && (int64_t)geom->res[l] + 1 <= TILE_ROWS;
+    if (tiles > 1) {
+      sp->plane0[l] = planes;
+      planes += tiles;
+    } else {
+      sp->plane0[l] = -1;
+    }
+    // expected share of the points that touch one tile
+    double frac = 1.0;
+    if (tiles > 1) frac = hashed ? (sp->xfree[l] ? 4.0 : 8.0) / tiles : 1.5 / tiles;
+    if (frac > 1.0) frac = 1.0;
+    int64_t slices = (int64_t)((double)N * frac / (double)HITS_PER_TASK + 0.999);
+    if (slices < 1) slices = 1;
+    if (slices > 64) slices = 64;
+    sp->slices[l] = (int)slices;
+    sp->task0[l] = task;
+    task += tiles * (int)slices;
+  }
+  sp->task0[geom->levels] = task;
+  for (int l = geom->levels + 1; l <= NF_MAX_LEVELS; ++l) sp->task0[l] = task;
+  sp->planes_pad = planes | 1;
+}
+
+int64_t bwd_scan_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype) {
+  if (!scan_applicable(geom, dout_dtype) || n_points <= 0) return 0;
+  ScanPlan sp;
+  make_plan(n_points, geom, &sp);
+  int planes = 0;
+  for (int l = 0; l < geom->levels; ++l)
+    if (sp.plane0[l] >= 0) planes = sp.plane0[l] + sp.tiles[l];
+  // at least one word so that a geometry without planes still reports "applicable"
+  return (int64_t)(planes > 0 ? planes : 1) * sp.words * 4;
+}
+
+int launch_bwd_scan(const void* coords, int cdt, int64_t csn, int64_t csd, const void* dout, int ddt, int64_t dout_stride,
+                    float* dtable, int64_t N, const nf_hash_geom* geom, const DevGeom& g, const int64_t* primes, float scale,
+                    void* workspace, hipStream_t s) {
+  ScanPlan sp;
+  make_plan(N, geom, &sp);
+  int planes = 0;
+  for (int l = 0; l < geom->levels; ++l)
+    if (sp.plane0[l] >= 0) planes = sp.plane0[l] + sp.tiles[l];
+  if (planes > 0) {
+    const size_t lds = (size_t)32 * sp.planes_pad * 4;
+    NF_REQUIRE(lds <= 150 * 1024, NF_EUNSUPPORTED, "%d tiles need %zu B of LDS in the plan kernel", planes, lds);
+    if (lds > 64 * 1024) {
+      hipError_t e = hipFuncSetAttribute((const void*)hash_bwd_plan_k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    }
+    hipLaunchKernelGGL(hash_bwd_plan_k, dim3((unsigned)(sp.words / 32)), dim3(PLAN_POINTS), lds, s, coords, cdt, csn, csd,
+                       (uint32_t*)workspace, N, g, sp, primes, scale);
+    if (int rc = check_launch("hash_bwd_plan")) return rc;
+  }
+  const size_t lds = (size_t)TILE_ROWS * sizeof(float2) + (size_t)SCAN_WAVES * QUEUE_CAP * 4;
+  const int tasks = sp.task0[geom->levels];
+  if (ddt == NF_F16) {
+    auto kern = hash_bwd_scan_k<F16>;
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    hipLaunchKernelGGL(kern, dim3((unsigned)tasks), dim3(SCAN_THREADS), lds, s, coords, cdt, csn, csd, (const uint16_t*)dout,
+                       dout_stride, dtable, (const uint32_t*)workspace, N, g, sp, primes, scale);
+  } else {
+    auto kern = hash_bwd_scan_k<BF16>;
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    hipLaunchKernelGGL(kern, dim3((unsigned)tasks), dim3(SCAN_THREADS), lds, s, coords, cdt, csn, csd, (const uint16_t*)dout,
+                       dout_stride, dtable, (const uint32_t*)workspace, N, g, sp, primes, scale);
+  }
+  return check_launch("hash_bwd_scan");
+}
+
+}  // namespace nf

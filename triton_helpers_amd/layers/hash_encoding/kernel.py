@@ -44,7 +44,7 @@ PI_3: Final = 805_459_861
 DIVIDER_CONFIGS: Dict[Any, int] = {}
 BWD_DIVIDER_CONFIGS: Dict[Any, int] = {}
 
-_FLAGS = 0  # test hook: set to _lib.NF_HASH_FORCE_GENERIC to exercise the generic kernels
+_FLAGS = 0  # test hook: _lib.NF_HASH_FORCE_GENERIC / NF_HASH_FORCE_ATOMIC select the simpler kernels
 
 
 # ---------------------------------------------------------------------------
@@ -128,10 +128,13 @@ def _launch_backward(coords2d: Tensor, do2d: Tensor, de: Tensor, pi: Tensor, T: 
     F = de.shape[-1]
     geom = level_geometry(T, levels, D, F, min_res, max_res)
     lib = _lib.load()
+    # scratch for the LDS-tile backward (bit-planes); torch's caching allocator makes this free after the first call
+    ws_bytes = 0 if _FLAGS else lib.nf_hash_encode_bwd_workspace_bytes(N, geom, _lib.dtype_code(do2d.dtype))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=coords2d.device) if ws_bytes > 0 else None
     rc = lib.nf_hash_encode_bwd(
         coords2d.data_ptr(), _lib.dtype_code(coords2d.dtype), coords2d.stride(0), coords2d.stride(1),
         do2d.data_ptr(), _lib.dtype_code(do2d.dtype), do2d.stride(0), de.data_ptr(), N,
-        geom, pi.data_ptr(), float(scale), _FLAGS, _lib.current_stream(coords2d.device),
+        geom, pi.data_ptr(), float(scale), _lib.ptr(ws), ws_bytes, _FLAGS, _lib.current_stream(coords2d.device),
     )
     _lib.check(rc, "nf_hash_encode_bwd")
 
