@@ -27,7 +27,8 @@ constexpr int SCAN_THREADS = 1024;
 constexpr int SCAN_WAVES = SCAN_THREADS / 64;
 constexpr int QUEUE_CAP = 128;     // per-wave queue entries (< 64 pending + <= 64 appended per round)
 constexpr int PLAN_POINTS = 1024;  // points per plan workgroup == 32 bit-plane words
-constexpr int64_t HITS_PER_TASK = 65536;
+constexpr int64_t HITS_PER_TASK_HASHED = 65536;  // (point, corner pair) hits per workgroup, hashed levels
+constexpr int64_t HITS_PER_TASK_DENSE = 8192;    // points per workgroup where all 8 corners of a point land in the tile
 
 struct ScanPlan {
   int n_levels;
@@ -131,36 +132,126 @@ __device__ __forceinline__ void lds_add2(float2* slot, float v0, float v1) {
   } while (old != assumed);
 }
 
-template <typename GT>
-__device__ __forceinline__ void scatter_point(float2* tile, uint32_t tile_id, int64_t n, int l, bool hashed, bool xfree,
-                                              const void* coords, int cdt, int64_t csn, int64_t csd, const uint16_t* dout,
-                                              int64_t dout_stride, const DevGeom& g, const uint32_t (&pi)[3], float scale) {
-  const uint32_t packed = *reinterpret_cast<const uint32_t*>(dout + n * dout_stride + 2 * l);
-  if ((packed & 0x7fff7fffu) == 0u) return;  // zero upstream gradient for both features
-  const float g0 = GT::to_f32((uint16_t)(packed & 0xffffu));
-  const float g1 = GT::to_f32((uint16_t)(packed >> 16));
-  const uint32_t res = (uint32_t)g.res[l];
-  const Located q = locate3(coords, cdt, csn, csd, n, scale, (float)g.res[l]);
-  float w[8];
-  weights_d3(q.fr, w);
-  const Corner8 r = rows_d3(q.c, hashed, res, g.rows[l] - 1, pi);
-  if (hashed && xfree) {
-    // both x corners of a (y, z) pair share the tile
-#pragma unroll
-    for (int j = 0; j < 8; j += 2) {
-      if ((r.row[j] >> TILE_ROWS_LOG2) == tile_id) {
-        lds_add2(tile + (r.row[j] & (TILE_ROWS - 1)), w[j] * g0, w[j] * g1);
-        lds_add2(tile + (r.row[j + 1] & (TILE_ROWS - 1)), w[j + 1] * g0, w[j + 1] * g1);
-      }
-    }
+// What a lane needs of one queued point: raw coordinates and the level's packed upstream gradient.
+struct PointData {
+  float x[3];
+  uint32_t packed;
+};
+
+// FAST: float32 coordinates stored [N][3] contiguously, scale 1, and all element offsets below 2^31.
+template <bool FAST>
+__device__ __forceinline__ PointData fetch_point(uint32_t n, int l, const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                 const uint16_t* dout, int64_t dout_stride) {
+  PointData p;
+  if (FAST) {
+    const float* c = reinterpret_cast<const float*>(coords) + n * 3u;
+    p.x[0] = c[0];
+    p.x[1] = c[1];
+    p.x[2] = c[2];
+    p.packed = *reinterpret_cast<const uint32_t*>(dout + n * (uint32_t)dout_stride + 2u * (uint32_t)l);
   } else {
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
-      if ((r.row[j] >> TILE_ROWS_LOG2) == tile_id) lds_add2(tile + (r.row[j] & (TILE_ROWS - 1)), w[j] * g0, w[j] * g1);
+    for (int d = 0; d < 3; ++d) p.x[d] = load_as_f32(coords, (int64_t)n * csn + d * csd, cdt);
+    p.packed = *reinterpret_cast<const uint32_t*>(dout + (int64_t)n * dout_stride + 2 * l);
+  }
+  return p;
+}
+
+__device__ __forceinline__ unsigned long long add2_bits(unsigned long long old, float v0, float v1) {
+  const float a = __uint_as_float((uint32_t)old) + v0;
+  const float b = __uint_as_float((uint32_t)(old >> 32)) + v1;
+  return (unsigned long long)__float_as_uint(a) | ((unsigned long long)__float_as_uint(b) << 32);
+}
+
+// K independent float2 += (v0, v1) on LDS slots by 64-bit compare-and-swap, all K in flight at once.
+template <int K>
+__device__ __forceinline__ void lds_add2_multi(float2* tile, const uint32_t (&slot)[K], const bool (&on)[K], const float (&v0)[K],
+                                               const float (&v1)[K]) {
+  unsigned long long old[K];
+  bool todo[K];
+  bool any = false;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    todo[k] = on[k];
+    any = any || on[k];
+    if (on[k]) old[k] = *reinterpret_cast<unsigned long long*>(tile + slot[k]);
+  }
+  while (any) {
+    unsigned long long got[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+      if (todo[k]) got[k] = atomicCAS(reinterpret_cast<unsigned long long*>(tile + slot[k]), old[k], add2_bits(old[k], v0[k], v1[k]));
+    any = false;
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+      if (todo[k]) {
+        todo[k] = got[k] != old[k];
+        old[k] = got[k];
+        any = any || todo[k];
+      }
   }
 }
 
 template <typename GT>
+__device__ __forceinline__ void scatter_point(float2* tile, uint32_t tile_id, const PointData& p, int l, bool hashed, bool xfree,
+                                              const DevGeom& g, const uint32_t (&pi)[3], float scale) {
+  if ((p.packed & 0x7fff7fffu) == 0u) return;  // zero upstream gradient for both features
+  const float g0 = GT::to_f32((uint16_t)(p.packed & 0xffffu));
+  const float g1 = GT::to_f32((uint16_t)(p.packed >> 16));
+  const uint32_t res = (uint32_t)g.res[l];
+  const float fres = (float)g.res[l];
+  Located q;
+#pragma unroll
+  for (int d = 0; d < 3; ++d) {
+    const float v = scale != 1.0f ? p.x[d] / scale : p.x[d];
+    const float pos = v * fres;
+    const float fl = floorf(pos);
+    q.c[d] = (uint32_t)(int)fl;
+    q.fr[d] = pos - fl;
+  }
+  if (hashed && xfree) {
+    // The tile id of a corner does not depend on its x offset: test the four (y, z) pairs, then handle
+    // the matching pairs one per round (a lane usually has exactly one), the x pair of each in flight together.
+    const uint32_t mask = g.rows[l] - 1;
+    const uint32_t y0 = q.c[1] * pi[1], y1 = y0 + pi[1];
+    const uint32_t z0 = q.c[2] * pi[2], z1 = z0 + pi[2];
+    const uint32_t m0 = (y0 ^ z0) & mask, m1 = (y1 ^ z0) & mask, m2 = (y0 ^ z1) & mask, m3 = (y1 ^ z1) & mask;
+    uint32_t match = ((m0 >> TILE_ROWS_LOG2) == tile_id ? 1u : 0u) | ((m1 >> TILE_ROWS_LOG2) == tile_id ? 2u : 0u) |
+                     ((m2 >> TILE_ROWS_LOG2) == tile_id ? 4u : 0u) | ((m3 >> TILE_ROWS_LOG2) == tile_id ? 8u : 0u);
+    const float fx = q.fr[0], gx = 1.0f - fx;
+    const uint32_t x0 = q.c[0] * pi[0], x1 = x0 + pi[0];
+    while (match != 0u) {
+      const uint32_t j = (uint32_t)__ffs((int)match) - 1u;
+      match &= match - 1u;
+      const uint32_t m = j == 0u ? m0 : (j == 1u ? m1 : (j == 2u ? m2 : m3));
+      const float wy = (j & 1u) ? q.fr[1] : 1.0f - q.fr[1];
+      const float wz = (j & 2u) ? q.fr[2] : 1.0f - q.fr[2];
+      const float w0 = (gx * wy) * wz, w1 = (fx * wy) * wz;
+      const uint32_t slot[2] = {(x0 ^ m) & (TILE_ROWS - 1), (x1 ^ m) & (TILE_ROWS - 1)};
+      const bool on[2] = {true, true};
+      const float v0[2] = {w0 * g0, w1 * g0};
+      const float v1[2] = {w0 * g1, w1 * g1};
+      lds_add2_multi<2>(tile, slot, on, v0, v1);
+    }
+  } else {
+    float w[8];
+    weights_d3(q.fr, w);
+    const Corner8 r = rows_d3(q.c, hashed, res, g.rows[l] - 1, pi);
+    uint32_t slot[8];
+    bool on[8];
+    float v0[8], v1[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      on[j] = (r.row[j] >> TILE_ROWS_LOG2) == tile_id;
+      slot[j] = r.row[j] & (TILE_ROWS - 1);
+      v0[j] = w[j] * g0;
+      v1[j] = w[j] * g1;
+    }
+    lds_add2_multi<8>(tile, slot, on, v0, v1);
+  }
+}
+
+template <typename GT, bool FAST>
 __global__ __launch_bounds__(SCAN_THREADS) void hash_bwd_scan_k(const void* coords, int cdt, int64_t csn, int64_t csd,
                                                                 const uint16_t* dout, int64_t dout_stride, float* dtable,
                                                                 const uint32_t* planes, int64_t N, DevGeom g, ScanPlan sp,
@@ -181,7 +272,9 @@ __global__ __launch_bounds__(SCAN_THREADS) void hash_bwd_scan_k(const void* coor
   const bool xfree = sp.xfree[l] != 0;
   const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], (uint32_t)primes[2]};
 
-  for (int i = tid; i < TILE_ROWS; i += SCAN_THREADS) tile[i] = make_float2(0.0f, 0.0f);
+  const int64_t row0 = (int64_t)tile_id * TILE_ROWS;
+  const int rows_here = (int)((int64_t)g.rows[l] - row0 < TILE_ROWS ? (int64_t)g.rows[l] - row0 : TILE_ROWS);
+  for (int i = tid; i < rows_here; i += SCAN_THREADS) tile[i] = make_float2(0.0f, 0.0f);
   __syncthreads();
 
   // ---- this slice's range of 32-point words
@@ -190,6 +283,11 @@ __global__ __launch_bounds__(SCAN_THREADS) void hash_bwd_scan_k(const void* coor
   const uint32_t* plane = sp.plane0[l] >= 0 ? planes + (int64_t)(sp.plane0[l] + (int)tile_id) * sp.words : nullptr;
   uint32_t* q = queues + wave * QUEUE_CAP;
   int qn = 0;  // wave-uniform number of queued point indices
+  // One batch of 64 points is always in flight: its loads were issued when it left the queue and are
+  // consumed one drain later, so memory latency overlaps the bit expansion and the previous batch's adds.
+  PointData pend;
+  pend.x[0] = pend.x[1] = pend.x[2] = 0.0f;
+  pend.packed = 0u;  // a zero gradient makes the first (empty) batch a no-op
 
   for (int64_t wb = w_begin + (int64_t)wave * 64; wb < w_end; wb += (int64_t)SCAN_WAVES * 64) {
     const int64_t wi = wb + lane;
@@ -217,24 +315,27 @@ __global__ __launch_bounds__(SCAN_THREADS) void hash_bwd_scan_k(const void* coor
       qn += __popcll(vote);
       __builtin_amdgcn_wave_barrier();
       if (qn >= 64) {
-        const int64_t n = (int64_t)q[qn - 64 + lane];
+        const uint32_t n = q[qn - 64 + lane];
         qn -= 64;
         __builtin_amdgcn_wave_barrier();
-        scatter_point<GT>(tile, tile_id, n, l, hashed, xfree, coords, cdt, csn, csd, dout, dout_stride, g, pi, scale);
+        const PointData next = fetch_point<FAST>(n, l, coords, cdt, csn, csd, dout, dout_stride);
+        scatter_point<GT>(tile, tile_id, pend, l, hashed, xfree, g, pi, scale);
+        pend = next;
       }
     }
   }
   __builtin_amdgcn_wave_barrier();
-  if (lane < qn)
-    scatter_point<GT>(tile, tile_id, (int64_t)q[lane], l, hashed, xfree, coords, cdt, csn, csd, dout, dout_stride, g, pi, scale);
+  scatter_point<GT>(tile, tile_id, pend, l, hashed, xfree, g, pi, scale);
+  if (lane < qn) {
+    const PointData last = fetch_point<FAST>(q[lane], l, coords, cdt, csn, csd, dout, dout_stride);
+    scatter_point<GT>(tile, tile_id, last, l, hashed, xfree, g, pi, scale);
+  }
   __syncthreads();
 
   // ---- add the tile to the global table: consecutive lanes -> consecutive floats (16 per atomic request)
-  const int64_t row0 = (int64_t)tile_id * TILE_ROWS;
-  const int64_t rows_here = (int64_t)g.rows[l] - row0 < TILE_ROWS ? (int64_t)g.rows[l] - row0 : TILE_ROWS;
   float* dst = dtable + (g.row_offset[l] + row0) * 2;
   const float* src = reinterpret_cast<const float*>(tile);
-  for (int64_t i = tid; i < rows_here * 2; i += SCAN_THREADS) {
+  for (int i = tid; i < rows_here * 2; i += SCAN_THREADS) {
     const float v = src[i];
     if (v != 0.0f) unsafeAtomicAdd(dst + i, v);
   }
@@ -272,9 +373,10 @@ static void make_plan(int64_t N, const nf_hash_geom* geom, ScanPlan* sp) {
     double frac = 1.0;
     if (tiles > 1) frac = hashed ? (sp->xfree[l] ? 4.0 : 8.0) / tiles : 1.5 / tiles;
     if (frac > 1.0) frac = 1.0;
-    int64_t slices = (int64_t)((double)N * frac / (double)HITS_PER_TASK + 0.999);
+    const int64_t per_task = hashed && tiles > 1 ? HITS_PER_TASK_HASHED : HITS_PER_TASK_DENSE;
+    int64_t slices = (int64_t)((double)N * frac / (double)per_task + 0.999);
     if (slices < 1) slices = 1;
-    if (slices > 64) slices = 64;
+    if (slices > 256) slices = 256;
     sp->slices[l] = (int)slices;
     sp->task0[l] = task;
     task += tiles * (int)slices;
@@ -316,19 +418,21 @@ int launch_bwd_scan(const void* coords, int cdt, int64_t csn, int64_t csd, const
   }
   const size_t lds = (size_t)TILE_ROWS * sizeof(float2) + (size_t)SCAN_WAVES * QUEUE_CAP * 4;
   const int tasks = sp.task0[geom->levels];
-  if (ddt == NF_F16) {
-    auto kern = hash_bwd_scan_k<F16>;
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    hipLaunchKernelGGL(kern, dim3((unsigned)tasks), dim3(SCAN_THREADS), lds, s, coords, cdt, csn, csd, (const uint16_t*)dout,
-                       dout_stride, dtable, (const uint32_t*)workspace, N, g, sp, primes, scale);
-  } else {
-    auto kern = hash_bwd_scan_k<BF16>;
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    hipLaunchKernelGGL(kern, dim3((unsigned)tasks), dim3(SCAN_THREADS), lds, s, coords, cdt, csn, csd, (const uint16_t*)dout,
-                       dout_stride, dtable, (const uint32_t*)workspace, N, g, sp, primes, scale);
-  }
+  const bool fast = cdt == NF_F32 && csn == 3 && csd == 1 && scale == 1.0f && N * 3 < ((int64_t)1 << 31) &&
+                    N * dout_stride < ((int64_t)1 << 31);
+  const void* kern = nullptr;
+  if (ddt == NF_F16)
+    kern = fast ? (const void*)hash_bwd_scan_k<F16, true> : (const void*)hash_bwd_scan_k<F16, false>;
+  else
+    kern = fast ? (const void*)hash_bwd_scan_k<BF16, true> : (const void*)hash_bwd_scan_k<BF16, false>;
+  hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  const uint16_t* dout16 = (const uint16_t*)dout;
+  const uint32_t* planes_c = (const uint32_t*)workspace;
+  void* args[] = {(void*)&coords, (void*)&cdt, (void*)&csn, (void*)&csd, (void*)&dout16, (void*)&dout_stride, (void*)&dtable,
+                  (void*)&planes_c, (void*)&N, (void*)&g, (void*)&sp, (void*)&primes, (void*)&scale};
+  e = hipLaunchKernel(kern, dim3((unsigned)tasks), dim3(SCAN_THREADS), args, lds, s);
+  if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(hash_bwd_scan): %s", hipGetErrorString(e));
   return check_launch("hash_bwd_scan");
 }
 
