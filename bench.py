@@ -236,6 +236,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extras", action="store_true", help="skip the MLP / end-to-end workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one out-of-place add over 256 MiB (a copy kernel of known traffic, for scaling "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (points are independent, so the work "
@@ -289,6 +292,12 @@ def main():
             "configs[3]": bench_rev(max(3, s // 2), 2),
             "configs[4]": bench_e2e(max(3, s // 2), 2),
         }
+    if args.calibrate_copy:
+        a = torch.zeros(64 * 2**20, dtype=torch.float32, device="cuda")
+        b = torch.empty_like(a)
+        for _ in range(3):
+            torch.add(a, 1.0, out=b)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_hash()
     print(json.dumps(out))

@@ -1,0 +1,131 @@
+"""CPU-only checks: the C-ABI library loads and exports every symbol the header declares, the host-side
+geometry equals the oracle's, and the operators refuse to run without a GPU (no fallback path exists)."""
+import ctypes
+import json
+import os
+import re
+
+import pytest
+import torch
+
+from oracle import hash_encoding as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = json.load(open(os.path.join(ROOT, "tests", "golden", "hash_geometry.json")))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "nf_cdna4.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(nf_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from triton_helpers_amd import _lib
+
+    if not _lib.LIB_PATH.exists():
+        pytest.skip("libnf_cdna4.so not built (run python -m triton_helpers_amd.build)")
+    lib = ctypes.CDLL(str(_lib.LIB_PATH))
+    names = _declared_functions()
+    assert len(names) >= 10
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/nf_cdna4.h but not exported"
+    assert set(names) == set(_lib.EXPORTS), "ctypes binding and header disagree"
+    lib.nf_abi_version.restype = ctypes.c_int
+    assert lib.nf_abi_version() == _lib.NF_ABI_VERSION
+    header = open(os.path.join(ROOT, "include", "nf_cdna4.h")).read()
+    assert f"#define NF_ABI_VERSION {_lib.NF_ABI_VERSION}" in header
+
+
+def test_argument_validation_without_gpu():
+    """Entry points validate before touching the device: bad arguments come back as negative codes."""
+    from triton_helpers_amd import _lib
+
+    if not _lib.LIB_PATH.exists():
+        pytest.skip("libnf_cdna4.so not built")
+    lib = _lib.load()
+    geom = _lib.HashGeom()
+    geom.dims = 7
+    rc = lib.nf_hash_encode_fwd(None, 0, 3, 1, None, 0, None, 32, 10, geom, None, 1.0, 0, None)
+    assert rc == -1 and b"dims" in lib.nf_last_error()
+    rc = lib.nf_mlp_fwd(None, 32, None, 16, None, None, None, None, None, None, 8, 32, 24, 16, 2, 1, _lib.NF_BF16, None)
+    assert rc == -1 and b"d_hidden" in lib.nf_last_error()
+    rc = lib.nf_mlp_fwd(None, 32, None, 16, None, None, None, None, None, None, 8, 32, 64, 16, 2, 1, _lib.NF_F32, None)
+    assert rc == -2
+    rc = lib.nf_revmlp_fwd(None, 128, None, 128, None, None, None, None, 8, 65, 4, 4, _lib.NF_BF16, None)
+    assert rc == -1
+    with pytest.raises(RuntimeError):
+        _lib.check(rc, "nf_revmlp_fwd")
+    # zero rows is a no-op that needs no device
+    assert lib.nf_mlp_fwd(None, 32, None, 16, None, None, None, None, None, None, 0, 32, 64, 16, 2, 1, _lib.NF_BF16, None) == 0
+
+
+@pytest.mark.parametrize("name", ["bench", "default"])
+def test_host_geometry_matches_oracle_and_golden(name):
+    from triton_helpers_amd.layers.hash_encoding import helpers as H
+
+    g = GOLDEN[name]
+    T, L, D, lo, hi = g["T"], g["levels"], g["dims"], g["min_res"], g["max_res"]
+    assert H.compute_resolutions(L, lo, hi) == g["resolutions"] == O.level_resolutions(L, lo, hi)
+    assert H.compute_embedding_counts(L, T, D, lo, hi) == g["rows"]
+    assert H.get_first_hash_level(lo, hi, L, T, D) == g["first_hash_level"]
+    assert H.compute_b(lo, hi, L) == O.growth_factor(lo, hi, L)
+    offs = O.level_row_offsets(L, T, D, lo, hi)
+    for l in range(L):
+        assert H.compute_level_embedding_offset(l, L, T, D, lo, hi) == offs[l]
+    e = torch.zeros(g["total_rows"], 2)
+    assert H.seek_to_level_embeddings(e, 5, L, T, D, lo, hi).shape[0] == g["rows"][5]
+    geom = H.level_geometry(T, L, D, 2, lo, hi)
+    assert list(geom.res)[:L] == g["resolutions"] and list(geom.rows)[:L] == g["rows"]
+    assert list(geom.row_offset)[:L] == offs[:L] and geom.first_hash_level == g["first_hash_level"]
+    assert H.get_first_hash_level(2, 4, 2, 10**9, 2) == 3  # "no hashing" is reported as L + 1
+
+
+def test_cpu_helpers_with_reference_names_match_oracle():
+    """The ``_cpu_*`` utilities kept for API presence agree with the oracle (literal tables included)."""
+    from tests.test_oracle_hash import DENSE_ROWS, HASHED_ROWS, QUADRANT_X
+    from triton_helpers_amd.layers.hash_encoding import kernel as K
+
+    pi = torch.tensor([K.PI_1, K.PI_2, K.PI_3])
+    x = torch.tensor(QUADRANT_X, dtype=torch.float32)
+    assert K._cpu_embedding_lookup(x, pi[:2], 2, 9, 2).tolist() == DENSE_ROWS
+    assert K._cpu_embedding_lookup(x, pi[:2], 2, 7, 2).tolist() == HASHED_ROWS
+    g = GOLDEN["default"]
+    torch.manual_seed(0)
+    xs = torch.rand(50, 3)
+    table = torch.randn(g["total_rows"], 2)
+    out = K._cpu_hash_encoding(xs, table, pi, torch.zeros(50, 32), 3, 2, g["T"], 16, 16, 512)
+    torch.testing.assert_close(out, O.encode_forward(xs, table, None, g["T"], 16, 16, 512))
+
+
+def test_operators_refuse_cpu_tensors():
+    from triton_helpers_amd.layers.fully_fused_mlp import fully_fused_mlp
+    from triton_helpers_amd.layers.hash_encoding import hash_encoding
+    from triton_helpers_amd.layers.reversible_mlp import reversible_mlp
+
+    g = GOLDEN["default"]
+    with pytest.raises(AssertionError):
+        hash_encoding(torch.rand(4, 3), torch.zeros(g["total_rows"], 2), max_entries_per_level=g["T"])
+    h = torch.zeros
+    with pytest.raises(AssertionError):
+        fully_fused_mlp(h(1, 4, 8).half(), h(16, 8).half(), None, h(4, 16).half(), None)
+    with pytest.raises(AssertionError):
+        reversible_mlp(h(4, 128).half(), h(128, 64).half(), None, h(128, 64).half(), None)
+
+
+def test_drop_in_alias_package():
+    import triton_helpers.layers.fully_fused_mlp as a
+    import triton_helpers.layers.hash_encoding as b
+    from triton_helpers.layers.hash_encoding.kernel import PI_2, _cpu_hash_encoding, compute_resolutions  # noqa: F401
+
+    assert PI_2 == 2_654_435_761
+    assert {"fully_fused_mlp", "FullyFusedMLP", "feedforward"} <= set(a.__all__)
+    assert {"hash_encoding", "HashEncoding"} <= set(b.__all__)
+
+
+def test_bench_rejects_more_than_one_gpu():
+    import subprocess
+    import sys
+
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in r.stderr

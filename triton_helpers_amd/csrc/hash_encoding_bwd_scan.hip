@@ -37,7 +37,15 @@ struct ScanPlan {
   int tiles[NF_MAX_LEVELS];       // tiles of the level
   int plane0[NF_MAX_LEVELS];      // first bit-plane of the level, -1: single tile, no planes
   int slices[NF_MAX_LEVELS];      // point slices per tile
-  int task0[NF_MAX_LEVELS + 1];   // first task of the level; task = task0[l] + tile * slices[l] + slice
+  // Tasks are ordered slice-major so that the workgroups running at the same time walk the same part of the
+  // point array (their coordinate / gradient reads then meet in L2).  Levels have different slice counts, so the
+  // order is cut into segments: within segment k every slice index s in [seg_s0[k], seg_s0[k+1]) contributes one
+  // task per tile of every level with slices[l] > s, levels in ascending order.
+  int n_segs;
+  int seg_s0[NF_MAX_LEVELS + 2];    // first slice index of the segment
+  int seg_task0[NF_MAX_LEVELS + 2]; // first task of the segment
+  int seg_width[NF_MAX_LEVELS + 1]; // tasks per slice index inside the segment
+  int n_tasks;
   int xfree[NF_MAX_LEVELS];       // hashed level whose tile id does not depend on the x corner (res + 1 <= TILE_ROWS)
 };
 
@@ -65,7 +73,8 @@ __device__ __forceinline__ Located locate3(const void* coords, int cdt, int64_t 
 // Plan: one bit per (level, tile, point)
 // ---------------------------------------------------------------------------------------
 __global__ __launch_bounds__(PLAN_POINTS) void hash_bwd_plan_k(const void* coords, int cdt, int64_t csn, int64_t csd,
-                                                               uint32_t* planes, int64_t N, DevGeom g, ScanPlan sp,
+                                                               const uint16_t* dout, int64_t dout_stride, uint32_t* planes,
+                                                               uint32_t* gT, int64_t N, DevGeom g, ScanPlan sp,
                                                                const int64_t* primes, float scale) {
   extern __shared__ uint32_t bm[];  // [32 words][planes_pad]
   const int tid = threadIdx.x;
@@ -78,7 +87,10 @@ __global__ __launch_bounds__(PLAN_POINTS) void hash_bwd_plan_k(const void* coord
     uint32_t* row = bm + (tid >> 5) * P;
     const uint32_t bit = 1u << (tid & 31);
     for (int l = 0; l < sp.n_levels; ++l) {
-      if (sp.plane0[l] < 0) continue;
+      // the level's packed upstream gradient, transposed to gT[level][point] for the scan's reads
+      const uint32_t packed = *reinterpret_cast<const uint32_t*>(dout + n * dout_stride + 2 * l);
+      gT[(int64_t)l * sp.words * 32 + n] = packed;
+      if (sp.plane0[l] < 0 || (packed & 0x7fff7fffu) == 0u) continue;  // no planes, or nothing to scatter
       const Located q = locate3(coords, cdt, csn, csd, n, scale, (float)g.res[l]);
       uint32_t* lrow = row + sp.plane0[l];
       if (l >= g.first_hash) {
@@ -138,22 +150,22 @@ struct PointData {
   uint32_t packed;
 };
 
-// FAST: float32 coordinates stored [N][3] contiguously, scale 1, and all element offsets below 2^31.
+// FAST: float32 coordinates stored [N][3] contiguously, scale 1, 3*N below 2^31.
+// gl: this level's row of the transposed gradient (one dword per point).
 template <bool FAST>
-__device__ __forceinline__ PointData fetch_point(uint32_t n, int l, const void* coords, int cdt, int64_t csn, int64_t csd,
-                                                 const uint16_t* dout, int64_t dout_stride) {
+__device__ __forceinline__ PointData fetch_point(uint32_t n, const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                 const uint32_t* gl) {
   PointData p;
   if (FAST) {
     const float* c = reinterpret_cast<const float*>(coords) + n * 3u;
     p.x[0] = c[0];
     p.x[1] = c[1];
     p.x[2] = c[2];
-    p.packed = *reinterpret_cast<const uint32_t*>(dout + n * (uint32_t)dout_stride + 2u * (uint32_t)l);
   } else {
 #pragma unroll
     for (int d = 0; d < 3; ++d) p.x[d] = load_as_f32(coords, (int64_t)n * csn + d * csd, cdt);
-    p.packed = *reinterpret_cast<const uint32_t*>(dout + (int64_t)n * dout_stride + 2 * l);
   }
+  p.packed = gl[n];
   return p;
 }
 
@@ -253,21 +265,29 @@ __device__ __forceinline__ void scatter_point(float2* tile, uint32_t tile_id, co
 
 template <typename GT, bool FAST>
 __global__ __launch_bounds__(SCAN_THREADS) void hash_bwd_scan_k(const void* coords, int cdt, int64_t csn, int64_t csd,
-                                                                const uint16_t* dout, int64_t dout_stride, float* dtable,
-                                                                const uint32_t* planes, int64_t N, DevGeom g, ScanPlan sp,
-                                                                const int64_t* primes, float scale) {
+                                                                const uint32_t* gT, float* dtable, const uint32_t* planes,
+                                                                int64_t N, DevGeom g, ScanPlan sp, const int64_t* primes,
+                                                                float scale) {
   extern __shared__ __align__(16) unsigned char smem[];
   float2* tile = reinterpret_cast<float2*>(smem);
   uint32_t* queues = reinterpret_cast<uint32_t*>(smem + (size_t)TILE_ROWS * sizeof(float2));
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
   // ---- which (level, tile, slice) is this workgroup
+  int seg = 0;
+  while (seg + 1 < sp.n_segs && (int)blockIdx.x >= sp.seg_task0[seg + 1]) ++seg;
+  const int in_seg = (int)blockIdx.x - sp.seg_task0[seg];
+  const int slice = sp.seg_s0[seg] + in_seg / sp.seg_width[seg];
+  int rest = in_seg % sp.seg_width[seg];
   int l = 0;
-  while (l + 1 < sp.n_levels && (int)blockIdx.x >= sp.task0[l + 1]) ++l;
-  const int local = (int)blockIdx.x - sp.task0[l];
+  for (; l < sp.n_levels; ++l) {
+    if (sp.slices[l] <= slice) continue;
+    if (rest < sp.tiles[l]) break;
+    rest -= sp.tiles[l];
+  }
   const int n_slices = sp.slices[l];
-  const uint32_t tile_id = (uint32_t)(local / n_slices);
-  const int slice = local - (int)tile_id * n_slices;
+  const uint32_t tile_id = (uint32_t)rest;
+  const uint32_t* gl = gT + (int64_t)l * sp.words * 32;
   const bool hashed = l >= g.first_hash;
   const bool xfree = sp.xfree[l] != 0;
   const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], (uint32_t)primes[2]};
@@ -318,7 +338,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void hash_bwd_scan_k(const void* coor
         const uint32_t n = q[qn - 64 + lane];
         qn -= 64;
         __builtin_amdgcn_wave_barrier();
-        const PointData next = fetch_point<FAST>(n, l, coords, cdt, csn, csd, dout, dout_stride);
+        const PointData next = fetch_point<FAST>(n, coords, cdt, csn, csd, gl);
         scatter_point<GT>(tile, tile_id, pend, l, hashed, xfree, g, pi, scale);
         pend = next;
       }
@@ -327,7 +347,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void hash_bwd_scan_k(const void* coor
   __builtin_amdgcn_wave_barrier();
   scatter_point<GT>(tile, tile_id, pend, l, hashed, xfree, g, pi, scale);
   if (lane < qn) {
-    const PointData last = fetch_point<FAST>(q[lane], l, coords, cdt, csn, csd, dout, dout_stride);
+    const PointData last = fetch_point<FAST>(q[lane], coords, cdt, csn, csd, gl);
     scatter_point<GT>(tile, tile_id, last, l, hashed, xfree, g, pi, scale);
   }
   __syncthreads();
@@ -378,11 +398,37 @@ static void make_plan(int64_t N, const nf_hash_geom* geom, ScanPlan* sp) {
     if (slices < 1) slices = 1;
     if (slices > 256) slices = 256;
     sp->slices[l] = (int)slices;
-    sp->task0[l] = task;
-    task += tiles * (int)slices;
   }
-  sp->task0[geom->levels] = task;
-  for (int l = geom->levels + 1; l <= NF_MAX_LEVELS; ++l) sp->task0[l] = task;
+  // segments between consecutive distinct slice counts
+  int bounds[NF_MAX_LEVELS + 1];
+  int nb = 0;
+  for (int l = 0; l < geom->levels; ++l) {
+    bool seen = false;
+    for (int i = 0; i < nb; ++i) seen = seen || bounds[i] == sp->slices[l];
+    if (!seen) bounds[nb++] = sp->slices[l];
+  }
+  for (int i = 0; i < nb; ++i)
+    for (int j = i + 1; j < nb; ++j)
+      if (bounds[j] < bounds[i]) {
+        const int t = bounds[i];
+        bounds[i] = bounds[j];
+        bounds[j] = t;
+      }
+  int s0 = 0;
+  sp->n_segs = nb;
+  for (int k = 0; k < nb; ++k) {
+    int width = 0;
+    for (int l = 0; l < geom->levels; ++l)
+      if (sp->slices[l] > s0) width += sp->tiles[l];
+    sp->seg_s0[k] = s0;
+    sp->seg_task0[k] = task;
+    sp->seg_width[k] = width;
+    task += width * (bounds[k] - s0);
+    s0 = bounds[k];
+  }
+  sp->seg_s0[nb] = s0;
+  sp->seg_task0[nb] = task;
+  sp->n_tasks = task;
   sp->planes_pad = planes | 1;
 }
 
@@ -393,8 +439,8 @@ int64_t bwd_scan_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int
   int planes = 0;
   for (int l = 0; l < geom->levels; ++l)
     if (sp.plane0[l] >= 0) planes = sp.plane0[l] + sp.tiles[l];
-  // at least one word so that a geometry without planes still reports "applicable"
-  return (int64_t)(planes > 0 ? planes : 1) * sp.words * 4;
+  // bit-planes, then the transposed gradient gT[level][point]
+  return ((int64_t)planes + (int64_t)geom->levels * 32) * sp.words * 4;
 }
 
 int launch_bwd_scan(const void* coords, int cdt, int64_t csn, int64_t csd, const void* dout, int ddt, int64_t dout_stride,
@@ -405,7 +451,9 @@ int launch_bwd_scan(const void* coords, int cdt, int64_t csn, int64_t csd, const
   int planes = 0;
   for (int l = 0; l < geom->levels; ++l)
     if (sp.plane0[l] >= 0) planes = sp.plane0[l] + sp.tiles[l];
-  if (planes > 0) {
+  uint32_t* planes_w = (uint32_t*)workspace;
+  uint32_t* gT = planes_w + (int64_t)planes * sp.words;
+  {
     const size_t lds = (size_t)32 * sp.planes_pad * 4;
     NF_REQUIRE(lds <= 150 * 1024, NF_EUNSUPPORTED, "%d tiles need %zu B of LDS in the plan kernel", planes, lds);
     if (lds > 64 * 1024) {
@@ -413,13 +461,12 @@ int launch_bwd_scan(const void* coords, int cdt, int64_t csn, int64_t csd, const
       if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     }
     hipLaunchKernelGGL(hash_bwd_plan_k, dim3((unsigned)(sp.words / 32)), dim3(PLAN_POINTS), lds, s, coords, cdt, csn, csd,
-                       (uint32_t*)workspace, N, g, sp, primes, scale);
+                       (const uint16_t*)dout, dout_stride, planes_w, gT, N, g, sp, primes, scale);
     if (int rc = check_launch("hash_bwd_plan")) return rc;
   }
   const size_t lds = (size_t)TILE_ROWS * sizeof(float2) + (size_t)SCAN_WAVES * QUEUE_CAP * 4;
-  const int tasks = sp.task0[geom->levels];
-  const bool fast = cdt == NF_F32 && csn == 3 && csd == 1 && scale == 1.0f && N * 3 < ((int64_t)1 << 31) &&
-                    N * dout_stride < ((int64_t)1 << 31);
+  const int tasks = sp.n_tasks;
+  const bool fast = cdt == NF_F32 && csn == 3 && csd == 1 && scale == 1.0f && N * 3 < ((int64_t)1 << 31);
   const void* kern = nullptr;
   if (ddt == NF_F16)
     kern = fast ? (const void*)hash_bwd_scan_k<F16, true> : (const void*)hash_bwd_scan_k<F16, false>;
@@ -427,9 +474,9 @@ int launch_bwd_scan(const void* coords, int cdt, int64_t csn, int64_t csd, const
     kern = fast ? (const void*)hash_bwd_scan_k<BF16, true> : (const void*)hash_bwd_scan_k<BF16, false>;
   hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-  const uint16_t* dout16 = (const uint16_t*)dout;
-  const uint32_t* planes_c = (const uint32_t*)workspace;
-  void* args[] = {(void*)&coords, (void*)&cdt, (void*)&csn, (void*)&csd, (void*)&dout16, (void*)&dout_stride, (void*)&dtable,
+  const uint32_t* planes_c = planes_w;
+  const uint32_t* gT_c = gT;
+  void* args[] = {(void*)&coords, (void*)&cdt, (void*)&csn, (void*)&csd, (void*)&gT_c, (void*)&dtable,
                   (void*)&planes_c, (void*)&N, (void*)&g, (void*)&sp, (void*)&primes, (void*)&scale};
   e = hipLaunchKernel(kern, dim3((unsigned)tasks), dim3(SCAN_THREADS), args, lds, s);
   if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(hash_bwd_scan): %s", hipGetErrorString(e));
