@@ -86,9 +86,29 @@ __global__ __launch_bounds__(PLAN_POINTS) void hash_bwd_plan_k(const void* coord
     const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], (uint32_t)primes[2]};
     uint32_t* row = bm + (tid >> 5) * P;
     const uint32_t bit = 1u << (tid & 31);
+    // this point's gradient row, read once (up to 16 levels live in registers)
+    const uint32_t* grow = reinterpret_cast<const uint32_t*>(dout + n * dout_stride);
+    uint32_t gr[16];
+    const bool row_vec = sp.n_levels <= 16 && (sp.n_levels & 3) == 0 && ((uintptr_t)grow & 15u) == 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (row_vec && 4 * i < sp.n_levels) v = reinterpret_cast<const uint4*>(grow)[i];
+      gr[4 * i] = v.x;
+      gr[4 * i + 1] = v.y;
+      gr[4 * i + 2] = v.z;
+      gr[4 * i + 3] = v.w;
+    }
     for (int l = 0; l < sp.n_levels; ++l) {
       // the level's packed upstream gradient, transposed to gT[level][point] for the scan's reads
-      const uint32_t packed = *reinterpret_cast<const uint32_t*>(dout + n * dout_stride + 2 * l);
+      uint32_t packed;
+      if (row_vec) {
+        packed = gr[0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) packed = (l == i) ? gr[i] : packed;
+      } else {
+        packed = grow[l];
+      }
       gT[(int64_t)l * sp.words * 32 + n] = packed;
       if (sp.plane0[l] < 0 || (packed & 0x7fff7fffu) == 0u) continue;  // no planes, or nothing to scatter
       const Located q = locate3(coords, cdt, csn, csd, n, scale, (float)g.res[l]);
