@@ -34,6 +34,9 @@ COMMON_FLAGS = [
 ]
 # Files whose float arithmetic must not be contracted into FMAs (bit-exact cell / weight math).
 NO_CONTRACT = {"hash_encoding.hip", "hash_encoding_bwd_scan.hip"}
+# Files whose MFMA results feed vector ALU work directly: keep them in architectural VGPRs instead of
+# bouncing every result through an accumulation register.
+MFMA_VGPR_FORM = {"fused_mlp_bwd2.hip"}
 
 
 def _hipcc() -> str:
@@ -69,6 +72,8 @@ def build(verbose: bool = True, jobs: int = 4) -> Path:
         flags = list(COMMON_FLAGS)
         if src.name in NO_CONTRACT:
             flags.append("-ffp-contract=off")
+        if src.name in MFMA_VGPR_FORM:
+            flags += ["-mllvm", "-amdgpu-mfma-vgpr-form"]
         cmds.append([hipcc, *flags, "-c", str(src), "-o", str(obj)])
         objs.append(obj)
     with ThreadPoolExecutor(max_workers=jobs) as ex:

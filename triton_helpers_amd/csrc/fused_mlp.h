@@ -1,0 +1,107 @@
+// Declarations shared by the fused-MLP translation units.
+#pragma once
+
+#include "mlp_tile.h"
+
+namespace nf {
+
+struct MlpArgs {
+  const uint16_t* x;
+  int64_t x_stride;
+  uint16_t* y;
+  int64_t y_stride;
+  const uint16_t* dy;
+  int64_t dy_stride;
+  uint16_t* dx;
+  int64_t dx_stride;
+  const uint16_t *w_in, *b_in, *w_hid, *b_hid, *w_out, *b_out;
+  float *dw_in, *db_in, *dw_hid, *db_hid, *dw_out, *db_out;
+  int64_t rows;
+  int d_in, d_hidden, d_out, depth, act;
+  int x_vec, y_vec, dy_vec, dx_vec;
+  int waves;  // waves per workgroup
+};
+
+constexpr int FRAG_ELEMS = 64 * 8;  // 16-bit elements per fragment (1 KiB)
+constexpr int TPITCH = 40;          // 16-bit elements per feature row of a transposed 32-row panel (80 B)
+
+template <typename T>
+__device__ __forceinline__ void stage_bias(float* dst, const uint16_t* b, int n_valid, int n_pad, int tid, int nthreads) {
+  for (int i = tid; i < n_pad; i += nthreads) dst[i] = (b != nullptr && i < n_valid) ? T::to_f32(b[i]) : 0.0f;
+}
+
+// acc[nt][mt] = bias + W(frags) * in[nt][kc]
+template <typename T, int MT, int KC>
+__device__ __forceinline__ void layer_mma(f32x4_t (&acc)[2][4], const Frag (&in)[2][2], const uint16_t* frags,
+                                          const float* bias, int lane) {
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(bias + 16 * mt + 4 * (lane >> 4));
+    acc[0][mt] = b4;
+    acc[1][mt] = b4;
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc) {
+      const Frag a = lds_frag(frags, mt * KC + kc, lane);
+      acc[0][mt] = mfma16<T>(a, in[0][kc], acc[0][mt]);
+      acc[1][mt] = mfma16<T>(a, in[1][kc], acc[1][mt]);
+    }
+  }
+}
+
+// Park an accumulator-layout tile (lane (n,g): features 16*mt + 4*g + r of row 16*nt + n) into a
+// transposed panel panel[feature][row].
+__device__ __forceinline__ void park_tile_T(uint16_t* panel, int mt, int nt, int lane, uint32_t p01, uint32_t p23) {
+  const int n = (lane & 15) + 16 * nt;
+  const int f = 16 * mt + 4 * (lane >> 4);
+  panel[(f + 0) * TPITCH + n] = (uint16_t)(p01 & 0xffffu);
+  panel[(f + 1) * TPITCH + n] = (uint16_t)(p01 >> 16);
+  panel[(f + 2) * TPITCH + n] = (uint16_t)(p23 & 0xffffu);
+  panel[(f + 3) * TPITCH + n] = (uint16_t)(p23 >> 16);
+}
+// Park a natural-order fragment (lane (n,g): features 32*kc + 8*g + j of row 16*nt + n).
+__device__ __forceinline__ void park_frag_T(uint16_t* panel, int kc, int nt, int lane, const Frag& f) {
+  const int n = (lane & 15) + 16 * nt;
+  const int c = 32 * kc + 8 * (lane >> 4);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    panel[(c + 2 * j) * TPITCH + n] = (uint16_t)(f.w[j] & 0xffffu);
+    panel[(c + 2 * j + 1) * TPITCH + n] = (uint16_t)(f.w[j] >> 16);
+  }
+}
+// Operand of a K = 32-rows product: lane (i, g) reads rows 8*g .. 8*g+7 of feature 16*t + i.
+__device__ __forceinline__ Frag panel_frag(const uint16_t* panel, int t, int lane) {
+  Frag f;
+  f.u = *reinterpret_cast<const uint4*>(panel + (16 * t + (lane & 15)) * TPITCH + 8 * (lane >> 4));
+  return f;
+}
+
+// dW tile (mt over output features, nt over input features): lane (n, g) reg r is
+// dW[16*mt + 4*g + r][16*nt + n].
+__device__ __forceinline__ void flush_dw_tile(float* dw, int out_dim, int in_dim, int mt, int nt, int lane, f32x4_t v) {
+  const int c = 16 * nt + (lane & 15);
+  const int r0 = 16 * mt + 4 * (lane >> 4);
+  if (c >= in_dim) return;
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+    if (r0 + r < out_dim) unsafeAtomicAdd(dw + (size_t)(r0 + r) * in_dim + c, v[r]);
+}
+
+inline int device_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) cus = p.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+constexpr size_t LDS_LIMIT = 160 * 1024;
+
+
+// Specialised backward for exactly one hidden layer (fused_mlp_bwd2.hip), bias gradients included.
+// *handled = false: shape not covered, nothing was launched.
+int launch_mlp_bwd2(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
+
+}  // namespace nf

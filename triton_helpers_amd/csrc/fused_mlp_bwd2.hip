@@ -1,0 +1,454 @@
+// Fused-MLP backward specialised for one hidden layer (in -> H -> H -> out): the shape of neural-field
+// decoders and of the benchmark (32 -> 64 -> 64 -> 16).
+//
+// Same algorithm as mlp_bwd_k (fused_mlp.hip) with everything static and no per-chunk LDS traffic:
+//   * the two hidden activations stay in registers as the next layer's B fragments; for ReLU they are the
+//     gates as well;
+//   * the products that contract over rows (dW = dz^T h) need both operands with the rows along K; the
+//     row-per-lane fragments are transposed by a matrix-core product with a 0/1 selector (transpose_tile),
+//     which is exact and costs one MFMA per 16x16 tile;
+//   * all three weight gradients live in float32 accumulators for the wave's whole row loop; bias gradients
+//     are two-element dot products of the transposed dz fragments with ones;
+//   * LDS only holds the weight fragments, so two workgroups fit a CU and hide each other's MFMA latency.
+#include "fused_mlp.h"
+
+namespace nf {
+
+// Bias gradient of feature 16*mt + n: the four lane groups hold partial sums over disjoint rows.
+__device__ __forceinline__ void flush_db(float* db, int dim, int mt, int lane, float v) {
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 32);
+  const int f = 16 * mt + lane;
+  if (db != nullptr && lane < 16 && f < dim) unsafeAtomicAdd(db + f, v);
+}
+
+typedef short s16x2_t __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+
+// ReLU on a packed pair of 16-bit floats: as signed integers, negative floats (sign bit set, -0 included)
+// are below zero and non-negative floats are unchanged, so one v_pk_max_i16 does both halves.
+__device__ __forceinline__ uint32_t relu_pk(uint32_t p) {
+  const s16x2_t z = {0, 0};
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(s16x2_t, p), z));
+}
+// dz = (h != 0) ? dh : 0 on packed pairs, h being a ReLU output (non-negative, never -0):
+// min(h, 1) as unsigned halves is the 0/1 gate, an integer multiply applies it.  The min goes through an
+// asm statement so that the optimiser does not turn the pair of packed ops back into per-half selects;
+// its result only feeds the multiply, which the compiler emits (and tracks for hazards) itself.
+__device__ __forceinline__ uint32_t relu_gate_pk(uint32_t dh, uint32_t h) {
+  uint32_t m;
+  asm("v_pk_min_u16 %0, %1, 1 op_sel_hi:[1,0]" : "=v"(m) : "v"(h));
+  return __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2_t, dh) * __builtin_bit_cast(u16x2_t, m));
+}
+
+template <typename T>
+__device__ __forceinline__ float dot2_ones(uint32_t p, float acc);
+template <>
+__device__ __forceinline__ float dot2_ones<BF16>(uint32_t p, float acc) {
+  const bf16x2_t one = {(__bf16)1.0f, (__bf16)1.0f};
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, p), one, acc, false);
+}
+template <>
+__device__ __forceinline__ float dot2_ones<F16>(uint32_t p, float acc) {
+  const f16x2_t one = {(_Float16)1.0f, (_Float16)1.0f};
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, p), one, acc, false);
+}
+
+// B fragment in chain order straight from global memory: lane (n, g) gets features
+// 32*kc + 4*g .. +3 and 32*kc + 16 + 4*g .. +3 of row row0 + n; zero beyond `rows` / `width`.
+__device__ __forceinline__ Frag load_rows_frag_chain(const uint16_t* base, int64_t stride, int64_t row0, int64_t rows,
+                                                     int width, int kc, int lane, bool vec_ok) {
+  Frag f;
+  f.u = make_uint4(0u, 0u, 0u, 0u);
+  const int64_t r = row0 + (lane & 15);
+  if (r >= rows) return f;
+  const int c0 = 32 * kc + 4 * (lane >> 4);
+  const uint16_t* p = base + r * stride + c0;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int c = c0 + 16 * h;
+    if (vec_ok && c + 4 <= width) {
+      const uint2 v = *reinterpret_cast<const uint2*>(p + 16 * h);
+      f.w[2 * h] = v.x;
+      f.w[2 * h + 1] = v.y;
+    } else if (c < width) {
+      uint16_t t[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) t[j] = (c + j < width) ? p[16 * h + j] : (uint16_t)0;
+      f.w[2 * h] = (uint32_t)t[0] | ((uint32_t)t[1] << 16);
+      f.w[2 * h + 1] = (uint32_t)t[2] | ((uint32_t)t[3] << 16);
+    }
+  }
+  return f;
+}
+
+// Transpose through the matrix core.  f0 / f1 are chain-order fragments of rows 0-15 / 16-31 of a chunk
+// (lane (row, g): 8 features of K-chunk kc); e selects 16 of those 32 features (sel_frag()).  The product
+// F * E has exactly one non-zero term per output, so it is exact; the result, packed back to 16 bit, is the
+// operand of a product that contracts over the chunk's 32 rows: lane (feature, g) holds rows 4g .. 4g+3 and
+// 16+4g .. 16+4g+3 of that feature.  Both operands of such a product use the same row order.
+template <typename T>
+__device__ __forceinline__ Frag transpose_tile(const Frag& f0, const Frag& f1, const Frag& e) {
+  const f32x4_t z = {0.0f, 0.0f, 0.0f, 0.0f};
+  const f32x4_t a = mfma16<T>(f0, e, z);
+  const f32x4_t b = mfma16<T>(f1, e, z);
+  Frag o;
+  o.w[0] = pack2<T>(a[0], a[1]);
+  o.w[1] = pack2<T>(a[2], a[3]);
+  o.w[2] = pack2<T>(b[0], b[1]);
+  o.w[3] = pack2<T>(b[2], b[3]);
+  return o;
+}
+// Selector of features 16*half .. 16*half+15 of a chain-order K-chunk: B[k][n] = 1 where slot k holds feature
+// 16*half + n, i.e. lane (n, g) with g == n / 4 carries a 1.0 in element 4*half + n % 4.
+template <typename T>
+__device__ __forceinline__ Frag sel_frag(int half, int lane) {
+  const int n = lane & 15, g = lane >> 4;
+  const uint32_t one = (pack2<T>(1.0f, 1.0f) & 0xffffu) << (16 * (n & 1));
+  const uint32_t v = (g == (n >> 2)) ? one : 0u;
+  const int d = 2 * half + ((n & 3) >> 1);
+  Frag e;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) e.w[i] = (i == d) ? v : 0u;
+  return e;
+}
+
+// Workgroups per CU the ReLU kernel is compiled for.
+#ifndef NF_BWD2_OCC
+#define NF_BWD2_OCC 1
+#endif
+template <typename T, int KIN, int HP, int OUTP, bool RELU>
+__global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArgs a) {
+  constexpr int KC_IN = KIN / 32, KC_H = HP / 32, MT_H = HP / 16, MT_I = KIN / 16, MT_O = OUTP / 16;
+  constexpr int KC_O = (OUTP + 31) / 32;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int lane = tid & 63, wave = tid >> 6;
+
+  uint16_t* f_in = reinterpret_cast<uint16_t*>(smem);          // W_in    [MT_H][KC_IN]
+  uint16_t* f_hid = f_in + MT_H * KC_IN * FRAG_ELEMS;          // W_hid   [MT_H][KC_H]
+  uint16_t* t_in = f_hid + MT_H * KC_H * FRAG_ELEMS;           // W_in^T  [MT_I][KC_H]
+  uint16_t* t_hid = t_in + MT_I * KC_H * FRAG_ELEMS;           // W_hid^T [MT_H][KC_H]
+  uint16_t* t_out = t_hid + MT_H * KC_H * FRAG_ELEMS;          // W_out^T [MT_H][KC_O]
+  float* bias_in = reinterpret_cast<float*>(t_out + MT_H * KC_O * FRAG_ELEMS);
+  float* bias_hid = bias_in + HP;
+
+  stage_weight_frags<true, false>(f_in, a.w_in, a.d_hidden, a.d_in, MT_H, KC_IN, tid, nthreads);
+  stage_weight_frags<true, false>(f_hid, a.w_hid, a.d_hidden, a.d_hidden, MT_H, KC_H, tid, nthreads);
+  stage_weight_frags<true, true>(t_in, a.w_in, a.d_hidden, a.d_in, MT_I, KC_H, tid, nthreads);
+  stage_weight_frags<true, true>(t_hid, a.w_hid, a.d_hidden, a.d_hidden, MT_H, KC_H, tid, nthreads);
+  stage_weight_frags<true, true>(t_out, a.w_out, a.d_out, a.d_hidden, MT_H, KC_O, tid, nthreads);
+  stage_bias<T>(bias_in, a.b_in, a.d_hidden, HP, tid, nthreads);
+  stage_bias<T>(bias_hid, a.b_hid, a.d_hidden, HP, tid, nthreads);
+  __syncthreads();
+
+  f32x4_t dw_in[MT_H][MT_I], dw_hid[MT_H][MT_H], dw_out[MT_O][MT_H];
+  float db_in[MT_H], db_hid[MT_H], db_out[MT_O];  // lane (feature, g): partial row sums of feature 16*tile + n
+  const f32x4_t zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int i = 0; i < MT_H; ++i) {
+#pragma unroll
+    for (int j = 0; j < MT_I; ++j) dw_in[i][j] = zero4;
+#pragma unroll
+    for (int j = 0; j < MT_H; ++j) dw_hid[i][j] = zero4;
+    db_in[i] = 0.0f;
+    db_hid[i] = 0.0f;
+  }
+#pragma unroll
+  for (int i = 0; i < MT_O; ++i) {
+#pragma unroll
+    for (int j = 0; j < MT_H; ++j) dw_out[i][j] = zero4;
+    db_out[i] = 0.0f;
+  }
+  const Frag sel[2] = {sel_frag<T>(0, lane), sel_frag<T>(1, lane)};
+
+  const int64_t n_chunks = (a.rows + 31) / 32;
+  const int64_t wave_stride = (int64_t)gridDim.x * 4;
+  const int64_t first_chunk = (int64_t)blockIdx.x * 4 + wave;
+  Frag nx[2][KC_IN], ndy[2][KC_O];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+    for (int kc = 0; kc < KC_IN; ++kc)
+      nx[nt][kc] = load_rows_frag_chain(a.x, a.x_stride, first_chunk * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+#pragma unroll
+    for (int kc = 0; kc < KC_O; ++kc)
+      ndy[nt][kc] = load_rows_frag_chain(a.dy, a.dy_stride, first_chunk * 32 + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
+  }
+
+  for (int64_t chunk = first_chunk; chunk < n_chunks; chunk += wave_stride) {
+    const int64_t row0 = chunk * 32;
+    Frag in[2][2], h1[2][2], h2[2][2], g1[2][2], g2[2][2], dz[2][2];
+    f32x4_t acc[2][4];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+      for (int kc = 0; kc < KC_IN; ++kc) {
+        in[nt][kc] = nx[nt][kc];
+        nx[nt][kc] = load_rows_frag_chain(a.x, a.x_stride, (chunk + wave_stride) * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+      }
+#pragma unroll
+      for (int kc = 0; kc < KC_O; ++kc) {
+        dz[nt][kc] = ndy[nt][kc];
+        ndy[nt][kc] = load_rows_frag_chain(a.dy, a.dy_stride, (chunk + wave_stride) * 32 + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
+      }
+    }
+
+    // ---- forward recompute: h1 = act(W_in x + b), h2 = act(W_hid h1 + b) ----
+    layer_mma<T, MT_H, KC_IN>(acc, in, f_in, bias_in, lane);
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT_H; ++mt) {
+        uint32_t p01, p23;
+        if (RELU) {
+          p01 = relu_pk(pack2<T>(acc[nt][mt][0], acc[nt][mt][1]));
+          p23 = relu_pk(pack2<T>(acc[nt][mt][2], acc[nt][mt][3]));
+        } else {
+          uint32_t q01, q23;
+          act_pack<T, false>(acc[nt][mt], a.act, p01, p23);
+          gate_pack<T, false>(acc[nt][mt], a.act, p01, p23, q01, q23);
+          g1[nt][mt >> 1].w[2 * (mt & 1)] = q01;
+          g1[nt][mt >> 1].w[2 * (mt & 1) + 1] = q23;
+        }
+        h1[nt][mt >> 1].w[2 * (mt & 1)] = p01;
+        h1[nt][mt >> 1].w[2 * (mt & 1) + 1] = p23;
+      }
+    layer_mma<T, MT_H, KC_H>(acc, h1, f_hid, bias_hid, lane);
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT_H; ++mt) {
+        uint32_t p01, p23;
+        if (RELU) {
+          p01 = relu_pk(pack2<T>(acc[nt][mt][0], acc[nt][mt][1]));
+          p23 = relu_pk(pack2<T>(acc[nt][mt][2], acc[nt][mt][3]));
+        } else {
+          uint32_t q01, q23;
+          act_pack<T, false>(acc[nt][mt], a.act, p01, p23);
+          gate_pack<T, false>(acc[nt][mt], a.act, p01, p23, q01, q23);
+          g2[nt][mt >> 1].w[2 * (mt & 1)] = q01;
+          g2[nt][mt >> 1].w[2 * (mt & 1) + 1] = q23;
+        }
+        h2[nt][mt >> 1].w[2 * (mt & 1)] = p01;
+        h2[nt][mt >> 1].w[2 * (mt & 1) + 1] = p23;
+      }
+
+    // ---- output layer: dW_out += dy^T h2, db_out += sum dy ; dh2 = W_out^T dy ----
+    {
+      Frag hb[MT_H];
+#pragma unroll
+      for (int j = 0; j < MT_H; ++j) hb[j] = transpose_tile<T>(h2[0][j >> 1], h2[1][j >> 1], sel[j & 1]);
+#pragma unroll
+      for (int i = 0; i < MT_O; ++i) {
+        const Frag da = transpose_tile<T>(dz[0][i >> 1], dz[1][i >> 1], sel[i & 1]);
+#pragma unroll
+        for (int j = 0; j < MT_H; ++j) dw_out[i][j] = mfma16<T>(da, hb[j], dw_out[i][j]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) db_out[i] = dot2_ones<T>(da.w[q], db_out[i]);
+      }
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT_H; ++mt) {
+      acc[0][mt] = zero4;
+      acc[1][mt] = zero4;
+#pragma unroll
+      for (int kc = 0; kc < KC_O; ++kc) {
+        const Frag wa = lds_frag(t_out, mt * KC_O + kc, lane);
+        acc[0][mt] = mfma16<T>(wa, dz[0][kc], acc[0][mt]);
+        acc[1][mt] = mfma16<T>(wa, dz[1][kc], acc[1][mt]);
+      }
+    }
+    // ---- hidden layer: dz2 = dh2 * act'(z2) ; dW_hid += dz2^T h1 ; dh1 = W_hid^T dz2 ----
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT_H; ++mt) {
+        uint32_t p01, p23;
+        if (RELU) {
+          p01 = relu_gate_pk(pack2<T>(acc[nt][mt][0], acc[nt][mt][1]), h2[nt][mt >> 1].w[2 * (mt & 1)]);
+          p23 = relu_gate_pk(pack2<T>(acc[nt][mt][2], acc[nt][mt][3]), h2[nt][mt >> 1].w[2 * (mt & 1) + 1]);
+        } else {
+          gate_apply<T, false>(acc[nt][mt], g2[nt][mt >> 1].w[2 * (mt & 1)], g2[nt][mt >> 1].w[2 * (mt & 1) + 1], p01, p23);
+        }
+        dz[nt][mt >> 1].w[2 * (mt & 1)] = p01;
+        dz[nt][mt >> 1].w[2 * (mt & 1) + 1] = p23;
+      }
+    {
+      Frag hb[MT_H];
+#pragma unroll
+      for (int j = 0; j < MT_H; ++j) hb[j] = transpose_tile<T>(h1[0][j >> 1], h1[1][j >> 1], sel[j & 1]);
+#pragma unroll
+      for (int i = 0; i < MT_H; ++i) {
+        const Frag da = transpose_tile<T>(dz[0][i >> 1], dz[1][i >> 1], sel[i & 1]);
+#pragma unroll
+        for (int j = 0; j < MT_H; ++j) dw_hid[i][j] = mfma16<T>(da, hb[j], dw_hid[i][j]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) db_hid[i] = dot2_ones<T>(da.w[q], db_hid[i]);
+      }
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT_H; ++mt) {
+      f32x4_t o0 = zero4, o1 = zero4;
+#pragma unroll
+      for (int kc = 0; kc < KC_H; ++kc) {
+        const Frag wa = lds_frag(t_hid, mt * KC_H + kc, lane);
+        o0 = mfma16<T>(wa, dz[0][kc], o0);
+        o1 = mfma16<T>(wa, dz[1][kc], o1);
+      }
+      acc[0][mt] = o0;
+      acc[1][mt] = o1;
+    }
+    // ---- input layer: dz1 = dh1 * act'(z1) ; dW_in += dz1^T x ; dx = W_in^T dz1 ----
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT_H; ++mt) {
+        uint32_t p01, p23;
+        if (RELU) {
+          p01 = relu_gate_pk(pack2<T>(acc[nt][mt][0], acc[nt][mt][1]), h1[nt][mt >> 1].w[2 * (mt & 1)]);
+          p23 = relu_gate_pk(pack2<T>(acc[nt][mt][2], acc[nt][mt][3]), h1[nt][mt >> 1].w[2 * (mt & 1) + 1]);
+        } else {
+          gate_apply<T, false>(acc[nt][mt], g1[nt][mt >> 1].w[2 * (mt & 1)], g1[nt][mt >> 1].w[2 * (mt & 1) + 1], p01, p23);
+        }
+        dz[nt][mt >> 1].w[2 * (mt & 1)] = p01;
+        dz[nt][mt >> 1].w[2 * (mt & 1) + 1] = p23;
+      }
+    {
+      Frag xb[MT_I];
+#pragma unroll
+      for (int j = 0; j < MT_I; ++j) xb[j] = transpose_tile<T>(in[0][j >> 1], in[1][j >> 1], sel[j & 1]);
+#pragma unroll
+      for (int i = 0; i < MT_H; ++i) {
+        const Frag da = transpose_tile<T>(dz[0][i >> 1], dz[1][i >> 1], sel[i & 1]);
+#pragma unroll
+        for (int j = 0; j < MT_I; ++j) dw_in[i][j] = mfma16<T>(da, xb[j], dw_in[i][j]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) db_in[i] = dot2_ones<T>(da.w[q], db_in[i]);
+      }
+    }
+    if (a.dx != nullptr) {
+#pragma unroll
+      for (int mt = 0; mt < MT_I; ++mt) {
+        f32x4_t o0 = zero4, o1 = zero4;
+#pragma unroll
+        for (int kc = 0; kc < KC_H; ++kc) {
+          const Frag wa = lds_frag(t_in, mt * KC_H + kc, lane);
+          o0 = mfma16<T>(wa, dz[0][kc], o0);
+          o1 = mfma16<T>(wa, dz[1][kc], o1);
+        }
+        store_rows_tile<T>(a.dx, a.dx_stride, row0, a.rows, a.d_in, mt, lane, o0, a.dx_vec);
+        store_rows_tile<T>(a.dx, a.dx_stride, row0 + 16, a.rows, a.d_in, mt, lane, o1, a.dx_vec);
+      }
+    }
+  }
+
+  // ---- reduce the gradients over the four waves through LDS (the weight fragments are dead by now), then
+  // one pass of atomics per workgroup ----
+  __syncthreads();
+  f32x4_t* red = reinterpret_cast<f32x4_t*>(smem) + lane;
+  float* redb = reinterpret_cast<float*>(smem) + (size_t)(MT_H * (MT_I + MT_H) + MT_O * MT_H) * 256 + lane;
+  for (int w = 1; w < 4; ++w) {
+    if (wave == w) {
+      int t = 0, u = 0;
+#pragma unroll
+      for (int i = 0; i < MT_H; ++i) {
+#pragma unroll
+        for (int j = 0; j < MT_I; ++j) red[64 * (t++)] = dw_in[i][j];
+#pragma unroll
+        for (int j = 0; j < MT_H; ++j) red[64 * (t++)] = dw_hid[i][j];
+        redb[64 * (u++)] = db_in[i];
+        redb[64 * (u++)] = db_hid[i];
+      }
+#pragma unroll
+      for (int i = 0; i < MT_O; ++i) {
+#pragma unroll
+        for (int j = 0; j < MT_H; ++j) red[64 * (t++)] = dw_out[i][j];
+        redb[64 * (u++)] = db_out[i];
+      }
+    }
+    __syncthreads();
+    if (wave == 0) {
+      int t = 0, u = 0;
+#pragma unroll
+      for (int i = 0; i < MT_H; ++i) {
+#pragma unroll
+        for (int j = 0; j < MT_I; ++j) dw_in[i][j] += red[64 * (t++)];
+#pragma unroll
+        for (int j = 0; j < MT_H; ++j) dw_hid[i][j] += red[64 * (t++)];
+        db_in[i] += redb[64 * (u++)];
+        db_hid[i] += redb[64 * (u++)];
+      }
+#pragma unroll
+      for (int i = 0; i < MT_O; ++i) {
+#pragma unroll
+        for (int j = 0; j < MT_H; ++j) dw_out[i][j] += red[64 * (t++)];
+        db_out[i] += redb[64 * (u++)];
+      }
+    }
+    __syncthreads();
+  }
+  if (wave != 0) return;
+#pragma unroll
+  for (int i = 0; i < MT_H; ++i) {
+#pragma unroll
+    for (int j = 0; j < MT_I; ++j) flush_dw_tile(a.dw_in, a.d_hidden, a.d_in, i, j, lane, dw_in[i][j]);
+#pragma unroll
+    for (int j = 0; j < MT_H; ++j) flush_dw_tile(a.dw_hid, a.d_hidden, a.d_hidden, i, j, lane, dw_hid[i][j]);
+    flush_db(a.db_in, a.d_hidden, i, lane, db_in[i]);
+    flush_db(a.db_hid, a.d_hidden, i, lane, db_hid[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < MT_O; ++i) {
+#pragma unroll
+    for (int j = 0; j < MT_H; ++j) flush_dw_tile(a.dw_out, a.d_out, a.d_hidden, i, j, lane, dw_out[i][j]);
+    flush_db(a.db_out, a.d_out, i, lane, db_out[i]);
+  }
+}
+
+template <typename T, int KIN, int HP, int OUTP>
+static int launch2(const MlpArgs& a0, hipStream_t s) {
+  MlpArgs a = a0;
+  constexpr int KC_O = (OUTP + 31) / 32;
+  constexpr int MT_H = HP / 16, MT_I = KIN / 16, MT_O = OUTP / 16;
+  constexpr size_t W_BYTES = ((size_t)MT_H * (KIN / 32) + (size_t)MT_I * (HP / 32) + 2 * (size_t)MT_H * (HP / 32) + (size_t)MT_H * KC_O) * 1024 +
+                             (size_t)2 * HP * 4;
+  constexpr size_t RED = (size_t)(MT_H * (MT_I + MT_H) + MT_O * MT_H) * 1024 + (size_t)(2 * MT_H + MT_O) * 256;
+  constexpr size_t LDS = W_BYTES > RED ? W_BYTES : RED;
+  static_assert(LDS <= 64 * 1024, "LDS budget");
+  a.waves = 4;
+  // chain-order loads move 8 bytes at a time
+  a.x_vec = ((uintptr_t)a.x % 8 == 0) && (a.x_stride % 4 == 0);
+  a.dy_vec = ((uintptr_t)a.dy % 8 == 0) && (a.dy_stride % 4 == 0);
+  const int64_t chunks = (a.rows + 31) / 32;
+  int64_t blocks = (chunks + 3) / 4;
+  const int64_t cap = (int64_t)device_cus() * (a.act == NF_ACT_RELU ? NF_BWD2_OCC : 1);
+  if (blocks > cap) blocks = cap;
+  const void* kern = a.act == NF_ACT_RELU ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false>;
+  void* args[] = {(void*)&a};
+  const hipError_t e = hipLaunchKernel(kern, dim3((unsigned)blocks), dim3(256), args, LDS, s);
+  if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(mlp_bwd2): %s", hipGetErrorString(e));
+  return check_launch("mlp_bwd2");
+}
+
+template <typename T>
+static int dispatch2(const MlpArgs& a, hipStream_t s, bool* handled) {
+  *handled = true;
+  const int kin = (a.d_in + 31) / 32 * 32, outp = a.d_out <= 16 ? 16 : 64;
+  if (a.d_hidden > 32) {
+    if (kin == 32 && outp == 16) return launch2<T, 32, 64, 16>(a, s);
+    if (kin == 32) return launch2<T, 32, 64, 64>(a, s);
+    if (outp == 16) return launch2<T, 64, 64, 16>(a, s);
+    return launch2<T, 64, 64, 64>(a, s);
+  }
+  *handled = false;  // narrow hidden layers stay on the general kernel
+  return 0;
+}
+
+int launch_mlp_bwd2(const MlpArgs& a, int dtype, hipStream_t s, bool* handled) {
+  *handled = false;
+  if (a.depth != 2) return 0;
+  return dtype == NF_BF16 ? dispatch2<BF16>(a, s, handled) : dispatch2<F16>(a, s, handled);
+}
+
+}  // namespace nf
