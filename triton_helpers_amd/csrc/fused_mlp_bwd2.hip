@@ -82,6 +82,44 @@ __device__ __forceinline__ Frag load_rows_frag_chain(const uint16_t* base, int64
   return f;
 }
 
+// Same fragment for the aligned case (8-byte aligned rows, width a multiple of 4): no branches, addresses of
+// lanes past the end of the batch or of the row are clamped in range and their data replaced by zero.
+__device__ __forceinline__ Frag load_rows_frag_chain_fast(const uint16_t* base, int64_t stride, int64_t row0, int64_t rows,
+                                                          int width, int kc, int lane) {
+  const int64_t r = row0 + (lane & 15);
+  const int c0 = 32 * kc + 4 * (lane >> 4);
+  const bool row_ok = r < rows;
+  const bool lo_ok = row_ok && c0 < width, hi_ok = row_ok && c0 + 16 < width;
+  const uint16_t* p = base + (row_ok ? r : 0) * stride;
+  const uint2 lo = *reinterpret_cast<const uint2*>(p + (lo_ok ? c0 : 0));
+  const uint2 hi = *reinterpret_cast<const uint2*>(p + (hi_ok ? c0 + 16 : 0));
+  Frag f;
+  f.w[0] = lo_ok ? lo.x : 0u;
+  f.w[1] = lo_ok ? lo.y : 0u;
+  f.w[2] = hi_ok ? hi.x : 0u;
+  f.w[3] = hi_ok ? hi.y : 0u;
+  return f;
+}
+
+// Store of an accumulator tile for the aligned case (width a multiple of 4, 8-byte aligned rows).
+template <typename T>
+__device__ __forceinline__ void store_rows_tile_fast(uint16_t* base, int64_t stride, int64_t row0, int64_t rows, int width,
+                                                     int mt, int lane, f32x4_t v) {
+  const int64_t r = row0 + (lane & 15);
+  const int c0 = 16 * mt + 4 * (lane >> 4);
+  uint2 o;
+  o.x = pack2<T>(v[0], v[1]);
+  o.y = pack2<T>(v[2], v[3]);
+  if (r < rows && c0 < width) *reinterpret_cast<uint2*>(base + r * stride + c0) = o;
+}
+
+template <bool FAST>
+__device__ __forceinline__ Frag load_chain(const uint16_t* base, int64_t stride, int64_t row0, int64_t rows, int width,
+                                           int kc, int lane, bool vec_ok) {
+  if (FAST) return load_rows_frag_chain_fast(base, stride, row0, rows, width, kc, lane);
+  return load_rows_frag_chain(base, stride, row0, rows, width, kc, lane, vec_ok);
+}
+
 // Transpose through the matrix core.  f0 / f1 are chain-order fragments of rows 0-15 / 16-31 of a chunk
 // (lane (row, g): 8 features of K-chunk kc); e selects 16 of those 32 features (sel_frag()).  The product
 // F * E has exactly one non-zero term per output, so it is exact; the result, packed back to 16 bit, is the
@@ -117,7 +155,7 @@ __device__ __forceinline__ Frag sel_frag(int half, int lane) {
 #ifndef NF_BWD2_OCC
 #define NF_BWD2_OCC 1
 #endif
-template <typename T, int KIN, int HP, int OUTP, bool RELU>
+template <typename T, int KIN, int HP, int OUTP, bool RELU, bool FAST>
 __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArgs a) {
   constexpr int KC_IN = KIN / 32, KC_H = HP / 32, MT_H = HP / 16, MT_I = KIN / 16, MT_O = OUTP / 16;
   constexpr int KC_O = (OUTP + 31) / 32;
@@ -170,10 +208,10 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
   for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
     for (int kc = 0; kc < KC_IN; ++kc)
-      nx[nt][kc] = load_rows_frag_chain(a.x, a.x_stride, first_chunk * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+      nx[nt][kc] = load_chain<FAST>(a.x, a.x_stride, first_chunk * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
 #pragma unroll
     for (int kc = 0; kc < KC_O; ++kc)
-      ndy[nt][kc] = load_rows_frag_chain(a.dy, a.dy_stride, first_chunk * 32 + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
+      ndy[nt][kc] = load_chain<FAST>(a.dy, a.dy_stride, first_chunk * 32 + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
   }
 
   for (int64_t chunk = first_chunk; chunk < n_chunks; chunk += wave_stride) {
@@ -185,12 +223,12 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
 #pragma unroll
       for (int kc = 0; kc < KC_IN; ++kc) {
         in[nt][kc] = nx[nt][kc];
-        nx[nt][kc] = load_rows_frag_chain(a.x, a.x_stride, (chunk + wave_stride) * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+        nx[nt][kc] = load_chain<FAST>(a.x, a.x_stride, (chunk + wave_stride) * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
       }
 #pragma unroll
       for (int kc = 0; kc < KC_O; ++kc) {
         dz[nt][kc] = ndy[nt][kc];
-        ndy[nt][kc] = load_rows_frag_chain(a.dy, a.dy_stride, (chunk + wave_stride) * 32 + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
+        ndy[nt][kc] = load_chain<FAST>(a.dy, a.dy_stride, (chunk + wave_stride) * 32 + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
       }
     }
 
@@ -337,8 +375,13 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
           o0 = mfma16<T>(wa, dz[0][kc], o0);
           o1 = mfma16<T>(wa, dz[1][kc], o1);
         }
-        store_rows_tile<T>(a.dx, a.dx_stride, row0, a.rows, a.d_in, mt, lane, o0, a.dx_vec);
-        store_rows_tile<T>(a.dx, a.dx_stride, row0 + 16, a.rows, a.d_in, mt, lane, o1, a.dx_vec);
+        if (FAST) {
+          store_rows_tile_fast<T>(a.dx, a.dx_stride, row0, a.rows, a.d_in, mt, lane, o0);
+          store_rows_tile_fast<T>(a.dx, a.dx_stride, row0 + 16, a.rows, a.d_in, mt, lane, o1);
+        } else {
+          store_rows_tile<T>(a.dx, a.dx_stride, row0, a.rows, a.d_in, mt, lane, o0, a.dx_vec);
+          store_rows_tile<T>(a.dx, a.dx_stride, row0 + 16, a.rows, a.d_in, mt, lane, o1, a.dx_vec);
+        }
       }
     }
   }
@@ -424,7 +467,13 @@ static int launch2(const MlpArgs& a0, hipStream_t s) {
   int64_t blocks = (chunks + 3) / 4;
   const int64_t cap = (int64_t)device_cus() * (a.act == NF_ACT_RELU ? NF_BWD2_OCC : 1);
   if (blocks > cap) blocks = cap;
-  const void* kern = a.act == NF_ACT_RELU ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false>;
+  const bool fast = a.x_vec && a.dy_vec && a.d_in % 4 == 0 && a.d_out % 4 == 0 &&
+                    (a.dx == nullptr || ((uintptr_t)a.dx % 8 == 0 && a.dx_stride % 4 == 0));
+  const void* kern;
+  if (a.act == NF_ACT_RELU)
+    kern = fast ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, true> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, false>;
+  else
+    kern = fast ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false, true> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false, false>;
   void* args[] = {(void*)&a};
   const hipError_t e = hipLaunchKernel(kern, dim3((unsigned)blocks), dim3(256), args, LDS, s);
   if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(mlp_bwd2): %s", hipGetErrorString(e));
