@@ -66,7 +66,8 @@ typedef struct nf_hash_geom {
 /* flags for the hash-encoding entry points */
 enum {
   NF_HASH_FORCE_GENERIC = 1,   /* use the one-thread-per-(point,level) kernel even where a faster kernel applies */
-  NF_HASH_FORCE_ATOMIC = 2     /* backward: scatter with global atomics even where the LDS-tile kernels apply */
+  NF_HASH_FORCE_ATOMIC = 2,    /* backward: scatter with global atomics even where the LDS-tile kernels apply */
+  NF_HASH_FORCE_PLANES = 4     /* backward: of the two LDS-tile variants take the bit-plane one (smaller workspace) */
 };
 
 int nf_abi_version(void);
@@ -84,7 +85,8 @@ int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t coords_stri
 /* dtable[row_offset[l] + row_j, f] += w_j * dout[n, l*F + f]   (float32 accumulators,
  * NOT cleared by the call).  dout rows of dout_dtype with row stride dout_stride_n.
  * workspace: optional device scratch of at least nf_hash_encode_bwd_workspace_bytes() bytes (4-byte
- * aligned); with it, large batches accumulate in LDS tiles instead of scattering global atomics.
+ * aligned, 16-byte for the fastest variant); with it, large batches accumulate in LDS tiles instead of scattering
+ * global atomics.
  * NULL / too small selects the atomic kernels.  Its contents are undefined afterwards. */
 int nf_hash_encode_bwd(const void* coords, int coords_dtype, int64_t coords_stride_n, int64_t coords_stride_d,
                        const void* dout, int dout_dtype, int64_t dout_stride_n, float* dtable, int64_t n_points,

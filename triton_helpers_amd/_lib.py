@@ -21,6 +21,7 @@ NF_MAX_LEVELS = 32
 NF_MAX_DIMS = 4
 NF_HASH_FORCE_GENERIC = 1
 NF_HASH_FORCE_ATOMIC = 2
+NF_HASH_FORCE_PLANES = 4
 
 _DTYPE_CODE = {torch.float32: NF_F32, torch.float16: NF_F16, torch.bfloat16: NF_BF16}
 

@@ -1,0 +1,549 @@
+// Hash-encoding backward by binning (D = 3, F = 2, 16-bit upstream gradient).
+//
+// Every (point, level, corner) contributes  w * dout[n, 2l .. 2l+1]  to one table row.  Scattering these with
+// global atomics is bound by the chip's atomic request rate; accumulating them in LDS needs the contributions to
+// one stretch of the table together.  So the contributions are first sorted by table bin (BIN_ROWS rows):
+//
+//   count   : per (level, bin) the number of records, for the whole batch (histogram) and per workgroup
+//   offsets : exclusive scan of the histogram -> where each bin's records start; list of accumulation tasks
+//   fill    : every workgroup takes FILL_POINTS points and, level by level, sorts their records by bin in LDS
+//             and copies them out in runs, into room reserved with one atomic per (workgroup, bin)
+//   accum   : one workgroup per (bin, slice of its records): the bin's rows live in LDS as two 64-bit integers
+//             each and every contribution is one integer LDS atomic per feature (float LDS atomics and
+//             compare-and-swap loops are an order of magnitude slower once a few thousand adds are in flight on
+//             a tile); the tile is then converted and added to the gradient table (plain read-modify-write when
+//             the bin has a single slice, atomics otherwise)
+//
+// A record is the pair of corners that differ in x only: 16 bytes {row0 | row1 << 13 inside the bin, w0, w1 as
+// float32, packed 16-bit gradient pair}.  The two rows of a pair share the bin: on a dense level they are
+// neighbours, on a hashed level the x prime is 1 and  (x+1) ^ a  differs from  x ^ a  only below the lowest zero
+// bit of x.  When they do not (bin border, 13 trailing ones in x) the pair becomes two records with one zero weight
+// each.  The count and fill kernels apply the same rule, so their record counts agree.
+//
+// Integer accumulation: fill also finds max |dout| per level; with 2^e the power of two above it, a contribution
+// w * g is accumulated as round(w * g * 2^(30 - e)), below 2^30 in magnitude, so a task's records cannot
+// overflow 64 bits, the rounding is 2^-30 of the level's largest gradient per contribution, and the sum does
+// not depend on the order of the records.  A level whose gradient holds an inf or a nan gets nan in every row
+// it touches.
+//
+// Arithmetic (cell, corner rows, weights) is the forward's, see hash_encoding.hip.
+#include "hash_common.h"
+
+namespace nf {
+
+constexpr int BIN_ROWS_LOG2 = 13;
+constexpr int BIN_ROWS = 1 << BIN_ROWS_LOG2;  // rows per bin (two 64-bit sums each: 128 KiB of LDS in the accumulation)
+constexpr uint32_t BIN_MASK = BIN_ROWS - 1;
+constexpr int FILL_POINTS = 512;              // points (= threads) per workgroup of count and fill
+constexpr int FILL_RECORDS = FILL_POINTS * 8; // most records a workgroup stages per level
+constexpr int ACC_THREADS = 1024;
+constexpr int ACC_INFLIGHT = 8;               // records in flight per thread
+constexpr uint32_t SLICE_RECORDS = 98304;     // a bin with at most this many records is one accumulation task
+constexpr uint32_t SPLIT_RECORDS = 32768;     // a bigger bin is cut into tasks of about this many
+constexpr int MAX_BINS_PER_LEVEL = 1024;
+constexpr int MAX_BINS_TOTAL = 2560;          // LDS of the count and fill kernels
+constexpr int AGG_MAX_BINS = 16;              // levels with at most this many bins rank through wave ballots
+
+struct BinPlan {
+  int n_levels;
+  int nbins[NF_MAX_LEVELS];
+  int binbase[NF_MAX_LEVELS + 1];  // first global bin of the level
+};
+
+// workspace (32-bit words): hist[NB] | gmax[32] | cursor[NB] | n_tasks, pad[3] | tasks[max_tasks][4] |
+// wg_counts[workgroups][NB] | records[R][4]      (hist and gmax are cleared together)
+struct BinWs {
+  uint32_t* hist;
+  uint32_t* gmax;  // per level: largest |dout| bit pattern (15 bits)
+  uint32_t* cursor;
+  uint32_t* n_tasks;
+  uint4* tasks;
+  uint32_t* wg_counts;
+  uint4* records;
+  uint32_t max_tasks;
+};
+
+// Workgroup barrier that orders LDS accesses only: global stores issued before it stay in flight (a plain
+// __syncthreads() would wait for them to complete).
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+struct Located3 {
+  uint32_t c[3];
+  float fr[3];
+};
+__device__ __forceinline__ Located3 locate(const float (&v)[3], float fres) {
+  Located3 r;
+#pragma unroll
+  for (int d = 0; d < 3; ++d) {
+    const float pos = v[d] * fres;
+    const float fl = floorf(pos);
+    r.c[d] = (uint32_t)(int)fl;
+    r.fr[d] = pos - fl;
+  }
+  return r;
+}
+__device__ __forceinline__ void load_point(const void* coords, int cdt, int64_t csn, int64_t csd, int64_t n, float scale,
+                                           float (&v)[3]) {
+#pragma unroll
+  for (int d = 0; d < 3; ++d) {
+    v[d] = load_as_f32(coords, n * csn + d * csd, cdt);
+    if (scale != 1.0f) v[d] = v[d] / scale;
+  }
+}
+
+// Position of every active lane among the wave's lanes with the same bin, on top of one LDS add per distinct bin.
+__device__ __forceinline__ uint32_t wave_rank(uint32_t* cnt, uint32_t bin, bool active, int lane) {
+  uint32_t rank = 0;
+  unsigned long long todo = __ballot(active);
+  while (todo) {
+    const int leader = __ffsll((long long)todo) - 1;
+    const uint32_t b = (uint32_t)__shfl((int)bin, leader);
+    const bool mine = active && bin == b;
+    const unsigned long long m = __ballot(mine);
+    uint32_t base = 0;
+    if (lane == leader) base = atomicAdd(cnt + b, (uint32_t)__popcll(m));
+    base = (uint32_t)__shfl((int)base, leader);
+    if (mine) rank = base + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
+    todo &= ~m;
+  }
+  return rank;
+}
+
+__global__ void hash_bwd_bin_zero_k(uint32_t* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
+// ---------------------------------------------------------------------------------------
+// count
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_count_k(const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                                    int64_t N, DevGeom g, BinPlan bp, const int64_t* primes,
+                                                                    float scale, uint32_t* hist, uint32_t* wg_counts) {
+  extern __shared__ uint32_t lh[];  // all bins of all levels
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int NB = bp.binbase[bp.n_levels];
+  for (int i = tid; i < NB; i += FILL_POINTS) lh[i] = 0u;
+  lds_barrier();
+  const int64_t n = (int64_t)blockIdx.x * FILL_POINTS + tid;
+  const bool valid = n < N;
+  float v[3] = {0.0f, 0.0f, 0.0f};
+  if (valid) load_point(coords, cdt, csn, csd, n, scale, v);
+  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], (uint32_t)primes[2]};
+  for (int l = 0; l < bp.n_levels; ++l) {
+    uint32_t* cnt = lh + bp.binbase[l];
+    const int nb = bp.nbins[l];
+    if (nb == 1) {
+      if (valid) {
+        const unsigned long long m = __ballot(true);
+        if (lane == __ffsll((long long)m) - 1) atomicAdd(cnt, 4u * (uint32_t)__popcll(m));
+      }
+      continue;
+    }
+    const Located3 q = locate(v, (float)g.res[l]);
+    const Corner8 r = rows_d3(q.c, l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const uint32_t b0 = r.row[2 * c] >> BIN_ROWS_LOG2, b1 = r.row[2 * c + 1] >> BIN_ROWS_LOG2;
+      if (nb <= AGG_MAX_BINS) {
+        wave_rank(cnt, b0, valid, lane);
+        if (__any(valid && b1 != b0)) wave_rank(cnt, b1, valid && b1 != b0, lane);
+      } else if (valid) {
+        atomicAdd(cnt + b0, 1u);
+        if (b1 != b0) atomicAdd(cnt + b1, 1u);
+      }
+    }
+  }
+  lds_barrier();
+  uint32_t* mine = wg_counts + (int64_t)blockIdx.x * NB;  // the fill kernel's workgroup of the same index reads these
+  for (int i = tid; i < NB; i += FILL_POINTS) {
+    const uint32_t c = lh[i];
+    mine[i] = c;
+    if (c) atomicAdd(hist + i, c);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// offsets: one workgroup
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t x, uint32_t* wave_sums, uint32_t* total) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
+  uint32_t incl = x;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const uint32_t y = (uint32_t)__shfl_up((int)incl, d);
+    if (lane >= d) incl += y;
+  }
+  __syncthreads();  // wave_sums may still be read from the previous call
+  if (lane == 63) wave_sums[wave] = incl;
+  __syncthreads();
+  uint32_t before = 0, all = 0;
+  for (int w = 0; w < nw; ++w) {
+    const uint32_t s = wave_sums[w];
+    if (w < wave) before += s;
+    all += s;
+  }
+  *total = all;
+  return before + incl - x;
+}
+
+__global__ __launch_bounds__(1024) void hash_bwd_bin_offsets_k(const uint32_t* hist, uint32_t* cursor, uint32_t* n_tasks,
+                                                               uint4* tasks, int NB, uint32_t max_tasks) {
+  __shared__ uint32_t wave_sums[16];
+  uint32_t rec_run = 0, task_run = 0;
+  for (int b0 = 0; b0 < NB; b0 += 1024) {
+    const int b = b0 + (int)threadIdx.x;
+    const uint32_t c = b < NB ? hist[b] : 0u;
+    const uint32_t slices = c <= SLICE_RECORDS ? (c ? 1u : 0u) : (c + SPLIT_RECORDS - 1u) / SPLIT_RECORDS;
+    uint32_t rec_total, task_total;
+    const uint32_t start = rec_run + block_exclusive_scan(c, wave_sums, &rec_total);
+    const uint32_t t0 = task_run + block_exclusive_scan(slices, wave_sums, &task_total);
+    if (b < NB) {
+      cursor[b] = start;
+      // equal slices, so that no workgroup gets a short tail
+      const uint32_t per = slices ? (c + slices - 1u) / slices : 0u;
+      for (uint32_t s = 0; s < slices; ++s) {
+        uint32_t lo = start + s * per, hi = start + (s + 1u) * per;
+        if (hi > start + c) hi = start + c;
+        if (lo > hi) lo = hi;
+        if (t0 + s < max_tasks) tasks[t0 + s] = make_uint4((uint32_t)b, lo, hi, slices > 1u ? 1u : 0u);
+      }
+    }
+    rec_run += rec_total;
+    task_run += task_total;
+  }
+  if (threadIdx.x == 0) *n_tasks = task_run < max_tasks ? task_run : max_tasks;
+}
+
+// ---------------------------------------------------------------------------------------
+// fill
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                                   const uint16_t* dout, int64_t dout_stride, int64_t N,
+                                                                   DevGeom g, BinPlan bp, const int64_t* primes, float scale,
+                                                                   const uint32_t* wg_counts, uint32_t* cursor, uint32_t* gmax,
+                                                                   uint4* records) {
+  extern __shared__ __align__(16) unsigned char fill_smem[];
+  const int NB = bp.binbase[bp.n_levels];
+  uint4* stage = reinterpret_cast<uint4*>(fill_smem);                     // [FILL_RECORDS] records sorted by bin
+  uint16_t* binid = reinterpret_cast<uint16_t*>(stage + FILL_RECORDS);    // bin (within the level) of each staged record
+  uint32_t* cur = reinterpret_cast<uint32_t*>(binid + FILL_RECORDS);      // [NB] next staged position of a bin
+  uint32_t* delta = cur + NB;                                             // [NB] global minus staged position
+  uint32_t* totals = delta + NB;                                          // [levels] records of this workgroup per level
+  uint32_t* lmax = totals + NF_MAX_LEVELS;                                // [levels] largest |dout| pattern
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t n0 = (int64_t)blockIdx.x * FILL_POINTS;
+  const int64_t n = n0 + tid;
+  const bool valid = n < N;
+  // This workgroup's share of every bin, counted by the count kernel: one reservation per non-empty bin, all in
+  // flight together.
+  for (int i = tid; i < NB; i += FILL_POINTS) {
+    const uint32_t c = wg_counts[(int64_t)blockIdx.x * NB + i];
+    cur[i] = c;
+    delta[i] = c ? atomicAdd(cursor + i, c) : 0u;
+  }
+  if (tid < NF_MAX_LEVELS) lmax[tid] = 0u;
+  float v[3] = {0.0f, 0.0f, 0.0f};
+  if (valid) load_point(coords, cdt, csn, csd, n, scale, v);
+  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], (uint32_t)primes[2]};
+  // this point's gradient row, read once (up to 16 levels live in registers)
+  const uint32_t* grow = reinterpret_cast<const uint32_t*>(dout + (valid ? n : 0) * dout_stride);
+  uint32_t gr[16];
+  const bool row_vec = bp.n_levels <= 16 && (bp.n_levels & 3) == 0 && ((uintptr_t)dout & 15u) == 0 && (dout_stride & 7) == 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    uint4 t = make_uint4(0u, 0u, 0u, 0u);
+    if (row_vec && valid && 4 * i < bp.n_levels) t = reinterpret_cast<const uint4*>(grow)[i];
+    gr[4 * i] = t.x;
+    gr[4 * i + 1] = t.y;
+    gr[4 * i + 2] = t.z;
+    gr[4 * i + 3] = t.w;
+  }
+  lds_barrier();
+  // staged start of every bin inside its level (exclusive scan of the counts), one wave per level
+  for (int l = wave; l < bp.n_levels; l += FILL_POINTS / 64) {
+    const int nb = bp.nbins[l], gb0 = bp.binbase[l];
+    uint32_t run = 0;
+    for (int b0 = 0; b0 < nb; b0 += 64) {
+      const int b = b0 + lane;
+      const uint32_t c = b < nb ? cur[gb0 + b] : 0u;
+      uint32_t incl = c;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t y = (uint32_t)__shfl_up((int)incl, d);
+        if (lane >= d) incl += y;
+      }
+      const uint32_t excl = run + incl - c;
+      if (b < nb) {
+        cur[gb0 + b] = excl;
+        delta[gb0 + b] -= excl;
+      }
+      run += (uint32_t)__shfl((int)incl, 63);
+    }
+    if (lane == 0) totals[l] = run;
+  }
+  lds_barrier();
+
+  for (int l = 0; l < bp.n_levels; ++l) {
+    const int nb = bp.nbins[l];
+    uint32_t* lcur = cur + bp.binbase[l];
+    const uint32_t* ldelta = delta + bp.binbase[l];
+    uint32_t packed = 0u;
+    if (row_vec) {
+      packed = gr[0];
+#pragma unroll
+      for (int i = 1; i < 16; ++i) packed = (l == i) ? gr[i] : packed;
+    } else if (valid) {
+      packed = grow[l];
+    }
+    {
+      // largest |g| of the level: positive 16-bit float patterns order like integers
+      const uint32_t pk = packed & 0x7fff7fffu;
+      uint32_t m = (pk & 0xffffu) > (pk >> 16) ? (pk & 0xffffu) : (pk >> 16);
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t o = (uint32_t)__shfl_xor((int)m, d);
+        m = o > m ? o : m;
+      }
+      if (lane == 0 && m) atomicMax(lmax + l, m);
+    }
+    {
+      const Located3 q = locate(v, (float)g.res[l]);
+      const Corner8 r = rows_d3(q.c, l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi);
+      float w[8];
+      weights_d3(q.fr, w);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const uint32_t r0 = r.row[2 * c], r1 = r.row[2 * c + 1];
+        const uint32_t b0 = r0 >> BIN_ROWS_LOG2, b1 = r1 >> BIN_ROWS_LOG2;
+        const bool split = b1 != b0;
+        uint32_t pos;
+        if (nb == 1) pos = (uint32_t)tid * 4u + (uint32_t)c;  // the valid points are the first of the workgroup
+        else if (nb <= AGG_MAX_BINS) pos = wave_rank(lcur, b0, valid, lane);
+        else pos = valid ? atomicAdd(lcur + b0, 1u) : 0u;
+        if (valid) {
+          const uint32_t rr = (r0 & BIN_MASK) | ((split ? r0 : r1) & BIN_MASK) << BIN_ROWS_LOG2;
+          stage[pos] = make_uint4(rr, __float_as_uint(w[2 * c]), split ? 0u : __float_as_uint(w[2 * c + 1]), packed);
+          binid[pos] = (uint16_t)b0;
+        }
+        if (nb > 1 && __any(valid && split)) {
+          const bool on = valid && split;
+          uint32_t pos1;
+          if (nb <= AGG_MAX_BINS) pos1 = wave_rank(lcur, b1, on, lane);
+          else pos1 = on ? atomicAdd(lcur + b1, 1u) : 0u;
+          if (on) {
+            const uint32_t rr = (r1 & BIN_MASK) | (r1 & BIN_MASK) << BIN_ROWS_LOG2;
+            stage[pos1] = make_uint4(rr, __float_as_uint(w[2 * c + 1]), 0u, packed);
+            binid[pos1] = (uint16_t)b1;
+          }
+        }
+      }
+    }
+    lds_barrier();
+    const uint32_t total = totals[l];
+    for (uint32_t i = tid; i < total; i += FILL_POINTS) records[i + ldelta[binid[i]]] = stage[i];
+    lds_barrier();  // the next level overwrites the stage
+  }
+  if (tid < bp.n_levels) {
+    const uint32_t m = lmax[tid];
+    if (m > *(volatile uint32_t*)(gmax + tid)) atomicMax(gmax + tid, m);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// accumulate
+// ---------------------------------------------------------------------------------------
+template <typename GT>
+__global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const uint4* records, const uint4* tasks,
+                                                                    const uint32_t* n_tasks, const uint32_t* gmax, float* dtable,
+                                                                    DevGeom g, BinPlan bp) {
+  extern __shared__ unsigned long long acc_tile[];  // [BIN_ROWS][2] fixed-point sums
+  if (blockIdx.x >= *n_tasks) return;
+  const int tid = threadIdx.x;
+  const uint4 task = tasks[blockIdx.x];
+  int l = 0;
+  while (l + 1 < bp.n_levels && (int)task.x >= bp.binbase[l + 1]) ++l;
+  const uint32_t row0 = (task.x - (uint32_t)bp.binbase[l]) << BIN_ROWS_LOG2;
+  const uint32_t left = g.rows[l] - row0;
+  const uint32_t nrows = left < (uint32_t)BIN_ROWS ? left : (uint32_t)BIN_ROWS;
+  // fixed-point scale 2^se of the level:  |w * g| * 2^se < 2^30
+  const float gm = GT::to_f32((uint16_t)gmax[l]);
+  const bool nonfinite = !(gm <= 3.0e38f);
+  int se = 0;
+  if (!nonfinite && gm > 0.0f) {
+    int ex;
+    frexpf(gm, &ex);  // gm = f * 2^ex, f in [0.5, 1)
+    se = 30 - ex;
+    se = se > 120 ? 120 : se;
+  }
+  const float s_lo = nonfinite ? 0.0f : ldexpf(1.0f, se / 2), s_hi = ldexpf(1.0f, se - se / 2);  // two steps stay inside float range
+  for (uint32_t i = tid; i < 2u * nrows; i += ACC_THREADS) acc_tile[i] = 0ull;
+  lds_barrier();
+  // the next round's records are loaded before this round's adds
+  uint4 q[ACC_INFLIGHT];
+#pragma unroll
+  for (int k = 0; k < ACC_INFLIGHT; ++k) {
+    const uint32_t i = task.y + k * ACC_THREADS + tid;
+    q[k] = i < task.z ? records[i] : make_uint4(0u, 0u, 0u, 0u);
+  }
+  for (uint32_t i0 = task.y; i0 < task.z; i0 += ACC_THREADS * ACC_INFLIGHT) {
+    uint32_t slot[ACC_INFLIGHT][2];
+    int32_t f[ACC_INFLIGHT][4];
+#pragma unroll
+    for (int k = 0; k < ACC_INFLIGHT; ++k) {
+      const float g0 = GT::to_f32((uint16_t)(q[k].w & 0xffffu)) * s_lo, g1 = GT::to_f32((uint16_t)(q[k].w >> 16)) * s_lo;
+      const float w0 = __uint_as_float(q[k].y), w1 = __uint_as_float(q[k].z);  // records past the end: zero weights
+      slot[k][0] = q[k].x & BIN_MASK;
+      slot[k][1] = (q[k].x >> BIN_ROWS_LOG2) & BIN_MASK;
+      f[k][0] = __float2int_rn(w0 * g0 * s_hi);
+      f[k][1] = __float2int_rn(w0 * g1 * s_hi);
+      f[k][2] = __float2int_rn(w1 * g0 * s_hi);
+      f[k][3] = __float2int_rn(w1 * g1 * s_hi);
+      if (nonfinite) {  // only mark the rows the level touches
+        f[k][0] = f[k][1] = w0 != 0.0f;
+        f[k][2] = f[k][3] = w1 != 0.0f;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < ACC_INFLIGHT; ++k) {
+      const uint32_t i = i0 + ACC_THREADS * ACC_INFLIGHT + k * ACC_THREADS + tid;
+      q[k] = i < task.z ? records[i] : make_uint4(0u, 0u, 0u, 0u);
+    }
+#pragma unroll
+    for (int k = 0; k < ACC_INFLIGHT; ++k)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (f[k][j]) atomicAdd(acc_tile + 2u * slot[k][j >> 1] + (uint32_t)(j & 1), (unsigned long long)(long long)f[k][j]);
+  }
+  lds_barrier();
+  float* dst = dtable + (g.row_offset[l] + (int64_t)row0) * 2;
+  const float qnan = __uint_as_float(0x7fc00000u);
+  const uint32_t nvals = 2u * nrows;
+  constexpr int U = 4;  // values per thread whose table reads are in flight together
+  for (uint32_t i0 = 0; i0 < nvals; i0 += ACC_THREADS * U) {
+    float x[U], old[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t i = i0 + u * ACC_THREADS + tid;
+      const long long a = i < nvals ? (long long)acc_tile[i] : 0ll;
+      // |a| < 2^48 is exact in double and so is the division by 2^se: one rounding, to float, at the end
+      x[u] = a == 0 ? 0.0f : (float)ldexp((double)a, -se);
+      if (nonfinite && a != 0) x[u] = qnan;
+      old[u] = (x[u] != 0.0f && !task.w) ? dst[i] : 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t i = i0 + u * ACC_THREADS + tid;
+      if (x[u] != 0.0f) {
+        if (task.w) unsafeAtomicAdd(dst + i, x[u]);
+        else dst[i] = old[u] + x[u];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------
+static bool bin_plan(int64_t N, const nf_hash_geom* geom, int dout_dtype, BinPlan* bp, int64_t* records, uint32_t* max_tasks) {
+  if (geom->dims != 3 || geom->feat != 2 || dout_dtype == NF_F32 || N <= 0) return false;
+  bp->n_levels = geom->levels;
+  int nb_total = 0;
+  for (int l = 0; l < geom->levels; ++l) {
+    const int64_t r = geom->rows[l];
+    if (l >= geom->first_hash_level && (r & (r - 1)) != 0) return false;  // hashed levels: power-of-two sizes
+    const int64_t nb = (r + BIN_ROWS - 1) / BIN_ROWS;
+    if (nb > MAX_BINS_PER_LEVEL) return false;
+    bp->nbins[l] = (int)nb;
+    bp->binbase[l] = nb_total;
+    nb_total += (int)nb;
+  }
+  bp->binbase[geom->levels] = nb_total;
+  if (nb_total > MAX_BINS_TOTAL) return false;
+  // room for every pair to be split in two; normally half of it is used
+  const int64_t R = N * geom->levels * 8;
+  if (R >= ((int64_t)1 << 32) - 4 * ACC_THREADS * ACC_INFLIGHT) return false;  // 32-bit record positions
+  *records = R;
+  *max_tasks = (uint32_t)(nb_total + R / SPLIT_RECORDS + 1);
+  return true;
+}
+
+static int64_t wg_count_words(int64_t N, int NB) { return (((N + FILL_POINTS - 1) / FILL_POINTS) * NB + 3) & ~(int64_t)3; }
+
+static int64_t bin_ws(void* workspace, const BinPlan& bp, int64_t N, int64_t R, uint32_t max_tasks, BinWs* ws) {
+  uint32_t* p = (uint32_t*)workspace;
+  const int NB = bp.binbase[bp.n_levels];
+  const int NBp = (NB + 3) & ~3;
+  int64_t o = 0;
+  ws->hist = p + o; o += NBp;
+  ws->gmax = p + o; o += 32;
+  ws->cursor = p + o; o += NBp;
+  ws->n_tasks = p + o; o += 4;
+  ws->tasks = reinterpret_cast<uint4*>(p + o); o += 4 * (int64_t)max_tasks;
+  ws->wg_counts = p + o; o += wg_count_words(N, NB);
+  ws->records = reinterpret_cast<uint4*>(p + o); o += 4 * R;
+  ws->max_tasks = max_tasks;
+  return o * 4;
+}
+
+int64_t bwd_bin_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype) {
+  BinPlan bp;
+  int64_t R;
+  uint32_t max_tasks;
+  if (!bin_plan(n_points, geom, dout_dtype, &bp, &R, &max_tasks)) return 0;
+  BinWs ws;
+  return bin_ws(nullptr, bp, n_points, R, max_tasks, &ws);
+}
+
+int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const void* dout, int ddt, int64_t dout_stride,
+                   float* dtable, int64_t N, const nf_hash_geom* geom, const DevGeom& g, const int64_t* primes, float scale,
+                   void* workspace, hipStream_t s) {
+  BinPlan bp;
+  int64_t R;
+  uint32_t max_tasks;
+  NF_REQUIRE(bin_plan(N, geom, ddt, &bp, &R, &max_tasks), NF_EUNSUPPORTED, "binned backward does not cover this geometry");
+  NF_REQUIRE(((uintptr_t)workspace & 15u) == 0, NF_EALIGN, "workspace must be 16-byte aligned");
+  BinWs ws;
+  bin_ws(workspace, bp, N, R, max_tasks, &ws);
+  const int NB = bp.binbase[bp.n_levels];
+  const int NBp = (NB + 3) & ~3;
+  const unsigned blocks = (unsigned)((N + FILL_POINTS - 1) / FILL_POINTS);
+
+  hipLaunchKernelGGL(hash_bwd_bin_zero_k, dim3((unsigned)((NBp + 32 + 255) / 256)), dim3(256), 0, s, ws.hist, NBp + 32);
+  if (int rc = check_launch("hash_bwd_bin_zero")) return rc;
+  hipLaunchKernelGGL(hash_bwd_bin_count_k, dim3(blocks), dim3(FILL_POINTS), (size_t)NB * 4, s, coords, cdt, csn, csd, N, g, bp,
+                     primes, scale, ws.hist, ws.wg_counts);
+  if (int rc = check_launch("hash_bwd_bin_count")) return rc;
+  hipLaunchKernelGGL(hash_bwd_bin_offsets_k, dim3(1), dim3(1024), 0, s, (const uint32_t*)ws.hist, ws.cursor, ws.n_tasks,
+                     ws.tasks, NB, max_tasks);
+  if (int rc = check_launch("hash_bwd_bin_offsets")) return rc;
+  {
+    const size_t lds = (size_t)FILL_RECORDS * (sizeof(uint4) + sizeof(uint16_t)) + ((size_t)2 * NB + 2 * NF_MAX_LEVELS) * 4;
+    hipError_t e = hipFuncSetAttribute((const void*)hash_bwd_bin_fill_k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    hipLaunchKernelGGL(hash_bwd_bin_fill_k, dim3(blocks), dim3(FILL_POINTS), lds, s, coords, cdt, csn, csd,
+                       (const uint16_t*)dout, dout_stride, N, g, bp, primes, scale, (const uint32_t*)ws.wg_counts, ws.cursor,
+                       ws.gmax, ws.records);
+    if (int rc = check_launch("hash_bwd_bin_fill")) return rc;
+  }
+  {
+    const size_t lds = (size_t)BIN_ROWS * 2 * sizeof(unsigned long long);
+    const void* kern = ddt == NF_F16 ? (const void*)hash_bwd_bin_accum_k<F16> : (const void*)hash_bwd_bin_accum_k<BF16>;
+    hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    const uint4* rc_ = ws.records;
+    const uint4* tk = ws.tasks;
+    const uint32_t* nt = ws.n_tasks;
+    const uint32_t* gm = ws.gmax;
+    void* args[] = {(void*)&rc_, (void*)&tk, (void*)&nt, (void*)&gm, (void*)&dtable, (void*)&g, (void*)&bp};
+    e = hipLaunchKernel(kern, dim3(max_tasks), dim3(ACC_THREADS), args, lds, s);
+    if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(hash_bwd_bin_accum): %s", hipGetErrorString(e));
+    return check_launch("hash_bwd_bin_accum");
+  }
+}
+
+}  // namespace nf

@@ -44,7 +44,7 @@ PI_3: Final = 805_459_861
 DIVIDER_CONFIGS: Dict[Any, int] = {}
 BWD_DIVIDER_CONFIGS: Dict[Any, int] = {}
 
-_FLAGS = 0  # test hook: _lib.NF_HASH_FORCE_GENERIC / NF_HASH_FORCE_ATOMIC select the simpler kernels
+_FLAGS = 0  # test hook: _lib.NF_HASH_FORCE_GENERIC / NF_HASH_FORCE_ATOMIC / NF_HASH_FORCE_PLANES select other kernels
 
 
 # ---------------------------------------------------------------------------
@@ -129,7 +129,7 @@ def _launch_backward(coords2d: Tensor, do2d: Tensor, de: Tensor, pi: Tensor, T: 
     geom = level_geometry(T, levels, D, F, min_res, max_res)
     lib = _lib.load()
     # scratch for the LDS-tile backward (bit-planes); torch's caching allocator makes this free after the first call
-    ws_bytes = 0 if _FLAGS else lib.nf_hash_encode_bwd_workspace_bytes(N, geom, _lib.dtype_code(do2d.dtype))
+    ws_bytes = 0 if (_FLAGS & 3) else lib.nf_hash_encode_bwd_workspace_bytes(N, geom, _lib.dtype_code(do2d.dtype))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=coords2d.device) if ws_bytes > 0 else None
     rc = lib.nf_hash_encode_bwd(
         coords2d.data_ptr(), _lib.dtype_code(coords2d.dtype), coords2d.stride(0), coords2d.stride(1),
