@@ -120,9 +120,12 @@ __device__ __forceinline__ void stage_bias_row(float* dst, const uint16_t* b, in
 // ---------------------------------------------------------------------------------------
 // Forward: up to FWD_GROUP blocks per launch
 // ---------------------------------------------------------------------------------------
-template <typename T, int HP>
-__global__ __launch_bounds__(256) void rev_fwd_k(RevArgs a) {
+// ACT >= 0 fixes the activation at compile time (no per-element selection); -1 reads it from the arguments.
+template <typename T, int HP, int ACT>
+__global__ __launch_bounds__(768) void rev_fwd_k(RevArgs a) {
   constexpr int MT = HP / 16, KC = HP / 32, LAYER = MT * KC * RFRAG;
+  const int act = ACT >= 0 ? ACT : a.act;
+  const int nwaves = (int)(blockDim.x >> 6);
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, nthreads = blockDim.x, lane = tid & 63, wave = tid >> 6;
   uint16_t* frags = reinterpret_cast<uint16_t*>(smem);  // [nblocks][F.w1, F.w2, G.w1, G.w2][LAYER]
@@ -139,7 +142,7 @@ __global__ __launch_bounds__(256) void rev_fwd_k(RevArgs a) {
   __syncthreads();
 
   const int64_t n_chunks = (a.rows + 31) / 32;
-  for (int64_t chunk = (int64_t)blockIdx.x * 4 + wave; chunk < n_chunks; chunk += (int64_t)gridDim.x * 4) {
+  for (int64_t chunk = (int64_t)blockIdx.x * nwaves + wave; chunk < n_chunks; chunk += (int64_t)gridDim.x * nwaves) {
     const int64_t row0 = chunk * 32;
     f32x4_t s1[2][4], s2[2][4];  // the two halves of the residual stream, float32
 #pragma unroll
@@ -172,7 +175,7 @@ __global__ __launch_bounds__(256) void rev_fwd_k(RevArgs a) {
           for (int mt = 0; mt < MT; ++mt) {
             f32x4_t z = acc[nt][mt];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) z[r] = act_fwd(z[r], a.act);
+            for (int r = 0; r < 4; ++r) z[r] = act_fwd(z[r], act);
             p[nt][mt] = pack4<T>(z);
           }
         tiles_to_frags<MT>(p, t);
@@ -450,15 +453,21 @@ static int launch_rev_fwd(RevArgs a, hipStream_t s) {
   constexpr int LAYER = (HP / 16) * (HP / 32) * RFRAG;
   const size_t lds = (size_t)a.nblocks * 4 * LAYER * 2 + (size_t)a.nblocks * 4 * HP * 4;
   const int64_t chunks = (a.rows + 31) / 32;
-  int64_t blocks = (chunks + 3) / 4;
+  // weights of several blocks leave room for one workgroup per CU only: give it 12 waves to keep three per SIMD
+  const int waves = lds > 80 * 1024 ? 12 : 4;
+  int64_t blocks = (chunks + waves - 1) / waves;
   const int64_t cap = (int64_t)rev_cus() * (lds > 80 * 1024 ? 1 : 2);
   if (blocks > cap) blocks = cap;
-  auto kern = rev_fwd_k<T, HP>;
+  const void* kern = a.act == NF_ACT_GELU   ? (const void*)rev_fwd_k<T, HP, NF_ACT_GELU>
+                     : a.act == NF_ACT_RELU ? (const void*)rev_fwd_k<T, HP, NF_ACT_RELU>
+                                            : (const void*)rev_fwd_k<T, HP, -1>;
   if (lds > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), lds, s, a);
+  void* args[] = {(void*)&a};
+  const hipError_t e = hipLaunchKernel(kern, dim3((unsigned)blocks), dim3(64 * waves), args, lds, s);
+  if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(rev_fwd): %s", hipGetErrorString(e));
   return check_launch("rev_fwd");
 }
 
