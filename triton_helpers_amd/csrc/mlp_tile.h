@@ -256,6 +256,52 @@ __device__ __forceinline__ void store_rows_tile(uint16_t* base, int64_t stride, 
   }
 }
 
+// ---- transposes and row sums for products that contract over the rows of a chunk -----------
+// Transpose through the matrix core.  f0 / f1 are chain-order fragments of rows 0-15 / 16-31 of a chunk
+// (lane (row, g): 8 features of K-chunk kc); e selects 16 of those 32 features (sel_frag()).  The product
+// F * E has exactly one non-zero term per output, so it is exact; the result, packed back to 16 bit, is the
+// operand of a product that contracts over the chunk's 32 rows: lane (feature, g) holds rows 4g .. 4g+3 and
+// 16+4g .. 16+4g+3 of that feature.  Both operands of such a product use the same row order.
+template <typename T>
+__device__ __forceinline__ Frag transpose_tile(const Frag& f0, const Frag& f1, const Frag& e) {
+  const f32x4_t z = {0.0f, 0.0f, 0.0f, 0.0f};
+  const f32x4_t a = mfma16<T>(f0, e, z);
+  const f32x4_t b = mfma16<T>(f1, e, z);
+  Frag o;
+  o.w[0] = pack2<T>(a[0], a[1]);
+  o.w[1] = pack2<T>(a[2], a[3]);
+  o.w[2] = pack2<T>(b[0], b[1]);
+  o.w[3] = pack2<T>(b[2], b[3]);
+  return o;
+}
+// Selector of features 16*half .. 16*half+15 of a chain-order K-chunk: B[k][n] = 1 where slot k holds feature
+// 16*half + n, i.e. lane (n, g) with g == n / 4 carries a 1.0 in element 4*half + n % 4.
+template <typename T>
+__device__ __forceinline__ Frag sel_frag(int half, int lane) {
+  const int n = lane & 15, g = lane >> 4;
+  const uint32_t one = (pack2<T>(1.0f, 1.0f) & 0xffffu) << (16 * (n & 1));
+  const uint32_t v = (g == (n >> 2)) ? one : 0u;
+  const int d = 2 * half + ((n & 3) >> 1);
+  Frag e;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) e.w[i] = (i == d) ? v : 0u;
+  return e;
+}
+
+// acc + lo + hi of a packed 16-bit pair (one v_dot2 instruction)
+template <typename T>
+__device__ __forceinline__ float dot2_ones(uint32_t p, float acc);
+template <>
+__device__ __forceinline__ float dot2_ones<BF16>(uint32_t p, float acc) {
+  const bf16x2_t one = {(__bf16)1.0f, (__bf16)1.0f};
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, p), one, acc, false);
+}
+template <>
+__device__ __forceinline__ float dot2_ones<F16>(uint32_t p, float acc) {
+  const f16x2_t one = {(_Float16)1.0f, (_Float16)1.0f};
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, p), one, acc, false);
+}
+
 inline bool vec_load_ok(const void* p, int64_t stride_elems, int width) {
   return ((uintptr_t)p % 16 == 0) && (stride_elems % 8 == 0) && (width % 8 == 0);
 }

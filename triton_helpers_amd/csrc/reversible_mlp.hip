@@ -8,7 +8,8 @@
 // (y, dy), rebuilds the block's input in-kernel (x2 = y2 - G(y1), x1 = y1 - F(x2)) while it
 // back-propagates, and writes (x, dx), which the next launch reads in place.  No activation
 // of the forward pass is ever stored.  The four weight gradients of a block accumulate in
-// float32 registers over the wave's whole row loop.
+// float32 registers over the wave's whole row loop; their operands (rows along K) are matrix-core
+// transposes of the row-per-lane fragments, so LDS only holds weights.
 //
 // There is no counterpart in the reference; the layer math is that of its fused MLP
 // (triton_helpers/layers/fully_fused_mlp/kernel.py:17-74).
@@ -17,7 +18,6 @@
 namespace nf {
 
 constexpr int RFRAG = 64 * 8;
-constexpr int RPITCH = 40;     // 16-bit elements per feature row of a transposed 32-row panel
 constexpr int FWD_GROUP = 4;   // coupling blocks per forward launch (LDS: 32 KiB of weights per block at H = 64)
 
 struct RevArgs {
@@ -199,57 +199,40 @@ __global__ __launch_bounds__(768) void rev_fwd_k(RevArgs a) {
 // ---------------------------------------------------------------------------------------
 // Backward of one coupling block
 // ---------------------------------------------------------------------------------------
-__device__ __forceinline__ void park_packed_T(uint16_t* panel, int mt, int nt, int lane, uint2 v) {
-  const int n = (lane & 15) + 16 * nt;
-  const int f = 16 * mt + 4 * (lane >> 4);
-  panel[(f + 0) * RPITCH + n] = (uint16_t)(v.x & 0xffffu);
-  panel[(f + 1) * RPITCH + n] = (uint16_t)(v.x >> 16);
-  panel[(f + 2) * RPITCH + n] = (uint16_t)(v.y & 0xffffu);
-  panel[(f + 3) * RPITCH + n] = (uint16_t)(v.y >> 16);
-}
-__device__ __forceinline__ Frag rpanel_frag(const uint16_t* panel, int t, int lane) {
-  Frag f;
-  f.u = *reinterpret_cast<const uint4*>(panel + (16 * t + (lane & 15)) * RPITCH + 8 * (lane >> 4));
-  return f;
-}
-
-// Sum over the 32 rows of feature `lane` of a transposed panel (lanes >= feats return 0).
-template <typename T>
-__device__ __forceinline__ float panel_rowsum(const uint16_t* panel, int feats, int lane) {
-  float s = 0.0f;
-  if (lane < feats) {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const uint4 v = *reinterpret_cast<const uint4*>(panel + lane * RPITCH + 8 * q);
-      s += unpack_lo<T>(v.x) + unpack_hi<T>(v.x) + unpack_lo<T>(v.y) + unpack_hi<T>(v.y) + unpack_lo<T>(v.z) +
-           unpack_hi<T>(v.z) + unpack_lo<T>(v.w) + unpack_hi<T>(v.w);
-    }
+// Activation and its derivative from one pre-activation (GELU shares the exponential between the two).
+template <int ACT>
+__device__ __forceinline__ void act_both(float z, int act, float& h, float& g) {
+  if (ACT == NF_ACT_GELU) {
+    float e;
+    const float cdf = normal_cdf(z, &e);
+    h = z * cdf;
+    g = cdf + z * (0.3989422804014327f * e);
+  } else if (ACT == NF_ACT_RELU) {
+    h = fmaxf(z, 0.0f);
+    g = z > 0.0f ? 1.0f : 0.0f;
+  } else {
+    h = act_fwd(z, act);
+    g = act_grad(z, act);
   }
-  return s;
 }
 
 // Back-propagate through one sub-MLP  out = in_other + S(u):
 //   given u (packed tiles), the incoming gradient d (packed tiles) w.r.t. S's output, computes
 //   s_out = S(u) (float32, returned in `sout`), accumulates dW1, dW2 (and db), and returns du = W1^T dz.
-template <typename T, int MT, int KC>
+// The operands of the weight-gradient products (rows along K) come from matrix-core transposes of the
+// row-per-lane fragments; nothing goes through LDS but the weights.
+// dw2_lds != nullptr: this wave's dW2 accumulator tiles live there ([MT*MT][64 lanes] float4) instead of dw2.
+template <typename T, int MT, int KC, int ACT>
 __device__ __forceinline__ void sub_backward(const uint2 (&u)[2][4], const uint2 (&d)[2][4], f32x4_t (&sout)[2][4],
-                                             f32x4_t (&du)[2][4], f32x4_t (&dw1)[4][4], f32x4_t (&dw2)[4][4],
-                                             float& db1, float& db2, bool want_db, const uint16_t* fw1,
-                                             const uint16_t* fw2, const uint16_t* tw1, const uint16_t* tw2, const float* b1,
-                                             const float* b2, uint16_t* p_in, uint16_t* p_t, uint16_t* p_d, uint16_t* p_dz,
-                                             int act, int lane) {
+                                             f32x4_t (&du)[2][4], f32x4_t (&dw1)[4][4], f32x4_t (&dw2)[4][4], f32x4_t* dw2_lds,
+                                             float (&db1)[4], float (&db2)[4], const uint16_t* fw1, const uint16_t* fw2,
+                                             const uint16_t* tw1, const uint16_t* tw2, const float* b1, const float* b2,
+                                             const Frag (&sel)[2], int act, int lane) {
   Frag uf[2][2], tf[2][2], df[2][2], dzf[2][2];
   uint2 tp[2][4], gp[2][4];
   f32x4_t acc[2][4];
   tiles_to_frags<MT>(u, uf);
   tiles_to_frags<MT>(d, df);
-#pragma unroll
-  for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      park_packed_T(p_in, mt, nt, lane, u[nt][mt]);
-      park_packed_T(p_d, mt, nt, lane, d[nt][mt]);
-    }
   // recompute hidden activation t = act(W1 u + b1) and act'(z)
   rev_layer<T, MT, KC>(acc, uf, fw1, b1, lane);
 #pragma unroll
@@ -259,26 +242,37 @@ __device__ __forceinline__ void sub_backward(const uint2 (&u)[2][4], const uint2
       f32x4_t h, g;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        h[r] = act_fwd(acc[nt][mt][r], act);
-        g[r] = act_grad(acc[nt][mt][r], act);
+        float hv, gv;
+        act_both<ACT>(acc[nt][mt][r], act, hv, gv);
+        h[r] = hv;
+        g[r] = gv;
       }
       tp[nt][mt] = pack4<T>(h);
       gp[nt][mt] = pack4<T>(g);
-      park_packed_T(p_t, mt, nt, lane, tp[nt][mt]);
     }
   tiles_to_frags<MT>(tp, tf);
   // S(u) = W2 t + b2
   rev_layer<T, MT, KC>(sout, tf, fw2, b2, lane);
-  // dW2 += d^T t
+  // dW2 += d^T t, db2 += sum d
   {
     Frag tb[MT];
 #pragma unroll
-    for (int j = 0; j < MT; ++j) tb[j] = rpanel_frag(p_t, j, lane);
+    for (int j = 0; j < MT; ++j) tb[j] = transpose_tile<T>(tf[0][j >> 1], tf[1][j >> 1], sel[j & 1]);
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
-      const Frag da = rpanel_frag(p_d, i, lane);
+      const Frag da = transpose_tile<T>(df[0][i >> 1], df[1][i >> 1], sel[i & 1]);
+      if (dw2_lds != nullptr) {
 #pragma unroll
-      for (int j = 0; j < MT; ++j) dw2[i][j] = mfma16<T>(da, tb[j], dw2[i][j]);
+        for (int j = 0; j < MT; ++j) {
+          f32x4_t* slot = dw2_lds + (i * MT + j) * 64 + lane;
+          *slot = mfma16<T>(da, tb[j], *slot);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < MT; ++j) dw2[i][j] = mfma16<T>(da, tb[j], dw2[i][j]);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) db2[i] = dot2_ones<T>(da.w[q], db2[i]);
     }
   }
   // dt = W2^T d ; dz = dt * act'(z)
@@ -292,28 +286,32 @@ __device__ __forceinline__ void sub_backward(const uint2 (&u)[2][4], const uint2
 #pragma unroll
       for (int r = 0; r < 4; ++r) dz[r] = acc[nt][mt][r] * g[r];
       tp[nt][mt] = pack4<T>(dz);
-      park_packed_T(p_dz, mt, nt, lane, tp[nt][mt]);
     }
   tiles_to_frags<MT>(tp, dzf);
-  if (want_db) {
-    // lane f sums the 32 parked rows of feature f: db1 from dz, db2 from the incoming gradient
-    db1 += panel_rowsum<T>(p_dz, 16 * MT, lane);
-    db2 += panel_rowsum<T>(p_d, 16 * MT, lane);
-  }
-  // dW1 += dz^T u
+  // dW1 += dz^T u, db1 += sum dz
   {
     Frag ub[MT];
 #pragma unroll
-    for (int j = 0; j < MT; ++j) ub[j] = rpanel_frag(p_in, j, lane);
+    for (int j = 0; j < MT; ++j) ub[j] = transpose_tile<T>(uf[0][j >> 1], uf[1][j >> 1], sel[j & 1]);
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
-      const Frag da = rpanel_frag(p_dz, i, lane);
+      const Frag da = transpose_tile<T>(dzf[0][i >> 1], dzf[1][i >> 1], sel[i & 1]);
 #pragma unroll
       for (int j = 0; j < MT; ++j) dw1[i][j] = mfma16<T>(da, ub[j], dw1[i][j]);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) db1[i] = dot2_ones<T>(da.w[q], db1[i]);
     }
   }
   // du = W1^T dz
   rev_layer<T, MT, KC>(du, dzf, tw1, nullptr, lane);
+}
+
+// Bias gradient of feature 16*mt + n: the four lane groups hold partial sums over disjoint rows.
+__device__ __forceinline__ void flush_db_rev(float* db, int dim, int mt, int lane, float v) {
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 32);
+  const int f = 16 * mt + lane;
+  if (db != nullptr && lane < 16 && f < dim) unsafeAtomicAdd(db + f, v);
 }
 
 __device__ __forceinline__ void flush_tile(float* dw, int dim, int mt, int nt, int lane, f32x4_t v) {
@@ -325,9 +323,10 @@ __device__ __forceinline__ void flush_tile(float* dw, int dim, int mt, int nt, i
     if (r0 + r < dim) unsafeAtomicAdd(dw + (size_t)(r0 + r) * dim + c, v[r]);
 }
 
-template <typename T, int HP>
+template <typename T, int HP, int ACT>
 __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
   constexpr int MT = HP / 16, KC = HP / 32, LAYER = MT * KC * RFRAG;
+  const int act = ACT >= 0 ? ACT : a.act;
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, nthreads = blockDim.x, lane = tid & 63, wave = tid >> 6;
   const int H = a.half;
@@ -335,8 +334,12 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
   uint16_t* fw = reinterpret_cast<uint16_t*>(smem);
   uint16_t* tw = fw + 4 * LAYER;
   float* bias = reinterpret_cast<float*>(tw + 4 * LAYER);  // [4][HP]
-  uint16_t* panels = reinterpret_cast<uint16_t*>(bias + 4 * HP) + (size_t)wave * 4 * HP * RPITCH;
-  uint16_t *p_in = panels, *p_t = panels + HP * RPITCH, *p_d = panels + 2 * HP * RPITCH, *p_dz = panels + 3 * HP * RPITCH;
+  // Four 64x64 float32 accumulators would fill the whole accumulation register file and leave none for the
+  // layer products: at HP = 64 the fourth (G's second layer) lives in LDS, 16 KiB per wave.
+  constexpr bool G2_LDS = HP > 32;
+  f32x4_t* g2acc = G2_LDS ? reinterpret_cast<f32x4_t*>(bias + 4 * HP) + (size_t)wave * MT * MT * 64 : nullptr;
+  if (G2_LDS)
+    for (int i = lane; i < MT * MT * 64; i += 64) g2acc[i] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
   for (int s = 0; s < 2; ++s) {
     stage_weight_frags<true, false>(fw + (2 * s) * LAYER, a.w1 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
     stage_weight_frags<true, false>(fw + (2 * s + 1) * LAYER, a.w2 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
@@ -348,48 +351,56 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
   __syncthreads();
 
   f32x4_t dwF1[4][4], dwF2[4][4], dwG1[4][4], dwG2[4][4];
-  float dbF1 = 0.0f, dbF2 = 0.0f, dbG1 = 0.0f, dbG2 = 0.0f;  // lane f: bias gradient of feature f
+  // lane (feature, g) of tile i: partial bias gradient of feature 16*i + n over the rows of lane group g
+  float dbF1[4] = {0.0f, 0.0f, 0.0f, 0.0f}, dbF2[4] = {0.0f, 0.0f, 0.0f, 0.0f}, dbG1[4] = {0.0f, 0.0f, 0.0f, 0.0f},
+        dbG2[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  const Frag sel[2] = {sel_frag<T>(0, lane), sel_frag<T>(1, lane)};
   const f32x4_t zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) dwF1[i][j] = dwF2[i][j] = dwG1[i][j] = dwG2[i][j] = zero4;
-  const bool want_db = a.db1 != nullptr || a.db2 != nullptr;
 
   const int64_t n_chunks = (a.rows + 31) / 32;
   for (int64_t chunk = (int64_t)blockIdx.x * 4 + wave; chunk < n_chunks; chunk += (int64_t)gridDim.x * 4) {
     const int64_t row0 = chunk * 32;
-    uint2 y1[2][4], y2[2][4], d1[2][4], d2[2][4];
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        y1[nt][mt] = load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in);
-        y2[nt][mt] = load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_in);
-        d1[nt][mt] = load_tile_packed(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_dy);
-        d2[nt][mt] = load_tile_packed(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_dy);
-      }
+    // Each half of y and dy is loaded where it is used (and again for the final residual adds, from L2) rather
+    // than held across the two sub-MLPs: registers are the scarce resource here.
+    uint2 x2[2][4], d1[2][4];
     f32x4_t sout[2][4], du[2][4];
-    // ---- G:  y2 = x2 + G(y1)  =>  x2 = y2 - G(y1),  dy1 += (dG/dy1)^T dy2
-    sub_backward<T, MT, KC>(y1, d2, sout, du, dwG1, dwG2, dbG1, dbG2, want_db, fw + 2 * LAYER, fw + 3 * LAYER,
-                            tw + 2 * LAYER, tw + 3 * LAYER, bias + 2 * HP, bias + 3 * HP, p_in, p_t, p_d, p_dz, a.act, lane);
-    uint2 x2[2][4];
+    {
+      uint2 y1[2][4], d2[2][4];
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          y1[nt][mt] = load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in);
+          d2[nt][mt] = load_tile_packed(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_dy);
+        }
+      // ---- G:  y2 = x2 + G(y1)  =>  x2 = y2 - G(y1),  dy1 += (dG/dy1)^T dy2
+      sub_backward<T, MT, KC, ACT>(y1, d2, sout, du, dwG1, dwG2, g2acc, dbG1, dbG2, fw + 2 * LAYER, fw + 3 * LAYER,
+                                   tw + 2 * LAYER, tw + 3 * LAYER, bias + 2 * HP, bias + 3 * HP, sel, act, lane);
+    }
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        x2[nt][mt] = pack4<T>(unpack4<T>(y2[nt][mt]) - sout[nt][mt]);
-        d1[nt][mt] = pack4<T>(unpack4<T>(d1[nt][mt]) + du[nt][mt]);
+        const uint2 y2 = load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_in);
+        const uint2 dy1 = load_tile_packed(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_dy);
+        x2[nt][mt] = pack4<T>(unpack4<T>(y2) - sout[nt][mt]);
+        d1[nt][mt] = pack4<T>(unpack4<T>(dy1) + du[nt][mt]);
       }
     // ---- F:  y1 = x1 + F(x2)  =>  x1 = y1 - F(x2),  dx2 = dy2 + (dF/dx2)^T dy1
-    sub_backward<T, MT, KC>(x2, d1, sout, du, dwF1, dwF2, dbF1, dbF2, want_db, fw, fw + LAYER, tw, tw + LAYER, bias,
-                            bias + HP, p_in, p_t, p_d, p_dz, a.act, lane);
+    sub_backward<T, MT, KC, ACT>(x2, d1, sout, du, dwF1, dwF2, nullptr, dbF1, dbF2, fw, fw + LAYER, tw, tw + LAYER, bias,
+                                 bias + HP, sel, act, lane);
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        const uint2 x1 = pack4<T>(unpack4<T>(y1[nt][mt]) - sout[nt][mt]);
-        const uint2 dx2 = pack4<T>(unpack4<T>(d2[nt][mt]) + du[nt][mt]);
+        const uint2 y1 = load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in);
+        const uint2 d2 = load_tile_packed(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_dy);
+        const uint2 x1 = pack4<T>(unpack4<T>(y1) - sout[nt][mt]);
+        const uint2 dx2 = pack4<T>(unpack4<T>(d2) + du[nt][mt]);
         store_tile_packed(a.out, a.out_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, x1, a.vec_out);
         store_tile_packed(a.out, a.out_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, x2[nt][mt], a.vec_out);
         store_tile_packed(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, d1[nt][mt], a.vec_dx);
@@ -406,17 +417,14 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
       flush_tile(a.dw1, H, i, j, lane, dwF1[i][j]);
       flush_tile(a.dw2, H, i, j, lane, dwF2[i][j]);
       flush_tile(a.dw1 + (size_t)H * H, H, i, j, lane, dwG1[i][j]);
-      flush_tile(a.dw2 + (size_t)H * H, H, i, j, lane, dwG2[i][j]);
+      flush_tile(a.dw2 + (size_t)H * H, H, i, j, lane, G2_LDS ? g2acc[(i * MT + j) * 64 + lane] : dwG2[i][j]);
     }
-  if (want_db && lane < H) {
-    if (a.db1 != nullptr) {
-      unsafeAtomicAdd(a.db1 + lane, dbF1);
-      unsafeAtomicAdd(a.db1 + H + lane, dbG1);
-    }
-    if (a.db2 != nullptr) {
-      unsafeAtomicAdd(a.db2 + lane, dbF2);
-      unsafeAtomicAdd(a.db2 + H + lane, dbG2);
-    }
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    flush_db_rev(a.db1, H, i, lane, dbF1[i]);
+    flush_db_rev(a.db1 ? a.db1 + H : nullptr, H, i, lane, dbG1[i]);
+    flush_db_rev(a.db2, H, i, lane, dbF2[i]);
+    flush_db_rev(a.db2 ? a.db2 + H : nullptr, H, i, lane, dbG2[i]);
   }
 }
 
@@ -474,17 +482,22 @@ static int launch_rev_fwd(RevArgs a, hipStream_t s) {
 template <typename T, int HP>
 static int launch_rev_bwd(RevArgs a, hipStream_t s) {
   constexpr int LAYER = (HP / 16) * (HP / 32) * RFRAG;
-  const size_t lds = (size_t)8 * LAYER * 2 + (size_t)4 * HP * 4 + (size_t)4 * 4 * HP * RPITCH * 2;
+  const size_t lds = (size_t)8 * LAYER * 2 + (size_t)4 * HP * 4 + (HP > 32 ? (size_t)4 * (HP / 16) * (HP / 16) * 64 * 16 : 0);
   const int64_t chunks = (a.rows + 31) / 32;
   int64_t blocks = (chunks + 3) / 4;
-  const int64_t cap = (int64_t)rev_cus() * (lds > 80 * 1024 ? 1 : 2);
+  // the weight-gradient accumulators take most of the register file: one wave per SIMD
+  const int64_t cap = (int64_t)rev_cus();
   if (blocks > cap) blocks = cap;
-  auto kern = rev_bwd_block_k<T, HP>;
+  const void* kern = a.act == NF_ACT_GELU   ? (const void*)rev_bwd_block_k<T, HP, NF_ACT_GELU>
+                     : a.act == NF_ACT_RELU ? (const void*)rev_bwd_block_k<T, HP, NF_ACT_RELU>
+                                            : (const void*)rev_bwd_block_k<T, HP, -1>;
   if (lds > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), lds, s, a);
+  void* args[] = {(void*)&a};
+  const hipError_t e = hipLaunchKernel(kern, dim3((unsigned)blocks), dim3(256), args, lds, s);
+  if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(rev_bwd_block): %s", hipGetErrorString(e));
   return check_launch("rev_bwd_block");
 }
 
