@@ -129,3 +129,22 @@ def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 def current_stream(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
+
+
+def zeros_like_f32(*tensors):
+    """float32 zero accumulators shaped like the given tensors (``None`` stays ``None``), carved out of one
+    buffer so that a single fill kernel clears them all."""
+    live = [t for t in tensors if t is not None]
+    if not live:
+        return tuple(None for _ in tensors)
+    sizes = [(t.numel() + 3) // 4 * 4 for t in live]  # 16-byte aligned pieces
+    flat = torch.zeros(sum(sizes), dtype=torch.float32, device=live[0].device)
+    out, off, k = [], 0, 0
+    for t in tensors:
+        if t is None:
+            out.append(None)
+            continue
+        out.append(flat[off:off + t.numel()].view(t.shape))
+        off += sizes[k]
+        k += 1
+    return tuple(out)

@@ -14,8 +14,10 @@
 //             a tile); the tile is then converted and added to the gradient table (plain read-modify-write when
 //             the bin has a single slice, atomics otherwise)
 //
-// A record is the pair of corners that differ in x only: 16 bytes {row0 | row1 << 13 inside the bin, w0, w1 as
-// float32, packed 16-bit gradient pair}.  The two rows of a pair share the bin: on a dense level they are
+// A record is the pair of corners that differ in x only: 12 bytes {row0 | row1 << 13 inside the bin, w0 and w1 in
+// 19-bit fixed point (rounded to nearest: each contribution is off by at most 2^-20 |dout|), packed 16-bit gradient
+// pair}.  The records are written once and read once, 4 bytes less per record are worth more than the last bits of
+// a weight.  The two rows of a pair share the bin: on a dense level they are
 // neighbours, on a hashed level the x prime is 1 and  (x+1) ^ a  differs from  x ^ a  only below the lowest zero
 // bit of x.  When they do not (bin border, 13 trailing ones in x) the pair becomes two records with one zero weight
 // each.  The count and fill kernels apply the same rule, so their record counts agree.
@@ -34,6 +36,8 @@ namespace nf {
 constexpr int BIN_ROWS_LOG2 = 13;
 constexpr int BIN_ROWS = 1 << BIN_ROWS_LOG2;  // rows per bin (two 64-bit sums each: 128 KiB of LDS in the accumulation)
 constexpr uint32_t BIN_MASK = BIN_ROWS - 1;
+constexpr int W_BITS = 19;
+constexpr uint32_t W_MAX = (1u << W_BITS) - 1u;
 constexpr int FILL_POINTS = 512;              // points (= threads) per workgroup of count and fill
 constexpr int FILL_RECORDS = FILL_POINTS * 8; // most records a workgroup stages per level
 constexpr int ACC_THREADS = 1024;
@@ -51,7 +55,7 @@ struct BinPlan {
 };
 
 // workspace (32-bit words): hist[NB] | gmax[32] | cursor[NB] | n_tasks, pad[3] | tasks[max_tasks][4] |
-// wg_counts[workgroups][NB] | records[R][4]      (hist and gmax are cleared together)
+// wg_counts[workgroups][NB] | records[R][3]      (hist and gmax are cleared together)
 struct BinWs {
   uint32_t* hist;
   uint32_t* gmax;  // per level: largest |dout| bit pattern (15 bits)
@@ -59,7 +63,7 @@ struct BinWs {
   uint32_t* n_tasks;
   uint4* tasks;
   uint32_t* wg_counts;
-  uint4* records;
+  uint3* records;
   uint32_t max_tasks;
 };
 
@@ -69,6 +73,12 @@ __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// record = {row0 | row1 << 13 | w1[18:13] << 26,  w0 | w1[12:0] << 19,  packed gradient pair}
+__device__ __forceinline__ uint3 make_record(uint32_t row0, uint32_t row1, float w0, float w1, uint32_t packed) {
+  const uint32_t q0 = (uint32_t)(w0 * (float)W_MAX + 0.5f), q1 = (uint32_t)(w1 * (float)W_MAX + 0.5f);
+  return make_uint3(row0 | row1 << BIN_ROWS_LOG2 | (q1 >> 13) << 26, q0 | (q1 & 0x1fffu) << W_BITS, packed);
 }
 
 struct Located3 {
@@ -226,10 +236,10 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
                                                                    const uint16_t* dout, int64_t dout_stride, int64_t N,
                                                                    DevGeom g, BinPlan bp, const int64_t* primes, float scale,
                                                                    const uint32_t* wg_counts, uint32_t* cursor, uint32_t* gmax,
-                                                                   uint4* records) {
+                                                                   uint3* records) {
   extern __shared__ __align__(16) unsigned char fill_smem[];
   const int NB = bp.binbase[bp.n_levels];
-  uint4* stage = reinterpret_cast<uint4*>(fill_smem);                     // [FILL_RECORDS] records sorted by bin
+  uint3* stage = reinterpret_cast<uint3*>(fill_smem);                     // [FILL_RECORDS] records sorted by bin
   uint16_t* binid = reinterpret_cast<uint16_t*>(stage + FILL_RECORDS);    // bin (within the level) of each staged record
   uint32_t* cur = reinterpret_cast<uint32_t*>(binid + FILL_RECORDS);      // [NB] next staged position of a bin
   uint32_t* delta = cur + NB;                                             // [NB] global minus staged position
@@ -326,8 +336,7 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
         else if (nb <= AGG_MAX_BINS) pos = wave_rank(lcur, b0, valid, lane);
         else pos = valid ? atomicAdd(lcur + b0, 1u) : 0u;
         if (valid) {
-          const uint32_t rr = (r0 & BIN_MASK) | ((split ? r0 : r1) & BIN_MASK) << BIN_ROWS_LOG2;
-          stage[pos] = make_uint4(rr, __float_as_uint(w[2 * c]), split ? 0u : __float_as_uint(w[2 * c + 1]), packed);
+          stage[pos] = make_record(r0 & BIN_MASK, (split ? r0 : r1) & BIN_MASK, w[2 * c], split ? 0.0f : w[2 * c + 1], packed);
           binid[pos] = (uint16_t)b0;
         }
         if (nb > 1 && __any(valid && split)) {
@@ -336,8 +345,7 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
           if (nb <= AGG_MAX_BINS) pos1 = wave_rank(lcur, b1, on, lane);
           else pos1 = on ? atomicAdd(lcur + b1, 1u) : 0u;
           if (on) {
-            const uint32_t rr = (r1 & BIN_MASK) | (r1 & BIN_MASK) << BIN_ROWS_LOG2;
-            stage[pos1] = make_uint4(rr, __float_as_uint(w[2 * c + 1]), 0u, packed);
+            stage[pos1] = make_record(r1 & BIN_MASK, r1 & BIN_MASK, w[2 * c + 1], 0.0f, packed);
             binid[pos1] = (uint16_t)b1;
           }
         }
@@ -358,7 +366,7 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
 // accumulate
 // ---------------------------------------------------------------------------------------
 template <typename GT>
-__global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const uint4* records, const uint4* tasks,
+__global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const uint3* records, const uint4* tasks,
                                                                     const uint32_t* n_tasks, const uint32_t* gmax, float* dtable,
                                                                     DevGeom g, BinPlan bp) {
   extern __shared__ unsigned long long acc_tile[];  // [BIN_ROWS][2] fixed-point sums
@@ -380,23 +388,25 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const uint4*
     se = 30 - ex;
     se = se > 120 ? 120 : se;
   }
-  const float s_lo = nonfinite ? 0.0f : ldexpf(1.0f, se / 2), s_hi = ldexpf(1.0f, se - se / 2);  // two steps stay inside float range
+  // two steps stay inside float range; the weight decode rides on the second
+  const float s_lo = nonfinite ? 0.0f : ldexpf(1.0f, se / 2), s_hi = ldexpf(1.0f, se - se / 2) * (1.0f / (float)W_MAX);
   for (uint32_t i = tid; i < 2u * nrows; i += ACC_THREADS) acc_tile[i] = 0ull;
   lds_barrier();
   // the next round's records are loaded before this round's adds
-  uint4 q[ACC_INFLIGHT];
+  uint3 q[ACC_INFLIGHT];
 #pragma unroll
   for (int k = 0; k < ACC_INFLIGHT; ++k) {
     const uint32_t i = task.y + k * ACC_THREADS + tid;
-    q[k] = i < task.z ? records[i] : make_uint4(0u, 0u, 0u, 0u);
+    q[k] = i < task.z ? records[i] : make_uint3(0u, 0u, 0u);
   }
   for (uint32_t i0 = task.y; i0 < task.z; i0 += ACC_THREADS * ACC_INFLIGHT) {
     uint32_t slot[ACC_INFLIGHT][2];
     int32_t f[ACC_INFLIGHT][4];
 #pragma unroll
     for (int k = 0; k < ACC_INFLIGHT; ++k) {
-      const float g0 = GT::to_f32((uint16_t)(q[k].w & 0xffffu)) * s_lo, g1 = GT::to_f32((uint16_t)(q[k].w >> 16)) * s_lo;
-      const float w0 = __uint_as_float(q[k].y), w1 = __uint_as_float(q[k].z);  // records past the end: zero weights
+      const float g0 = GT::to_f32((uint16_t)(q[k].z & 0xffffu)) * s_lo, g1 = GT::to_f32((uint16_t)(q[k].z >> 16)) * s_lo;
+      // records past the end: zero weights
+      const float w0 = (float)(q[k].y & W_MAX), w1 = (float)((q[k].x >> 26) << 13 | q[k].y >> W_BITS);
       slot[k][0] = q[k].x & BIN_MASK;
       slot[k][1] = (q[k].x >> BIN_ROWS_LOG2) & BIN_MASK;
       f[k][0] = __float2int_rn(w0 * g0 * s_hi);
@@ -411,7 +421,7 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const uint4*
 #pragma unroll
     for (int k = 0; k < ACC_INFLIGHT; ++k) {
       const uint32_t i = i0 + ACC_THREADS * ACC_INFLIGHT + k * ACC_THREADS + tid;
-      q[k] = i < task.z ? records[i] : make_uint4(0u, 0u, 0u, 0u);
+      q[k] = i < task.z ? records[i] : make_uint3(0u, 0u, 0u);
     }
 #pragma unroll
     for (int k = 0; k < ACC_INFLIGHT; ++k)
@@ -485,7 +495,7 @@ static int64_t bin_ws(void* workspace, const BinPlan& bp, int64_t N, int64_t R, 
   ws->n_tasks = p + o; o += 4;
   ws->tasks = reinterpret_cast<uint4*>(p + o); o += 4 * (int64_t)max_tasks;
   ws->wg_counts = p + o; o += wg_count_words(N, NB);
-  ws->records = reinterpret_cast<uint4*>(p + o); o += 4 * R;
+  ws->records = reinterpret_cast<uint3*>(p + o); o += 3 * R;
   ws->max_tasks = max_tasks;
   return o * 4;
 }
@@ -522,7 +532,7 @@ int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const 
                      ws.tasks, NB, max_tasks);
   if (int rc = check_launch("hash_bwd_bin_offsets")) return rc;
   {
-    const size_t lds = (size_t)FILL_RECORDS * (sizeof(uint4) + sizeof(uint16_t)) + ((size_t)2 * NB + 2 * NF_MAX_LEVELS) * 4;
+    const size_t lds = (size_t)FILL_RECORDS * (sizeof(uint3) + sizeof(uint16_t)) + ((size_t)2 * NB + 2 * NF_MAX_LEVELS) * 4;
     hipError_t e = hipFuncSetAttribute((const void*)hash_bwd_bin_fill_k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     hipLaunchKernelGGL(hash_bwd_bin_fill_k, dim3(blocks), dim3(FILL_POINTS), lds, s, coords, cdt, csn, csd,
@@ -535,7 +545,7 @@ int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const 
     const void* kern = ddt == NF_F16 ? (const void*)hash_bwd_bin_accum_k<F16> : (const void*)hash_bwd_bin_accum_k<BF16>;
     hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    const uint4* rc_ = ws.records;
+    const uint3* rc_ = ws.records;
     const uint4* tk = ws.tasks;
     const uint32_t* nt = ws.n_tasks;
     const uint32_t* gm = ws.gmax;

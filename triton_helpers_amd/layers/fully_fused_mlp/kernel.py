@@ -177,10 +177,7 @@ class _fully_fused_mlp(Function):
         need_dx = ctx.needs_input_grad[0]
         dx = x.new_empty(x.shape) if need_dx else None
 
-        def acc(t: Optional[Tensor]) -> Optional[Tensor]:
-            return None if t is None else torch.zeros(t.shape, dtype=torch.float32, device=t.device)
-
-        dw_in, db_in, dw_out, db_out, dw_hid, db_hid = (acc(t) for t in (w_in, b_in, w_out, b_out, w_hid, b_hid))
+        dw_in, db_in, dw_out, db_out, dw_hid, db_hid = _lib.zeros_like_f32(w_in, b_in, w_out, b_out, w_hid, b_hid)
         lib = _lib.load()
         rc = lib.nf_mlp_bwd(
             x2.data_ptr(), x2.stride(0), do2.data_ptr(), do2.stride(0),

@@ -86,10 +86,7 @@ class _reversible_mlp(Function):
         dx = y.new_empty(y.shape)
         x_rec = y.new_empty(y.shape)
 
-        def acc(t: Optional[Tensor]) -> Optional[Tensor]:
-            return None if t is None else torch.zeros(t.shape, dtype=torch.float32, device=t.device)
-
-        dw1, db1, dw2, db2 = (acc(t) for t in (w1, b1, w2, b2))
+        dw1, db1, dw2, db2 = _lib.zeros_like_f32(w1, b1, w2, b2)
         lib = _lib.load()
         rc = lib.nf_revmlp_bwd(
             y2.data_ptr(), y2.stride(0), dy2.data_ptr(), dy2.stride(0), dx.data_ptr(), 2 * H, x_rec.data_ptr(), 2 * H,
