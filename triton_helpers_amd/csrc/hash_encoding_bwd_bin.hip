@@ -38,7 +38,7 @@ constexpr int BIN_ROWS = 1 << BIN_ROWS_LOG2;  // rows per bin (two 64-bit sums e
 constexpr uint32_t BIN_MASK = BIN_ROWS - 1;
 constexpr int W_BITS = 19;
 constexpr uint32_t W_MAX = (1u << W_BITS) - 1u;
-constexpr int FILL_POINTS = 512;              // points (= threads) per workgroup of count and fill
+constexpr int FILL_POINTS = 1024;              // points (= threads) per workgroup of count and fill
 constexpr int FILL_RECORDS = FILL_POINTS * 8; // most records a workgroup stages per level
 constexpr int ACC_THREADS = 1024;
 constexpr int ACC_INFLIGHT = 8;               // records in flight per thread
