@@ -9,8 +9,10 @@ gradient, float32 table gradient.  One step = forward launch + clearing the floa
 gradient table + backward launch(es), inputs resident in HBM.  ``value`` is Mpoints/s.
 
 Extra objects in the same line:
-  roofline      the dominant kernel of the step (longest average launch), algorithmic bytes
-                per launch / measured launch time against the 8 TB/s HBM peak;
+  roofline      the dominant kernel of the step (the forward gather kernel: the backward is a
+                chain of five shorter kernels), algorithmic bytes per launch / launch time measured
+                here with events against the 8 TB/s HBM peak; ``traffic`` is that kernel's HBM
+                traffic from the FETCH_SIZE / WRITE_SIZE counters of a profiler run;
   cpu_baseline  the CPU oracle (a port of the reference's PyTorch path) timed on this host
                 on a 65536-point sample of the same workload;
   workloads     the other BASELINE configs (fused MLP, reversible MLP, end-to-end step) with
@@ -40,6 +42,9 @@ N_POINTS = 2**20
 # algorithmic bytes per point: fwd = 4D + L*2^D*F*2 + L*F*2 ; bwd = 4D + L*F*2 + L*2^D*F*4
 FWD_BYTES_PER_POINT = 4 * D + L * 8 * F * 2 + L * F * 2  # 588
 BWD_BYTES_PER_POINT = 4 * D + L * F * 2 + L * 8 * F * 4  # 1100
+# HBM bytes per forward launch at N = 2^20 measured with rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a 256 MiB copy
+# kernel gives for that counter) + WRITE_SIZE (x1.0): 1694 MB + 67 MB
+FWD_TRAFFIC_BYTES = 1.761e9
 
 
 def event_times(fn, reps):
@@ -250,13 +255,11 @@ def main():
     torch.cuda.set_device(0)
 
     h = bench_hash(args.steps, args.warmup)
-    kernels = {
-        "hash_fwd": (h["t_fwd"], FWD_BYTES_PER_POINT * N_POINTS),
-        "hash_bwd": (h["t_bwd"], BWD_BYTES_PER_POINT * N_POINTS),
-    }
-    dom = max(kernels, key=lambda k: kernels[k][0])
-    dom_ms, dom_bytes = kernels[dom]
+    # The forward is one kernel (hash_fwd_tiled_k); the backward is zero + count + offsets + fill + accumulate, each
+    # shorter than the forward kernel.
+    dom, dom_ms, dom_bytes = "hash_fwd_tiled_k", h["t_fwd"], FWD_BYTES_PER_POINT * N_POINTS
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    bwd_achieved = BWD_BYTES_PER_POINT * N_POINTS / (h["t_bwd"] * 1e-3) / 1e9
     step_bytes = (FWD_BYTES_PER_POINT + BWD_BYTES_PER_POINT) * N_POINTS + h["E"] * F * 4
     out = {
         "metric": "Mpoints/s fwd+bwd: hash-enc+fused MLP @2^20 pts; % HBM / MFMA peak",
@@ -278,10 +281,11 @@ def main():
         },
         "roofline": {
             "bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "frac": achieved / HBM_PEAK_GBS, "traffic": FWD_TRAFFIC_BYTES,
             "launch_ms": dom_ms, "algorithmic_bytes_per_launch": dom_bytes,
         },
-        "kernels_ms": {"hash_fwd": h["t_fwd"], "grad_zero_fill": h["t_zero"], "hash_bwd": h["t_bwd"]},
+        "phases_ms": {"hash_fwd": h["t_fwd"], "grad_zero_fill": h["t_zero"], "hash_bwd": h["t_bwd"]},
+        "bwd_roofline_frac": bwd_achieved / HBM_PEAK_GBS,
         "step_roofline_frac": step_bytes / (h["ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "autograd_ms_per_step": h["ms_autograd"],
     }
