@@ -161,8 +161,9 @@ def test_backward_vs_oracle(N, D, F, T, L, lo, hi, scale, do_dtype, flags, monke
         (45000, 2**12, 4, 8, 64),       # hashed levels smaller than a tile
     ],
 )
-def test_backward_lds_tile_path(N, T, L, lo, hi, do_dtype):
-    """The LDS-tile backward (plan + scan kernels) against the oracle and against the scattered-atomic kernel."""
+@pytest.mark.parametrize("variant", [0, 4])  # 0: binned records, 4: bit-planes (NF_HASH_FORCE_PLANES)
+def test_backward_lds_tile_path(N, T, L, lo, hi, do_dtype, variant):
+    """Both LDS-tile backwards against the oracle and against the scattered-atomic kernel."""
     hk = _hk()
     torch.manual_seed(3)
     x = torch.rand(N, 3)
@@ -172,7 +173,7 @@ def test_backward_lds_tile_path(N, T, L, lo, hi, do_dtype):
     do = torch.randn(N, L * 2).to(do_dtype)
     do[100:200] = 0  # rows with no upstream gradient are skipped
     want = O.encode_backward(x, do, E, 2, None, T, L, lo, hi)
-    hk._FLAGS = 0
+    hk._FLAGS = variant
     got = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, 2, None, T, lo, hi, L)
     hk._FLAGS = 2
     try:
@@ -181,6 +182,47 @@ def test_backward_lds_tile_path(N, T, L, lo, hi, do_dtype):
         hk._FLAGS = 0
     torch.testing.assert_close(got.cpu(), want, rtol=1e-3, atol=1e-4)
     torch.testing.assert_close(got, ref, rtol=1e-3, atol=1e-4)
+
+
+def test_backward_binned_clustered_points():
+    """Clustered input: a few cells receive everything, so their bins are cut into several accumulation tasks
+    (atomic flush), and x = 8191 sits on a bin border of the dense levels / has 13 trailing ones on hashed levels, so
+    corner pairs are split into two records."""
+    hk = _hk()
+    torch.manual_seed(5)
+    N, T, L, lo, hi = 150000, 2**19, 16, 16, 16384
+    x = torch.rand(N, 3)
+    x[: N // 2] = torch.tensor([0.3, 0.6, 0.9]) + 1e-4 * torch.rand(N // 2, 3)       # one cell on the coarse levels
+    x[N // 2: N // 2 + 20000, 0] = (8191.0 + 0.5 * torch.rand(20000)) / 16384.0       # x cell 8191 at resolution 16384
+    E = O.level_row_offsets(L, T, 3, lo, hi)[-1]
+    do = torch.randn(N, L * 2).half()
+    want = O.encode_backward(x, do, E, 2, None, T, L, lo, hi)
+    got = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, 2, None, T, lo, hi, L)
+    # sums of up to 75000 terms: compare with a tolerance scaled to the largest row
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-3, atol=1e-4 * float(want.abs().max()))
+    # bins cut into several tasks meet in float atomics, so two runs agree to rounding only
+    again = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, 2, None, T, lo, hi, L)
+    torch.testing.assert_close(got, again, rtol=1e-5, atol=1e-6 * float(want.abs().max()))
+
+
+def test_backward_binned_nonfinite_gradient():
+    """An inf in one level's upstream gradient turns the rows that level touches into nan and leaves the other
+    levels exact."""
+    hk = _hk()
+    torch.manual_seed(6)
+    N, T, L, lo, hi = 40000, 2**16, 4, 16, 256
+    x = torch.rand(N, 3)
+    E = O.level_row_offsets(L, T, 3, lo, hi)[-1]
+    offs = O.level_row_offsets(L, T, 3, lo, hi)
+    do = torch.randn(N, L * 2).half()
+    clean = O.encode_backward(x, do, E, 2, None, T, L, lo, hi)
+    do[123, 2 * 2] = float("inf")  # level 2, feature 0
+    got = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, 2, None, T, lo, hi, L).cpu()
+    lvl2 = slice(offs[2], offs[3])
+    assert not torch.isfinite(got[lvl2]).all()
+    keep = torch.ones(E, dtype=torch.bool)
+    keep[lvl2] = False
+    torch.testing.assert_close(got[keep], clean[keep], rtol=1e-3, atol=1e-4)
 
 
 def test_autograd_round_trip_fp16_table():

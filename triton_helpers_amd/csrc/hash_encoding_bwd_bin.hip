@@ -24,8 +24,8 @@
 //
 // Integer accumulation: fill also finds max |dout| per level; with 2^e the power of two above it, a contribution
 // w * g is accumulated as round(w * g * 2^(30 - e)), below 2^30 in magnitude, so a task's records cannot
-// overflow 64 bits, the rounding is 2^-30 of the level's largest gradient per contribution, and the sum does
-// not depend on the order of the records.  A level whose gradient holds an inf or a nan gets nan in every row
+// overflow 64 bits, the rounding is 2^-30 of the level's largest gradient per contribution, and a task's sum does
+// not depend on the order of its records (tasks of a split bin still meet in float atomics).  A level whose gradient holds an inf or a nan gets nan in every row
 // it touches.
 //
 // Arithmetic (cell, corner rows, weights) is the forward's, see hash_encoding.hip.
