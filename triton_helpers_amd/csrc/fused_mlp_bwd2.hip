@@ -107,11 +107,35 @@ __device__ __forceinline__ Frag load_chain(const uint16_t* base, int64_t stride,
   return load_rows_frag_chain(base, stride, row0, rows, width, kc, lane, vec_ok);
 }
 
+// 16-row tiles per chunk.
+#ifndef NF_BWD2_NT
+#define NF_BWD2_NT 4
+#endif
 // Workgroups per CU the ReLU kernel is compiled for.
 #ifndef NF_BWD2_OCC
 #define NF_BWD2_OCC 1
 #endif
-template <typename T, int KIN, int HP, int OUTP, bool RELU, bool FAST>
+// acc[nt][mt] = bias (or 0) + W(frags) * in[nt][kc], one weight fragment read per NT products
+template <typename T, int NT, int MT, int KC>
+__device__ __forceinline__ void layer_nt(f32x4_t (&acc)[NT][4], const Frag (&in)[NT][2], const uint16_t* frags, const float* bias,
+                                         int lane) {
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    f32x4_t b4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (bias != nullptr) b4 = *reinterpret_cast<const f32x4_t*>(bias + 16 * mt + 4 * (lane >> 4));
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[nt][mt] = b4;
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc) {
+      const Frag w = lds_frag(frags, mt * KC + kc, lane);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[nt][mt] = mfma16<T>(w, in[nt][kc], acc[nt][mt]);
+    }
+  }
+}
+
+// NT: 16-row tiles per chunk (2 or 4).  Four give the scheduler two independent 32-row groups to interleave.
+template <typename T, int KIN, int HP, int OUTP, bool RELU, bool FAST, int NT>
 __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArgs a) {
   constexpr int KC_IN = KIN / 32, KC_H = HP / 32, MT_H = HP / 16, MT_I = KIN / 16, MT_O = OUTP / 16;
   constexpr int KC_O = (OUTP + 31) / 32;
@@ -156,42 +180,43 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
   }
   const Frag sel[2] = {sel_frag<T>(0, lane), sel_frag<T>(1, lane)};
 
-  const int64_t n_chunks = (a.rows + 31) / 32;
+  constexpr int ROWS = 16 * NT;  // rows per chunk: NT / 2 independent groups of 32 rows
+  const int64_t n_chunks = (a.rows + ROWS - 1) / ROWS;
   const int64_t wave_stride = (int64_t)gridDim.x * 4;
   const int64_t first_chunk = (int64_t)blockIdx.x * 4 + wave;
-  Frag nx[2][KC_IN], ndy[2][KC_O];
+  Frag nx[NT][KC_IN], ndy[NT][KC_O];
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt) {
+  for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
     for (int kc = 0; kc < KC_IN; ++kc)
-      nx[nt][kc] = load_chain<FAST>(a.x, a.x_stride, first_chunk * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+      nx[nt][kc] = load_chain<FAST>(a.x, a.x_stride, first_chunk * ROWS + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
 #pragma unroll
     for (int kc = 0; kc < KC_O; ++kc)
-      ndy[nt][kc] = load_chain<FAST>(a.dy, a.dy_stride, first_chunk * 32 + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
+      ndy[nt][kc] = load_chain<FAST>(a.dy, a.dy_stride, first_chunk * ROWS + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
   }
 
   for (int64_t chunk = first_chunk; chunk < n_chunks; chunk += wave_stride) {
-    const int64_t row0 = chunk * 32;
-    Frag in[2][2], h1[2][2], h2[2][2], g1[2][2], g2[2][2], dz[2][2];
-    f32x4_t acc[2][4];
+    const int64_t row0 = chunk * ROWS;
+    Frag in[NT][2], h1[NT][2], h2[NT][2], g1[NT][2], g2[NT][2], dz[NT][2];
+    f32x4_t acc[NT][4];
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
+    for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
       for (int kc = 0; kc < KC_IN; ++kc) {
         in[nt][kc] = nx[nt][kc];
-        nx[nt][kc] = load_chain<FAST>(a.x, a.x_stride, (chunk + wave_stride) * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+        nx[nt][kc] = load_chain<FAST>(a.x, a.x_stride, (chunk + wave_stride) * ROWS + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
       }
 #pragma unroll
       for (int kc = 0; kc < KC_O; ++kc) {
         dz[nt][kc] = ndy[nt][kc];
-        ndy[nt][kc] = load_chain<FAST>(a.dy, a.dy_stride, (chunk + wave_stride) * 32 + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
+        ndy[nt][kc] = load_chain<FAST>(a.dy, a.dy_stride, (chunk + wave_stride) * ROWS + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
       }
     }
 
     // ---- forward recompute: h1 = act(W_in x + b), h2 = act(W_hid h1 + b) ----
-    layer_mma<T, MT_H, KC_IN>(acc, in, f_in, bias_in, lane);
+    layer_nt<T, NT, MT_H, KC_IN>(acc, in, f_in, bias_in, lane);
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+    for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
       for (int mt = 0; mt < MT_H; ++mt) {
         uint32_t p01, p23;
@@ -208,9 +233,9 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
         h1[nt][mt >> 1].w[2 * (mt & 1)] = p01;
         h1[nt][mt >> 1].w[2 * (mt & 1) + 1] = p23;
       }
-    layer_mma<T, MT_H, KC_H>(acc, h1, f_hid, bias_hid, lane);
+    layer_nt<T, NT, MT_H, KC_H>(acc, h1, f_hid, bias_hid, lane);
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+    for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
       for (int mt = 0; mt < MT_H; ++mt) {
         uint32_t p01, p23;
@@ -229,33 +254,24 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
       }
 
     // ---- output layer: dW_out += dy^T h2, db_out += sum dy ; dh2 = W_out^T dy ----
-    {
+#pragma unroll
+    for (int p = 0; p < NT / 2; ++p) {
       Frag hb[MT_H];
 #pragma unroll
-      for (int j = 0; j < MT_H; ++j) hb[j] = transpose_tile<T>(h2[0][j >> 1], h2[1][j >> 1], sel[j & 1]);
+      for (int j = 0; j < MT_H; ++j) hb[j] = transpose_tile<T>(h2[2 * p][j >> 1], h2[2 * p + 1][j >> 1], sel[j & 1]);
 #pragma unroll
       for (int i = 0; i < MT_O; ++i) {
-        const Frag da = transpose_tile<T>(dz[0][i >> 1], dz[1][i >> 1], sel[i & 1]);
+        const Frag da = transpose_tile<T>(dz[2 * p][i >> 1], dz[2 * p + 1][i >> 1], sel[i & 1]);
 #pragma unroll
         for (int j = 0; j < MT_H; ++j) dw_out[i][j] = mfma16<T>(da, hb[j], dw_out[i][j]);
 #pragma unroll
         for (int q = 0; q < 4; ++q) db_out[i] = dot2_ones<T>(da.w[q], db_out[i]);
       }
     }
-#pragma unroll
-    for (int mt = 0; mt < MT_H; ++mt) {
-      acc[0][mt] = zero4;
-      acc[1][mt] = zero4;
-#pragma unroll
-      for (int kc = 0; kc < KC_O; ++kc) {
-        const Frag wa = lds_frag(t_out, mt * KC_O + kc, lane);
-        acc[0][mt] = mfma16<T>(wa, dz[0][kc], acc[0][mt]);
-        acc[1][mt] = mfma16<T>(wa, dz[1][kc], acc[1][mt]);
-      }
-    }
+    layer_nt<T, NT, MT_H, KC_O>(acc, dz, t_out, nullptr, lane);
     // ---- hidden layer: dz2 = dh2 * act'(z2) ; dW_hid += dz2^T h1 ; dh1 = W_hid^T dz2 ----
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+    for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
       for (int mt = 0; mt < MT_H; ++mt) {
         uint32_t p01, p23;
@@ -268,34 +284,24 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
         dz[nt][mt >> 1].w[2 * (mt & 1)] = p01;
         dz[nt][mt >> 1].w[2 * (mt & 1) + 1] = p23;
       }
-    {
+#pragma unroll
+    for (int p = 0; p < NT / 2; ++p) {
       Frag hb[MT_H];
 #pragma unroll
-      for (int j = 0; j < MT_H; ++j) hb[j] = transpose_tile<T>(h1[0][j >> 1], h1[1][j >> 1], sel[j & 1]);
+      for (int j = 0; j < MT_H; ++j) hb[j] = transpose_tile<T>(h1[2 * p][j >> 1], h1[2 * p + 1][j >> 1], sel[j & 1]);
 #pragma unroll
       for (int i = 0; i < MT_H; ++i) {
-        const Frag da = transpose_tile<T>(dz[0][i >> 1], dz[1][i >> 1], sel[i & 1]);
+        const Frag da = transpose_tile<T>(dz[2 * p][i >> 1], dz[2 * p + 1][i >> 1], sel[i & 1]);
 #pragma unroll
         for (int j = 0; j < MT_H; ++j) dw_hid[i][j] = mfma16<T>(da, hb[j], dw_hid[i][j]);
 #pragma unroll
         for (int q = 0; q < 4; ++q) db_hid[i] = dot2_ones<T>(da.w[q], db_hid[i]);
       }
     }
-#pragma unroll
-    for (int mt = 0; mt < MT_H; ++mt) {
-      f32x4_t o0 = zero4, o1 = zero4;
-#pragma unroll
-      for (int kc = 0; kc < KC_H; ++kc) {
-        const Frag wa = lds_frag(t_hid, mt * KC_H + kc, lane);
-        o0 = mfma16<T>(wa, dz[0][kc], o0);
-        o1 = mfma16<T>(wa, dz[1][kc], o1);
-      }
-      acc[0][mt] = o0;
-      acc[1][mt] = o1;
-    }
+    layer_nt<T, NT, MT_H, KC_H>(acc, dz, t_hid, nullptr, lane);
     // ---- input layer: dz1 = dh1 * act'(z1) ; dW_in += dz1^T x ; dx = W_in^T dz1 ----
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+    for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
       for (int mt = 0; mt < MT_H; ++mt) {
         uint32_t p01, p23;
@@ -308,13 +314,14 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
         dz[nt][mt >> 1].w[2 * (mt & 1)] = p01;
         dz[nt][mt >> 1].w[2 * (mt & 1) + 1] = p23;
       }
-    {
+#pragma unroll
+    for (int p = 0; p < NT / 2; ++p) {
       Frag xb[MT_I];
 #pragma unroll
-      for (int j = 0; j < MT_I; ++j) xb[j] = transpose_tile<T>(in[0][j >> 1], in[1][j >> 1], sel[j & 1]);
+      for (int j = 0; j < MT_I; ++j) xb[j] = transpose_tile<T>(in[2 * p][j >> 1], in[2 * p + 1][j >> 1], sel[j & 1]);
 #pragma unroll
       for (int i = 0; i < MT_H; ++i) {
-        const Frag da = transpose_tile<T>(dz[0][i >> 1], dz[1][i >> 1], sel[i & 1]);
+        const Frag da = transpose_tile<T>(dz[2 * p][i >> 1], dz[2 * p + 1][i >> 1], sel[i & 1]);
 #pragma unroll
         for (int j = 0; j < MT_I; ++j) dw_in[i][j] = mfma16<T>(da, xb[j], dw_in[i][j]);
 #pragma unroll
@@ -322,23 +329,14 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
       }
     }
     if (a.dx != nullptr) {
+      layer_nt<T, NT, MT_I, KC_H>(acc, dz, t_in, nullptr, lane);
 #pragma unroll
-      for (int mt = 0; mt < MT_I; ++mt) {
-        f32x4_t o0 = zero4, o1 = zero4;
+      for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int kc = 0; kc < KC_H; ++kc) {
-          const Frag wa = lds_frag(t_in, mt * KC_H + kc, lane);
-          o0 = mfma16<T>(wa, dz[0][kc], o0);
-          o1 = mfma16<T>(wa, dz[1][kc], o1);
+        for (int mt = 0; mt < MT_I; ++mt) {
+          if (FAST) store_rows_tile_fast<T>(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, a.d_in, mt, lane, acc[nt][mt]);
+          else store_rows_tile<T>(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, a.d_in, mt, lane, acc[nt][mt], a.dx_vec);
         }
-        if (FAST) {
-          store_rows_tile_fast<T>(a.dx, a.dx_stride, row0, a.rows, a.d_in, mt, lane, o0);
-          store_rows_tile_fast<T>(a.dx, a.dx_stride, row0 + 16, a.rows, a.d_in, mt, lane, o1);
-        } else {
-          store_rows_tile<T>(a.dx, a.dx_stride, row0, a.rows, a.d_in, mt, lane, o0, a.dx_vec);
-          store_rows_tile<T>(a.dx, a.dx_stride, row0 + 16, a.rows, a.d_in, mt, lane, o1, a.dx_vec);
-        }
-      }
     }
   }
 
@@ -419,7 +417,10 @@ static int launch2(const MlpArgs& a0, hipStream_t s) {
   // chain-order loads move 8 bytes at a time
   a.x_vec = ((uintptr_t)a.x % 8 == 0) && (a.x_stride % 4 == 0);
   a.dy_vec = ((uintptr_t)a.dy % 8 == 0) && (a.dy_stride % 4 == 0);
-  const int64_t chunks = (a.rows + 31) / 32;
+  // four tiles only where the registers allow it: ReLU (no gate images) and the narrow input / output shapes
+  constexpr int NT = (KIN == 32 && OUTP == 16) ? NF_BWD2_NT : 2;
+  const int nt = a.act == NF_ACT_RELU ? NT : 2;
+  const int64_t chunks = (a.rows + 16 * nt - 1) / (16 * nt);
   int64_t blocks = (chunks + 3) / 4;
   const int64_t cap = (int64_t)device_cus() * (a.act == NF_ACT_RELU ? NF_BWD2_OCC : 1);
   if (blocks > cap) blocks = cap;
@@ -427,9 +428,9 @@ static int launch2(const MlpArgs& a0, hipStream_t s) {
                     (a.dx == nullptr || ((uintptr_t)a.dx % 8 == 0 && a.dx_stride % 4 == 0));
   const void* kern;
   if (a.act == NF_ACT_RELU)
-    kern = fast ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, true> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, false>;
+    kern = fast ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, true, NT> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, false, NT>;
   else
-    kern = fast ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false, true> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false, false>;
+    kern = fast ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false, true, 2> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false, false, 2>;
   void* args[] = {(void*)&a};
   const hipError_t e = hipLaunchKernel(kern, dim3((unsigned)blocks), dim3(256), args, LDS, s);
   if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(mlp_bwd2): %s", hipGetErrorString(e));

@@ -203,10 +203,10 @@ __global__ __launch_bounds__(768) void rev_fwd_k(RevArgs a) {
 template <int ACT>
 __device__ __forceinline__ void act_both(float z, int act, float& h, float& g) {
   if (ACT == NF_ACT_GELU) {
-    float e;
-    const float cdf = normal_cdf(z, &e);
+    float pdf;
+    const float cdf = normal_cdf_pdf(z, &pdf);
     h = z * cdf;
-    g = cdf + z * (0.3989422804014327f * e);
+    g = cdf + z * pdf;
   } else if (ACT == NF_ACT_RELU) {
     h = fmaxf(z, 0.0f);
     g = z > 0.0f ? 1.0f : 0.0f;
