@@ -30,7 +30,8 @@ __device__ __forceinline__ void stage_bias(float* dst, const uint16_t* b, int n_
   for (int i = tid; i < n_pad; i += nthreads) dst[i] = (b != nullptr && i < n_valid) ? T::to_f32(b[i]) : 0.0f;
 }
 
-// acc[nt][mt] = bias + W(frags) * in[nt][kc]
+// acc[nt][mt] = bias + W(frags) * in[nt][kc]; K chunks outermost, so that the products into one accumulator tile are
+// 2 * MT instructions apart
 template <typename T, int MT, int KC>
 __device__ __forceinline__ void layer_mma(f32x4_t (&acc)[2][4], const Frag (&in)[2][2], const uint16_t* frags,
                                           const float* bias, int lane) {
@@ -39,13 +40,15 @@ __device__ __forceinline__ void layer_mma(f32x4_t (&acc)[2][4], const Frag (&in)
     const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(bias + 16 * mt + 4 * (lane >> 4));
     acc[0][mt] = b4;
     acc[1][mt] = b4;
+  }
 #pragma unroll
-    for (int kc = 0; kc < KC; ++kc) {
+  for (int kc = 0; kc < KC; ++kc)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
       const Frag a = lds_frag(frags, mt * KC + kc, lane);
       acc[0][mt] = mfma16<T>(a, in[0][kc], acc[0][mt]);
       acc[1][mt] = mfma16<T>(a, in[1][kc], acc[1][mt]);
     }
-  }
 }
 
 // Park an accumulator-layout tile (lane (n,g): features 16*mt + 4*g + r of row 16*nt + n) into a

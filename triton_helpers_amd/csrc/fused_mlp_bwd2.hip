@@ -115,7 +115,8 @@ __device__ __forceinline__ Frag load_chain(const uint16_t* base, int64_t stride,
 #ifndef NF_BWD2_OCC
 #define NF_BWD2_OCC 1
 #endif
-// acc[nt][mt] = bias (or 0) + W(frags) * in[nt][kc], one weight fragment read per NT products
+// acc[nt][mt] = bias (or 0) + W(frags) * in[nt][kc], one weight fragment read per NT products; K chunks outermost, so
+// that the products into one accumulator tile are MT * NT instructions apart
 template <typename T, int NT, int MT, int KC>
 __device__ __forceinline__ void layer_nt(f32x4_t (&acc)[NT][4], const Frag (&in)[NT][2], const uint16_t* frags, const float* bias,
                                          int lane) {
@@ -125,13 +126,15 @@ __device__ __forceinline__ void layer_nt(f32x4_t (&acc)[NT][4], const Frag (&in)
     if (bias != nullptr) b4 = *reinterpret_cast<const f32x4_t*>(bias + 16 * mt + 4 * (lane >> 4));
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[nt][mt] = b4;
+  }
 #pragma unroll
-    for (int kc = 0; kc < KC; ++kc) {
+  for (int kc = 0; kc < KC; ++kc)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
       const Frag w = lds_frag(frags, mt * KC + kc, lane);
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) acc[nt][mt] = mfma16<T>(w, in[nt][kc], acc[nt][mt]);
     }
-  }
 }
 
 // NT: 16-row tiles per chunk (2 or 4).  Four give the scheduler two independent 32-row groups to interleave.

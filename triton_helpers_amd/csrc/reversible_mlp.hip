@@ -94,6 +94,7 @@ __device__ __forceinline__ void tiles_to_frags(const uint2 (&p)[2][4], Frag (&f)
     }
 }
 
+// K chunks outermost: the two products into one accumulator tile are MT * 2 instructions apart.
 template <typename T, int MT, int KC>
 __device__ __forceinline__ void rev_layer(f32x4_t (&acc)[2][4], const Frag (&in)[2][2], const uint16_t* frags, const float* bias,
                                           int lane) {
@@ -103,13 +104,15 @@ __device__ __forceinline__ void rev_layer(f32x4_t (&acc)[2][4], const Frag (&in)
     if (bias != nullptr) b4 = *reinterpret_cast<const f32x4_t*>(bias + 16 * mt + 4 * (lane >> 4));
     acc[0][mt] = b4;
     acc[1][mt] = b4;
+  }
 #pragma unroll
-    for (int kc = 0; kc < KC; ++kc) {
+  for (int kc = 0; kc < KC; ++kc)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
       const Frag a = lds_frag(frags, mt * KC + kc, lane);
       acc[0][mt] = mfma16<T>(a, in[0][kc], acc[0][mt]);
       acc[1][mt] = mfma16<T>(a, in[1][kc], acc[1][mt]);
     }
-  }
 }
 
 template <typename T>
@@ -364,11 +367,39 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
   const int64_t n_chunks = (a.rows + 31) / 32;
   for (int64_t chunk = (int64_t)blockIdx.x * 4 + wave; chunk < n_chunks; chunk += (int64_t)gridDim.x * 4) {
     const int64_t row0 = chunk * 32;
-    // Each half of y and dy is loaded where it is used (and again for the final residual adds, from L2) rather
-    // than held across the two sub-MLPs: registers are the scarce resource here.
+    // The halves of y and dy that a sub-MLP's residual adds need are requested before that sub-MLP runs, so their
+    // latency hides behind its products; nothing is held across both sub-MLPs (registers are the scarce resource).
     uint2 x2[2][4], d1[2][4];
     f32x4_t sout[2][4], du[2][4];
     {
+      uint2 y1[2][4], d2[2][4], y2[2][4], dy1[2][4];
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          y1[nt][mt] = load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in);
+          d2[nt][mt] = load_tile_packed(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_dy);
+        }
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          y2[nt][mt] = load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_in);
+          dy1[nt][mt] = load_tile_packed(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_dy);
+        }
+      // ---- G:  y2 = x2 + G(y1)  =>  x2 = y2 - G(y1),  dy1 += (dG/dy1)^T dy2
+      sub_backward<T, MT, KC, ACT>(y1, d2, sout, du, dwG1, dwG2, g2acc, dbG1, dbG2, fw + 2 * LAYER, fw + 3 * LAYER,
+                                   tw + 2 * LAYER, tw + 3 * LAYER, bias + 2 * HP, bias + 3 * HP, sel, act, lane);
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          x2[nt][mt] = pack4<T>(unpack4<T>(y2[nt][mt]) - sout[nt][mt]);
+          d1[nt][mt] = pack4<T>(unpack4<T>(dy1[nt][mt]) + du[nt][mt]);
+        }
+    }
+    {
+      // the other halves again (L2 hits), in flight during F
       uint2 y1[2][4], d2[2][4];
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
@@ -377,35 +408,21 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
           y1[nt][mt] = load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in);
           d2[nt][mt] = load_tile_packed(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_dy);
         }
-      // ---- G:  y2 = x2 + G(y1)  =>  x2 = y2 - G(y1),  dy1 += (dG/dy1)^T dy2
-      sub_backward<T, MT, KC, ACT>(y1, d2, sout, du, dwG1, dwG2, g2acc, dbG1, dbG2, fw + 2 * LAYER, fw + 3 * LAYER,
-                                   tw + 2 * LAYER, tw + 3 * LAYER, bias + 2 * HP, bias + 3 * HP, sel, act, lane);
+      // ---- F:  y1 = x1 + F(x2)  =>  x1 = y1 - F(x2),  dx2 = dy2 + (dF/dx2)^T dy1
+      sub_backward<T, MT, KC, ACT>(x2, d1, sout, du, dwF1, dwF2, nullptr, dbF1, dbF2, fw, fw + LAYER, tw, tw + LAYER, bias,
+                                   bias + HP, sel, act, lane);
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const uint2 x1 = pack4<T>(unpack4<T>(y1[nt][mt]) - sout[nt][mt]);
+          const uint2 dx2 = pack4<T>(unpack4<T>(d2[nt][mt]) + du[nt][mt]);
+          store_tile_packed(a.out, a.out_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, x1, a.vec_out);
+          store_tile_packed(a.out, a.out_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, x2[nt][mt], a.vec_out);
+          store_tile_packed(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, d1[nt][mt], a.vec_dx);
+          store_tile_packed(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, dx2, a.vec_dx);
+        }
     }
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const uint2 y2 = load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_in);
-        const uint2 dy1 = load_tile_packed(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_dy);
-        x2[nt][mt] = pack4<T>(unpack4<T>(y2) - sout[nt][mt]);
-        d1[nt][mt] = pack4<T>(unpack4<T>(dy1) + du[nt][mt]);
-      }
-    // ---- F:  y1 = x1 + F(x2)  =>  x1 = y1 - F(x2),  dx2 = dy2 + (dF/dx2)^T dy1
-    sub_backward<T, MT, KC, ACT>(x2, d1, sout, du, dwF1, dwF2, nullptr, dbF1, dbF2, fw, fw + LAYER, tw, tw + LAYER, bias,
-                                 bias + HP, sel, act, lane);
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const uint2 y1 = load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in);
-        const uint2 d2 = load_tile_packed(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_dy);
-        const uint2 x1 = pack4<T>(unpack4<T>(y1) - sout[nt][mt]);
-        const uint2 dx2 = pack4<T>(unpack4<T>(d2) + du[nt][mt]);
-        store_tile_packed(a.out, a.out_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, x1, a.vec_out);
-        store_tile_packed(a.out, a.out_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, x2[nt][mt], a.vec_out);
-        store_tile_packed(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, d1[nt][mt], a.vec_dx);
-        store_tile_packed(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, dx2, a.vec_dx);
-      }
   }
 
   // ---- weight gradients: every wave adds its float32 accumulators (64-byte coalesced atomics) ----
