@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define NF_ABI_VERSION 2
+#define NF_ABI_VERSION 3
 
 /* element types */
 enum { NF_F32 = 0, NF_F16 = 1, NF_BF16 = 2 };
@@ -93,10 +93,11 @@ int nf_hash_encode_bwd(const void* coords, int coords_dtype, int64_t coords_stri
                        const nf_hash_geom* geom, const int64_t* primes, float scale, void* workspace,
                        int64_t workspace_bytes, int flags, void* stream);
 
-/* Scratch bytes nf_hash_encode_bwd can use for this call shape; 0 when the workspace would not be used.
+/* Scratch bytes nf_hash_encode_bwd can use for this call shape and these flags (NF_HASH_FORCE_PLANES gives the
+ * size of the smaller variant); 0 when the workspace would not be used.
  * (No counterpart in the reference: its backward allocates nothing besides the gradient table,
  * triton_helpers/layers/hash_encoding/kernel.py:636.) */
-int64_t nf_hash_encode_bwd_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype);
+int64_t nf_hash_encode_bwd_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype, int flags);
 
 /* Level-local table rows of all 2^D corners: out_rows [n_points, L, 2^D] int64, and
  * (optional, may be NULL) the interpolation weights out_w [n_points, L, 2^D] float32. */

@@ -388,10 +388,11 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
   }
 }
 
-extern "C" int64_t nf_hash_encode_bwd_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype) {
-  if (geom == nullptr || n_points < SCAN_MIN_POINTS) return 0;
-  const int64_t bin = bwd_bin_workspace_bytes(n_points, geom, dout_dtype);
+extern "C" int64_t nf_hash_encode_bwd_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype, int flags) {
+  if (geom == nullptr || n_points < SCAN_MIN_POINTS || (flags & (NF_HASH_FORCE_GENERIC | NF_HASH_FORCE_ATOMIC))) return 0;
   const int64_t scan = bwd_scan_workspace_bytes(n_points, geom, dout_dtype);
+  if (flags & NF_HASH_FORCE_PLANES) return scan;
+  const int64_t bin = bwd_bin_workspace_bytes(n_points, geom, dout_dtype);
   return bin > scan ? bin : scan;
 }
 

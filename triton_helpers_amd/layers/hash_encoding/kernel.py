@@ -128,8 +128,8 @@ def _launch_backward(coords2d: Tensor, do2d: Tensor, de: Tensor, pi: Tensor, T: 
     F = de.shape[-1]
     geom = level_geometry(T, levels, D, F, min_res, max_res)
     lib = _lib.load()
-    # scratch for the LDS-tile backward (bit-planes); torch's caching allocator makes this free after the first call
-    ws_bytes = 0 if (_FLAGS & 3) else lib.nf_hash_encode_bwd_workspace_bytes(N, geom, _lib.dtype_code(do2d.dtype))
+    # scratch for the LDS-tile backward; torch's caching allocator makes this free after the first call
+    ws_bytes = lib.nf_hash_encode_bwd_workspace_bytes(N, geom, _lib.dtype_code(do2d.dtype), _FLAGS)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=coords2d.device) if ws_bytes > 0 else None
     rc = lib.nf_hash_encode_bwd(
         coords2d.data_ptr(), _lib.dtype_code(coords2d.dtype), coords2d.stride(0), coords2d.stride(1),
