@@ -224,7 +224,8 @@ def bench_e2e(steps, warmup, n=2**21):
     def step():
         table.grad = w_in.grad = w_hid.grad = w_out.grad = None
         enc = hk.hash_encoding(x, table, None, None, T, MIN_RES, MAX_RES, L)
-        y = mk.fully_fused_mlp(enc.to(torch.bfloat16).unsqueeze(0), w_in, None, w_out, None, w_hid, None, "relu")
+        # the fp16 encoding goes straight into the bf16 MLP, which converts it while loading (and writes dx as fp16)
+        y = mk.fully_fused_mlp(enc.unsqueeze(0), w_in, None, w_out, None, w_hid, None, "relu")
         # summed (not averaged) squared error: keeps the fp16 gradient that reaches the encoder out of underflow
         loss = torch.nn.functional.mse_loss(y.float().squeeze(0), target, reduction="sum")
         loss.backward()

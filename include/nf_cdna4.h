@@ -105,21 +105,25 @@ int nf_hash_encode_indices(const void* coords, int coords_dtype, int64_t coords_
                            int64_t* out_rows, float* out_w, int64_t n_points, const nf_hash_geom* geom,
                            const int64_t* primes, float scale, void* stream);
 
-/* Fully fused MLP.  x [rows, d_in] (row stride x_stride), y [rows, d_out] (row stride y_stride);
+/* Fully fused MLP.  x [rows, d_in] (row stride x_stride) in x_dtype, y [rows, d_out] (row stride y_stride) in `dtype`;
  * w_in [d_hidden, d_in], w_hid [(depth-1)*d_hidden, d_hidden], w_out [d_out, d_hidden], all
  * row-contiguous in `dtype`; biases b_in [d_hidden], b_hid [depth-1, d_hidden], b_out [d_out]
  * may each be NULL.  depth >= 1 counts the input layer plus the hidden layers. */
 int nf_mlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_stride, const void* w_in, const void* b_in,
                const void* w_hid, const void* b_hid, const void* w_out, const void* b_out, int64_t rows, int d_in,
-               int d_hidden, int d_out, int depth, int act, int dtype, void* stream);
+               int d_hidden, int d_out, int depth, int act, int dtype, int x_dtype, void* stream);
 
-/* Backward.  dx [rows, d_in] in `dtype`; the dw_ and db_ arguments are float32 accumulators shaped like the
+/* x_dtype may be the other 16-bit type than `dtype` (an fp16 encoder output feeding bf16 weights): the rows are
+ * converted while they are loaded, as a cast kernel in front would, and the backward writes dx in x_dtype.
+ * nf_mlp_bwd takes a differing x_dtype for depth == 2 and d_hidden > 32 only (NF_EUNSUPPORTED otherwise).
+ *
+ * Backward.  dx [rows, d_in] in x_dtype; the dw_ and db_ arguments are float32 accumulators shaped like the
  * weights/biases, NOT cleared by the call (db_* may be NULL; dx may be NULL). */
 int nf_mlp_bwd(const void* x, int64_t x_stride, const void* dy, int64_t dy_stride, void* dx, int64_t dx_stride,
                const void* w_in, const void* b_in, const void* w_hid, const void* b_hid, const void* w_out,
                const void* b_out, float* dw_in, float* db_in, float* dw_hid, float* db_hid, float* dw_out,
                float* db_out, int64_t rows, int d_in, int d_hidden, int d_out, int depth, int act, int dtype,
-               void* stream);
+               int x_dtype, void* stream);
 
 /* Reversible MLP of `blocks` additive couplings over rows of width 2*half:
  *   y1 = x1 + F_k(x2),  y2 = x2 + G_k(y1),  F/G(u) = act(u W1^T + b1) W2^T + b2.

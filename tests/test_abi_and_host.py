@@ -48,16 +48,16 @@ def test_argument_validation_without_gpu():
     geom.dims = 7
     rc = lib.nf_hash_encode_fwd(None, 0, 3, 1, None, 0, None, 32, 10, geom, None, 1.0, 0, None)
     assert rc == -1 and b"dims" in lib.nf_last_error()
-    rc = lib.nf_mlp_fwd(None, 32, None, 16, None, None, None, None, None, None, 8, 32, 24, 16, 2, 1, _lib.NF_BF16, None)
+    rc = lib.nf_mlp_fwd(None, 32, None, 16, None, None, None, None, None, None, 8, 32, 24, 16, 2, 1, _lib.NF_BF16, _lib.NF_BF16, None)
     assert rc == -1 and b"d_hidden" in lib.nf_last_error()
-    rc = lib.nf_mlp_fwd(None, 32, None, 16, None, None, None, None, None, None, 8, 32, 64, 16, 2, 1, _lib.NF_F32, None)
+    rc = lib.nf_mlp_fwd(None, 32, None, 16, None, None, None, None, None, None, 8, 32, 64, 16, 2, 1, _lib.NF_F32, _lib.NF_BF16, None)
     assert rc == -2
     rc = lib.nf_revmlp_fwd(None, 128, None, 128, None, None, None, None, 8, 65, 4, 4, _lib.NF_BF16, None)
     assert rc == -1
     with pytest.raises(RuntimeError):
         _lib.check(rc, "nf_revmlp_fwd")
     # zero rows is a no-op that needs no device
-    assert lib.nf_mlp_fwd(None, 32, None, 16, None, None, None, None, None, None, 0, 32, 64, 16, 2, 1, _lib.NF_BF16, None) == 0
+    assert lib.nf_mlp_fwd(None, 32, None, 16, None, None, None, None, None, None, 0, 32, 64, 16, 2, 1, _lib.NF_BF16, _lib.NF_BF16, None) == 0
 
 
 @pytest.mark.parametrize("name", ["bench", "default"])

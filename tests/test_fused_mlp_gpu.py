@@ -191,6 +191,35 @@ def test_module_autocast(depth):
     assert set(layer.state_dict().keys()) == expect
 
 
+@pytest.mark.parametrize("x_dtype,w_dtype", [(torch.float16, torch.bfloat16), (torch.bfloat16, torch.float16)])
+@pytest.mark.parametrize("depth,bias", [(2, True), (2, False), (3, True)])
+def test_input_in_the_other_16bit_dtype(x_dtype, w_dtype, depth, bias):
+    """x stored in the other 16-bit dtype than the parameters (an fp16 encoder output in front of bf16 weights): the
+    result is bit-identical to casting x first, y comes in the parameters' dtype and dx in x's."""
+    mk = _mk()
+    torch.manual_seed(11)
+    p = {k: _dev(v) for k, v in _params(32, 64, 16, depth, bias, w_dtype, seed=5).items()}
+    rows = 4099
+    x = torch.randn(1, rows, 32).to(x_dtype).to(DEV)
+    dy = torch.randn(1, rows, 16).to(w_dtype).to(DEV)
+
+    def run(xin):
+        xin = xin.clone().requires_grad_(True)
+        ws = {k: (None if v is None else v.clone().requires_grad_(True)) for k, v in p.items()}
+        y = mk.fully_fused_mlp(xin, ws["w_in"], ws["b_in"], ws["w_out"], ws["b_out"], ws["w_hid"], ws["b_hid"], "relu")
+        y.backward(dy)
+        return y, xin.grad, {k: v.grad for k, v in ws.items() if v is not None}
+
+    y_mixed, dx_mixed, g_mixed = run(x)
+    y_cast, dx_cast, g_cast = run(x.to(w_dtype))
+    assert y_mixed.dtype == w_dtype and dx_mixed.dtype == x_dtype
+    assert torch.equal(y_mixed, y_cast)
+    # dx is rounded once from float32 to x's dtype instead of to the parameters' dtype and then again by autograd
+    torch.testing.assert_close(dx_mixed.float(), dx_cast.float(), rtol=1e-2, atol=1e-3)
+    for k in g_cast:
+        torch.testing.assert_close(g_mixed[k].float(), g_cast[k].float(), rtol=2e-2, atol=2e-2 * float(g_cast[k].float().abs().max()))
+
+
 def test_argument_errors():
     mk = _mk()
     p = {k: _dev(v) for k, v in _params(8, 16, 4, 1, True, torch.float16).items()}

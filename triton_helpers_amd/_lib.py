@@ -83,9 +83,9 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.nf_hash_encode_indices.restype = c_int
     lib.nf_hash_encode_indices.argtypes = [P, I, I64, I64, P, P, I64, POINTER(HashGeom), P, c_float, P]
     lib.nf_mlp_fwd.restype = c_int
-    lib.nf_mlp_fwd.argtypes = [P, I64, P, I64, P, P, P, P, P, P, I64, I, I, I, I, I, I, P]
+    lib.nf_mlp_fwd.argtypes = [P, I64, P, I64, P, P, P, P, P, P, I64, I, I, I, I, I, I, I, P]
     lib.nf_mlp_bwd.restype = c_int
-    lib.nf_mlp_bwd.argtypes = [P, I64, P, I64, P, I64, P, P, P, P, P, P, P, P, P, P, P, P, I64, I, I, I, I, I, I, P]
+    lib.nf_mlp_bwd.argtypes = [P, I64, P, I64, P, I64, P, P, P, P, P, P, P, P, P, P, P, P, I64, I, I, I, I, I, I, I, P]
     lib.nf_revmlp_fwd.restype = c_int
     lib.nf_revmlp_fwd.argtypes = [P, I64, P, I64, P, P, P, P, I64, I, I, I, I, P]
     lib.nf_revmlp_bwd.restype = c_int
@@ -131,20 +131,30 @@ def current_stream(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
-def zeros_like_f32(*tensors):
-    """float32 zero accumulators shaped like the given tensors (``None`` stays ``None``), carved out of one
-    buffer so that a single fill kernel clears them all."""
-    live = [t for t in tensors if t is not None]
-    if not live:
-        return tuple(None for _ in tensors)
-    sizes = [(t.numel() + 3) // 4 * 4 for t in live]  # 16-byte aligned pieces
-    flat = torch.zeros(sum(sizes), dtype=torch.float32, device=live[0].device)
-    out, off, k = [], 0, 0
-    for t in tensors:
-        if t is None:
-            out.append(None)
-            continue
-        out.append(flat[off:off + t.numel()].view(t.shape))
-        off += sizes[k]
-        k += 1
-    return tuple(out)
+class GradBuffers:
+    """float32 zero accumulators shaped like the given tensors (``None`` stays ``None``), carved out of one buffer
+    so that a single fill kernel clears them all and a single cast kernel rounds them all to the parameters' dtype.
+    The kernels only need addresses, so no view tensors are made for the accumulators (each tensor op costs the host
+    a few microseconds, which is what bounds a small step)."""
+
+    def __init__(self, *tensors):
+        self._like = tensors
+        self._offsets, off = [], 0
+        for t in tensors:
+            self._offsets.append(off)
+            if t is not None:
+                off += (t.numel() + 3) // 4 * 4  # 16-byte aligned pieces
+        self.flat = torch.zeros(off, dtype=torch.float32, device=next(t for t in tensors if t is not None).device) if off else None
+
+    def pointers(self):
+        """Device addresses of the accumulators (``None`` where the tensor is absent)."""
+        base = self.flat.data_ptr() if self.flat is not None else 0
+        return tuple(None if t is None else base + 4 * o for t, o in zip(self._like, self._offsets))
+
+    def rounded(self, dtype):
+        """The accumulators rounded once to ``dtype`` (what autograd would do tensor by tensor), as views."""
+        if self.flat is None:
+            return tuple(None for _ in self._like)
+        flat = self.flat if dtype == torch.float32 else self.flat.to(dtype)
+        return tuple(None if t is None else flat.as_strided(t.shape, t.stride(), o) if t.is_contiguous()
+                     else flat[o:o + t.numel()].view(t.shape) for t, o in zip(self._like, self._offsets))

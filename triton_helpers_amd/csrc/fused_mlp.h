@@ -20,10 +20,23 @@ struct MlpArgs {
   int d_in, d_hidden, d_out, depth, act;
   int x_vec, y_vec, dy_vec, dx_vec;
   int waves;  // waves per workgroup
+  int x_conv; // 0: x / dx stored like the weights; 1: stored as float16 (weights bfloat16); 2: stored as bfloat16 (weights float16)
 };
 
 constexpr int FRAG_ELEMS = 64 * 8;  // 16-bit elements per fragment (1 KiB)
 constexpr int TPITCH = 40;          // 16-bit elements per feature row of a transposed 32-row panel (80 B)
+
+// Fragment of 8 values stored in the other 16-bit type -> the compute type (what a cast kernel in front would do).
+__device__ __forceinline__ Frag convert_frag(Frag f, int x_conv) {
+  if (x_conv == 1) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f.w[i] = pack2<BF16>(unpack_lo<F16>(f.w[i]), unpack_hi<F16>(f.w[i]));
+  } else if (x_conv == 2) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f.w[i] = pack2<F16>(unpack_lo<BF16>(f.w[i]), unpack_hi<BF16>(f.w[i]));
+  }
+  return f;
+}
 
 template <typename T>
 __device__ __forceinline__ void stage_bias(float* dst, const uint16_t* b, int n_valid, int n_pad, int tid, int nthreads) {

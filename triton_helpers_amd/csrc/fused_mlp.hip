@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void mlp_fwd_k(MlpArgs a) {
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
       for (int kc = 0; kc < KC_IN; ++kc) {
-        in[nt][kc] = nxt[nt][kc];
+        in[nt][kc] = convert_frag(nxt[nt][kc], a.x_conv);
         nxt[nt][kc] = load_rows_frag(a.x, a.x_stride, (chunk + wave_stride) * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
       }
 
@@ -616,8 +616,9 @@ using namespace nf;
 
 extern "C" int nf_mlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_stride, const void* w_in, const void* b_in,
                           const void* w_hid, const void* b_hid, const void* w_out, const void* b_out, int64_t rows,
-                          int d_in, int d_hidden, int d_out, int depth, int act, int dtype, void* stream) {
+                          int d_in, int d_hidden, int d_out, int depth, int act, int dtype, int x_dtype, void* stream) {
   if (int rc = validate(rows, d_in, d_hidden, d_out, depth, act, dtype)) return rc;
+  NF_REQUIRE(x_dtype == NF_F16 || x_dtype == NF_BF16, NF_EUNSUPPORTED, "x_dtype code %d: float16 or bfloat16", x_dtype);
   if (rows == 0) return 0;
   NF_REQUIRE(x && y && w_in && w_out, NF_EINVAL, "NULL pointer argument");
   NF_REQUIRE(depth == 1 || w_hid, NF_EINVAL, "w_hid is NULL but depth=%d", depth);
@@ -629,6 +630,7 @@ extern "C" int nf_mlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_st
   a.rows = rows; a.d_in = d_in; a.d_hidden = d_hidden; a.d_out = d_out; a.depth = depth; a.act = act;
   a.x_vec = vec_load_ok(x, x_stride, d_in);
   a.y_vec = vec_store_ok(y, y_stride, d_out);
+  a.x_conv = x_dtype == dtype ? 0 : (x_dtype == NF_F16 ? 1 : 2);
   hipStream_t s = (hipStream_t)stream;
   return dtype == NF_BF16 ? dispatch_fwd<BF16>(a, s) : dispatch_fwd<F16>(a, s);
 }
@@ -637,8 +639,9 @@ extern "C" int nf_mlp_bwd(const void* x, int64_t x_stride, const void* dy, int64
                           const void* w_in, const void* b_in, const void* w_hid, const void* b_hid, const void* w_out,
                           const void* b_out, float* dw_in, float* db_in, float* dw_hid, float* db_hid, float* dw_out,
                           float* db_out, int64_t rows, int d_in, int d_hidden, int d_out, int depth, int act, int dtype,
-                          void* stream) {
+                          int x_dtype, void* stream) {
   if (int rc = validate(rows, d_in, d_hidden, d_out, depth, act, dtype)) return rc;
+  NF_REQUIRE(x_dtype == NF_F16 || x_dtype == NF_BF16, NF_EUNSUPPORTED, "x_dtype code %d: float16 or bfloat16", x_dtype);
   if (rows == 0) return 0;
   NF_REQUIRE(x && dy && w_in && w_out && dw_in && dw_out, NF_EINVAL, "NULL pointer argument");
   NF_REQUIRE(depth == 1 || (w_hid && dw_hid), NF_EINVAL, "w_hid / dw_hid is NULL but depth=%d", depth);
@@ -654,9 +657,11 @@ extern "C" int nf_mlp_bwd(const void* x, int64_t x_stride, const void* dy, int64
   a.x_vec = vec_load_ok(x, x_stride, d_in);
   a.dy_vec = vec_load_ok(dy, dy_stride, d_out);
   a.dx_vec = dx ? vec_store_ok(dx, dx_stride, d_in) : 0;
+  a.x_conv = x_dtype == dtype ? 0 : (x_dtype == NF_F16 ? 1 : 2);
   hipStream_t s = (hipStream_t)stream;
   bool handled = false;
   const int rc = launch_mlp_bwd2(a, dtype, s, &handled);
   if (rc != 0 || handled) return rc;
+  NF_REQUIRE(a.x_conv == 0, NF_EUNSUPPORTED, "x_dtype != dtype needs depth == 2 and d_hidden > 32 in the backward");
   return dtype == NF_BF16 ? dispatch_bwd<BF16>(a, s) : dispatch_bwd<F16>(a, s);
 }

@@ -115,6 +115,13 @@ __device__ __forceinline__ Frag load_chain(const uint16_t* base, int64_t stride,
 #ifndef NF_BWD2_OCC
 #define NF_BWD2_OCC 1
 #endif
+// dx tile in the type x is stored in
+template <typename XT, bool FAST>
+__device__ __forceinline__ void store_dx(const MlpArgs& a, int64_t row0, int mt, int lane, f32x4_t v) {
+  if (FAST) store_rows_tile_fast<XT>(a.dx, a.dx_stride, row0, a.rows, a.d_in, mt, lane, v);
+  else store_rows_tile<XT>(a.dx, a.dx_stride, row0, a.rows, a.d_in, mt, lane, v, a.dx_vec);
+}
+
 // acc[nt][mt] = bias (or 0) + W(frags) * in[nt][kc], one weight fragment read per NT products; K chunks outermost, so
 // that the products into one accumulator tile are MT * NT instructions apart
 template <typename T, int NT, int MT, int KC>
@@ -206,7 +213,7 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
     for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
       for (int kc = 0; kc < KC_IN; ++kc) {
-        in[nt][kc] = nx[nt][kc];
+        in[nt][kc] = convert_frag(nx[nt][kc], a.x_conv);
         nx[nt][kc] = load_chain<FAST>(a.x, a.x_stride, (chunk + wave_stride) * ROWS + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
       }
 #pragma unroll
@@ -337,8 +344,9 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
       for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int mt = 0; mt < MT_I; ++mt) {
-          if (FAST) store_rows_tile_fast<T>(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, a.d_in, mt, lane, acc[nt][mt]);
-          else store_rows_tile<T>(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, a.d_in, mt, lane, acc[nt][mt], a.dx_vec);
+          if (a.x_conv == 1) store_dx<F16, FAST>(a, row0 + 16 * nt, mt, lane, acc[nt][mt]);
+          else if (a.x_conv == 2) store_dx<BF16, FAST>(a, row0 + 16 * nt, mt, lane, acc[nt][mt]);
+          else store_dx<T, FAST>(a, row0 + 16 * nt, mt, lane, acc[nt][mt]);
         }
     }
   }

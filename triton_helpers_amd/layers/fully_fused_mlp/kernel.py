@@ -81,13 +81,17 @@ def feedforward_bwd_dx(w: Tensor, dz: Tensor, DTYPE: torch.dtype = torch.float32
 
 
 # ---------------------------------------------------------------------------
-def _check_storage(x: Tensor, *others: Optional[Tensor]) -> None:
-    if x.dtype not in (torch.float16, torch.bfloat16):
-        raise NotImplementedError(
-            f"fully_fused_mlp runs on float16 / bfloat16 storage, got {x.dtype}; cast the tensors or use autocast"
-        )
+def _check_storage(x: Tensor, w_in: Tensor, *others: Optional[Tensor]) -> None:
+    """Parameters share one 16-bit dtype; ``x`` may be in the other 16-bit dtype (an fp16 encoder output in front of
+    bf16 weights): the kernels convert it while loading, exactly as a cast in front would."""
+    for t in (x, w_in):
+        if t.dtype not in (torch.float16, torch.bfloat16):
+            raise NotImplementedError(
+                f"fully_fused_mlp runs on float16 / bfloat16 storage, got {t.dtype}; cast the tensors or use autocast"
+            )
     for t in others:
-        assert t is None or t.dtype == x.dtype, f"All tensors must share one dtype, got {x.dtype} and {t.dtype}"
+        assert t is None or t.dtype == w_in.dtype, f"All parameters must share one dtype, got {w_in.dtype} and {t.dtype}"
+    for t in (w_in, *others):
         assert t is None or t.device == x.device, "All tensors must be on the same device"
     assert x.device.type == "cuda", "All tensors must be on a GPU device"
 
@@ -145,14 +149,14 @@ class _fully_fused_mlp(Function):
 
         w_in, b_in, w_out, b_out, w_hid, b_hid = (_c(t) for t in (w_in, b_in, w_out, b_out, w_hid, b_hid))
         x2 = _rows2d(x, D_in)
-        o = x.new_empty((B, L, D_out))
+        o = x.new_empty((B, L, D_out), dtype=w_in.dtype)
         o2 = o.view(-1, D_out)
         lib = _lib.load()
         rc = lib.nf_mlp_fwd(
             x2.data_ptr(), x2.stride(0), o2.data_ptr(), o2.stride(0),
             w_in.data_ptr(), _lib.ptr(b_in), _lib.ptr(w_hid), _lib.ptr(b_hid), w_out.data_ptr(), _lib.ptr(b_out),
-            x2.shape[0], D_in, D_hidden, D_out, depth, _lib.NF_ACT[activation], _lib.dtype_code(x.dtype),
-            _lib.current_stream(x.device),
+            x2.shape[0], D_in, D_hidden, D_out, depth, _lib.NF_ACT[activation], _lib.dtype_code(w_in.dtype),
+            _lib.dtype_code(x.dtype), _lib.current_stream(x.device),
         )
         _lib.check(rc, "nf_mlp_fwd")
 
@@ -170,25 +174,29 @@ class _fully_fused_mlp(Function):
         B, L, D_in = x.shape
         D_hidden = w_in.shape[0]
         D_out = w_out.shape[0]
-        if do.dtype != x.dtype:
-            do = do.to(x.dtype)
+        if do.dtype != w_in.dtype:
+            do = do.to(w_in.dtype)
+        if x.dtype != w_in.dtype and not (ctx.depth == 2 and D_hidden > 32):
+            x = x.to(w_in.dtype)  # only the one-hidden-layer backward converts on the fly
         x2 = _rows2d(x, D_in)
         do2 = _rows2d(do, D_out)
         need_dx = ctx.needs_input_grad[0]
         dx = x.new_empty(x.shape) if need_dx else None
 
-        dw_in, db_in, dw_out, db_out, dw_hid, db_hid = _lib.zeros_like_f32(w_in, b_in, w_out, b_out, w_hid, b_hid)
+        grads = _lib.GradBuffers(w_in, b_in, w_out, b_out, w_hid, b_hid)
+        p_dw_in, p_db_in, p_dw_out, p_db_out, p_dw_hid, p_db_hid = grads.pointers()
         lib = _lib.load()
         rc = lib.nf_mlp_bwd(
             x2.data_ptr(), x2.stride(0), do2.data_ptr(), do2.stride(0),
             _lib.ptr(dx), D_in,
             w_in.data_ptr(), _lib.ptr(b_in), _lib.ptr(w_hid), _lib.ptr(b_hid), w_out.data_ptr(), _lib.ptr(b_out),
-            dw_in.data_ptr(), _lib.ptr(db_in), _lib.ptr(dw_hid), _lib.ptr(db_hid), dw_out.data_ptr(), _lib.ptr(db_out),
-            x2.shape[0], D_in, D_hidden, D_out, ctx.depth, _lib.NF_ACT[ctx.activation], _lib.dtype_code(x.dtype),
-            _lib.current_stream(x.device),
+            p_dw_in, p_db_in, p_dw_hid, p_db_hid, p_dw_out, p_db_out,
+            x2.shape[0], D_in, D_hidden, D_out, ctx.depth, _lib.NF_ACT[ctx.activation], _lib.dtype_code(w_in.dtype),
+            _lib.dtype_code(x.dtype), _lib.current_stream(x.device),
         )
         _lib.check(rc, "nf_mlp_bwd")
-        # float32 accumulators; autograd rounds them once to each parameter's dtype
+        # float32 accumulators, rounded once to the parameters' dtype (one kernel for all of them)
+        dw_in, db_in, dw_out, db_out, dw_hid, db_hid = grads.rounded(w_in.dtype)
         return dx, dw_in, db_in, dw_out, db_out, dw_hid, db_hid, None, None
 
 

@@ -86,15 +86,17 @@ class _reversible_mlp(Function):
         dx = y.new_empty(y.shape)
         x_rec = y.new_empty(y.shape)
 
-        dw1, db1, dw2, db2 = _lib.zeros_like_f32(w1, b1, w2, b2)
+        grads = _lib.GradBuffers(w1, b1, w2, b2)
+        p_dw1, p_db1, p_dw2, p_db2 = grads.pointers()
         lib = _lib.load()
         rc = lib.nf_revmlp_bwd(
             y2.data_ptr(), y2.stride(0), dy2.data_ptr(), dy2.stride(0), dx.data_ptr(), 2 * H, x_rec.data_ptr(), 2 * H,
             w1.data_ptr(), _lib.ptr(b1), w2.data_ptr(), _lib.ptr(b2),
-            dw1.data_ptr(), _lib.ptr(db1), dw2.data_ptr(), _lib.ptr(db2),
+            p_dw1, p_db1, p_dw2, p_db2,
             y2.shape[0], H, ctx.blocks, _lib.NF_ACT[ctx.activation], _lib.dtype_code(y.dtype), _lib.current_stream(y.device),
         )
         _lib.check(rc, "nf_revmlp_bwd")
+        dw1, db1, dw2, db2 = grads.rounded(w1.dtype)
         return dx, dw1, db1, dw2, db2, None
 
 
