@@ -115,7 +115,8 @@ int nf_mlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_stride, const
 
 /* x_dtype may be the other 16-bit type than `dtype` (an fp16 encoder output feeding bf16 weights): the rows are
  * converted while they are loaded, as a cast kernel in front would, and the backward writes dx in x_dtype.
- * nf_mlp_bwd takes a differing x_dtype for depth == 2 and d_hidden > 32 only (NF_EUNSUPPORTED otherwise).
+ * nf_mlp_bwd takes a differing x_dtype for depth == 2, d_hidden > 32, ReLU and 8-byte aligned rows only
+ * (NF_EUNSUPPORTED otherwise).
  *
  * Backward.  dx [rows, d_in] in x_dtype; the dw_ and db_ arguments are float32 accumulators shaped like the
  * weights/biases, NOT cleared by the call (db_* may be NULL; dx may be NULL). */

@@ -32,7 +32,8 @@ __device__ __forceinline__ void hidden_epilogue(const f32x4_t (&acc)[2][4], Frag
 // ---------------------------------------------------------------------------------------
 // Forward
 // ---------------------------------------------------------------------------------------
-template <typename T, int KIN, int HP, int OUTP>
+// XC: how x is stored (MlpArgs::x_conv), fixed at compile time.
+template <typename T, int KIN, int HP, int OUTP, int XC>
 __global__ __launch_bounds__(256) void mlp_fwd_k(MlpArgs a) {
   constexpr int KC_IN = KIN / 32, KC_H = HP / 32, MT_H = HP / 16, MT_O = OUTP / 16;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -78,7 +79,7 @@ __global__ __launch_bounds__(256) void mlp_fwd_k(MlpArgs a) {
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
       for (int kc = 0; kc < KC_IN; ++kc) {
-        in[nt][kc] = convert_frag(nxt[nt][kc], a.x_conv);
+        in[nt][kc] = XC == 0 ? nxt[nt][kc] : convert_frag(nxt[nt][kc], XC);
         nxt[nt][kc] = load_rows_frag(a.x, a.x_stride, (chunk + wave_stride) * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
       }
 
@@ -530,12 +531,15 @@ static int launch_fwd(const MlpArgs& a0, hipStream_t s) {
   int64_t blocks = (chunks + a.waves - 1) / a.waves;
   const int64_t cap = (int64_t)device_cus() * (lds > 64 * 1024 ? 1 : (lds > 40 * 1024 ? 2 : 3));
   if (blocks > cap) blocks = cap;
-  auto kern = mlp_fwd_k<T, KIN, HP, OUTP>;
+  constexpr int XC_OTHER = T::code == NF_BF16 ? 1 : 2;
+  const void* kern = a.x_conv == 0 ? (const void*)mlp_fwd_k<T, KIN, HP, OUTP, 0> : (const void*)mlp_fwd_k<T, KIN, HP, OUTP, XC_OTHER>;
   if (lds > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(64 * a.waves), lds, s, a);
+  void* args[] = {(void*)&a};
+  const hipError_t le = hipLaunchKernel(kern, dim3((unsigned)blocks), dim3(64 * a.waves), args, lds, s);
+  if (le != hipSuccess) return fail((int)le, "hipLaunchKernel(mlp_fwd): %s", hipGetErrorString(le));
   return check_launch("mlp_fwd");
 }
 

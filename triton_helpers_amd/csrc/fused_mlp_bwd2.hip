@@ -145,7 +145,8 @@ __device__ __forceinline__ void layer_nt(f32x4_t (&acc)[NT][4], const Frag (&in)
 }
 
 // NT: 16-row tiles per chunk (2 or 4).  Four give the scheduler two independent 32-row groups to interleave.
-template <typename T, int KIN, int HP, int OUTP, bool RELU, bool FAST, int NT>
+// XC: how x / dx are stored (MlpArgs::x_conv), fixed at compile time so that the usual case pays nothing for it.
+template <typename T, int KIN, int HP, int OUTP, bool RELU, bool FAST, int NT, int XC>
 __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArgs a) {
   constexpr int KC_IN = KIN / 32, KC_H = HP / 32, MT_H = HP / 16, MT_I = KIN / 16, MT_O = OUTP / 16;
   constexpr int KC_O = (OUTP + 31) / 32;
@@ -213,7 +214,7 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
     for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
       for (int kc = 0; kc < KC_IN; ++kc) {
-        in[nt][kc] = convert_frag(nx[nt][kc], a.x_conv);
+        in[nt][kc] = XC == 0 ? nx[nt][kc] : convert_frag(nx[nt][kc], XC);
         nx[nt][kc] = load_chain<FAST>(a.x, a.x_stride, (chunk + wave_stride) * ROWS + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
       }
 #pragma unroll
@@ -344,8 +345,8 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
       for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int mt = 0; mt < MT_I; ++mt) {
-          if (a.x_conv == 1) store_dx<F16, FAST>(a, row0 + 16 * nt, mt, lane, acc[nt][mt]);
-          else if (a.x_conv == 2) store_dx<BF16, FAST>(a, row0 + 16 * nt, mt, lane, acc[nt][mt]);
+          if (XC == 1) store_dx<F16, FAST>(a, row0 + 16 * nt, mt, lane, acc[nt][mt]);
+          else if (XC == 2) store_dx<BF16, FAST>(a, row0 + 16 * nt, mt, lane, acc[nt][mt]);
           else store_dx<T, FAST>(a, row0 + 16 * nt, mt, lane, acc[nt][mt]);
         }
     }
@@ -437,11 +438,18 @@ static int launch2(const MlpArgs& a0, hipStream_t s) {
   if (blocks > cap) blocks = cap;
   const bool fast = a.x_vec && a.dy_vec && a.d_in % 4 == 0 && a.d_out % 4 == 0 &&
                     (a.dx == nullptr || ((uintptr_t)a.dx % 8 == 0 && a.dx_stride % 4 == 0));
+  // x in the other 16-bit type: built for the aligned ReLU case only (the end-to-end encoder -> MLP step)
+  constexpr int XC_OTHER = T::code == NF_BF16 ? 1 : 2;
   const void* kern;
-  if (a.act == NF_ACT_RELU)
-    kern = fast ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, true, NT> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, false, NT>;
-  else
-    kern = fast ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false, true, 2> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false, false, 2>;
+  if (a.x_conv != 0) {
+    NF_REQUIRE(fast && a.act == NF_ACT_RELU && a.x_conv == XC_OTHER, NF_EUNSUPPORTED,
+               "x_dtype != dtype: the backward covers ReLU with 8-byte aligned rows only");
+    kern = (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, true, NT, XC_OTHER>;
+  } else if (a.act == NF_ACT_RELU) {
+    kern = fast ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, true, NT, 0> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, false, NT, 0>;
+  } else {
+    kern = fast ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false, true, 2, 0> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false, false, 2, 0>;
+  }
   void* args[] = {(void*)&a};
   const hipError_t e = hipLaunchKernel(kern, dim3((unsigned)blocks), dim3(256), args, LDS, s);
   if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(mlp_bwd2): %s", hipGetErrorString(e));

@@ -176,24 +176,28 @@ class _fully_fused_mlp(Function):
         D_out = w_out.shape[0]
         if do.dtype != w_in.dtype:
             do = do.to(w_in.dtype)
-        if x.dtype != w_in.dtype and not (ctx.depth == 2 and D_hidden > 32):
-            x = x.to(w_in.dtype)  # only the one-hidden-layer backward converts on the fly
-        x2 = _rows2d(x, D_in)
+        if x.dtype != w_in.dtype and not (ctx.depth == 2 and D_hidden > 32 and ctx.activation == "relu"):
+            x = x.to(w_in.dtype)  # only the one-hidden-layer ReLU backward converts on the fly
         do2 = _rows2d(do, D_out)
         need_dx = ctx.needs_input_grad[0]
-        dx = x.new_empty(x.shape) if need_dx else None
-
         grads = _lib.GradBuffers(w_in, b_in, w_out, b_out, w_hid, b_hid)
         p_dw_in, p_db_in, p_dw_out, p_db_out, p_dw_hid, p_db_hid = grads.pointers()
         lib = _lib.load()
-        rc = lib.nf_mlp_bwd(
-            x2.data_ptr(), x2.stride(0), do2.data_ptr(), do2.stride(0),
-            _lib.ptr(dx), D_in,
-            w_in.data_ptr(), _lib.ptr(b_in), _lib.ptr(w_hid), _lib.ptr(b_hid), w_out.data_ptr(), _lib.ptr(b_out),
-            p_dw_in, p_db_in, p_dw_hid, p_db_hid, p_dw_out, p_db_out,
-            x2.shape[0], D_in, D_hidden, D_out, ctx.depth, _lib.NF_ACT[ctx.activation], _lib.dtype_code(w_in.dtype),
-            _lib.dtype_code(x.dtype), _lib.current_stream(x.device),
-        )
+        while True:
+            x2 = _rows2d(x, D_in)
+            dx = x.new_empty(x.shape) if need_dx else None
+            rc = lib.nf_mlp_bwd(
+                x2.data_ptr(), x2.stride(0), do2.data_ptr(), do2.stride(0),
+                _lib.ptr(dx), D_in,
+                w_in.data_ptr(), _lib.ptr(b_in), _lib.ptr(w_hid), _lib.ptr(b_hid), w_out.data_ptr(), _lib.ptr(b_out),
+                p_dw_in, p_db_in, p_dw_hid, p_db_hid, p_dw_out, p_db_out,
+                x2.shape[0], D_in, D_hidden, D_out, ctx.depth, _lib.NF_ACT[ctx.activation], _lib.dtype_code(w_in.dtype),
+                _lib.dtype_code(x.dtype), _lib.current_stream(x.device),
+            )
+            if rc == _lib.NF_EUNSUPPORTED and x.dtype != w_in.dtype:
+                x = x.to(w_in.dtype)  # a shape / alignment the converting backward does not cover: cast first
+                continue
+            break
         _lib.check(rc, "nf_mlp_bwd")
         # float32 accumulators, rounded once to the parameters' dtype (one kernel for all of them)
         dw_in, db_in, dw_out, db_out, dw_hid, db_hid = grads.rounded(w_in.dtype)
