@@ -425,7 +425,51 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
     }
   }
 
-  // ---- weight gradients: every wave adds its float32 accumulators (64-byte coalesced atomics) ----
+  // ---- weight gradients: summed over the four waves through LDS (the weight fragments are dead by now), then one
+  // pass of 64-byte coalesced atomics per workgroup ----
+  __syncthreads();
+  constexpr int NREG = G2_LDS ? 3 : 4;  // accumulators that live in registers
+  f32x4_t* red = reinterpret_cast<f32x4_t*>(smem) + lane;
+  float* redb = reinterpret_cast<float*>(smem) + (size_t)NREG * MT * MT * 256 + lane;
+  for (int w = 1; w < 4; ++w) {
+    if (wave == w) {
+      int t = 0, u = 0;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+          red[64 * (t++)] = dwF1[i][j];
+          red[64 * (t++)] = dwF2[i][j];
+          red[64 * (t++)] = dwG1[i][j];
+          if (!G2_LDS) red[64 * (t++)] = dwG2[i][j];
+        }
+        redb[64 * (u++)] = dbF1[i];
+        redb[64 * (u++)] = dbF2[i];
+        redb[64 * (u++)] = dbG1[i];
+        redb[64 * (u++)] = dbG2[i];
+      }
+    }
+    __syncthreads();
+    if (wave == 0) {
+      int t = 0, u = 0;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+          dwF1[i][j] += red[64 * (t++)];
+          dwF2[i][j] += red[64 * (t++)];
+          dwG1[i][j] += red[64 * (t++)];
+          if (!G2_LDS) dwG2[i][j] += red[64 * (t++)];
+        }
+        dbF1[i] += redb[64 * (u++)];
+        dbF2[i] += redb[64 * (u++)];
+        dbG1[i] += redb[64 * (u++)];
+        dbG2[i] += redb[64 * (u++)];
+      }
+    }
+    __syncthreads();
+  }
+  if (wave != 0) return;
   // layer order in dw1 / dw2: sub-MLP F is row block 0, G is row block 1 of this coupling block
 #pragma unroll
   for (int i = 0; i < MT; ++i)
@@ -434,7 +478,12 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
       flush_tile(a.dw1, H, i, j, lane, dwF1[i][j]);
       flush_tile(a.dw2, H, i, j, lane, dwF2[i][j]);
       flush_tile(a.dw1 + (size_t)H * H, H, i, j, lane, dwG1[i][j]);
-      flush_tile(a.dw2 + (size_t)H * H, H, i, j, lane, G2_LDS ? g2acc[(i * MT + j) * 64 + lane] : dwG2[i][j]);
+      if (G2_LDS) {
+        constexpr int PER_WAVE = MT * MT * 64;
+        const int at = (i * MT + j) * 64 + lane;  // wave 0's g2acc is the first of the four
+        dwG2[i][j] = (g2acc[at] + g2acc[PER_WAVE + at]) + (g2acc[2 * PER_WAVE + at] + g2acc[3 * PER_WAVE + at]);
+      }
+      flush_tile(a.dw2 + (size_t)H * H, H, i, j, lane, dwG2[i][j]);
     }
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
@@ -499,7 +548,10 @@ static int launch_rev_fwd(RevArgs a, hipStream_t s) {
 template <typename T, int HP>
 static int launch_rev_bwd(RevArgs a, hipStream_t s) {
   constexpr int LAYER = (HP / 16) * (HP / 32) * RFRAG;
-  const size_t lds = (size_t)8 * LAYER * 2 + (size_t)4 * HP * 4 + (HP > 32 ? (size_t)4 * (HP / 16) * (HP / 16) * 64 * 16 : 0);
+  size_t lds = (size_t)8 * LAYER * 2 + (size_t)4 * HP * 4 + (HP > 32 ? (size_t)4 * (HP / 16) * (HP / 16) * 64 * 16 : 0);
+  // the closing reduction over the waves reuses the front of LDS: the register accumulators and 4 bias sums per tile row
+  const size_t red = (size_t)(HP > 32 ? 3 : 4) * (HP / 16) * (HP / 16) * 64 * 16 + (size_t)4 * (HP / 16) * 64 * 4;
+  if (HP <= 32 && lds < red) lds = red;
   const int64_t chunks = (a.rows + 31) / 32;
   int64_t blocks = (chunks + 3) / 4;
   // the weight-gradient accumulators take most of the register file: one wave per SIMD
