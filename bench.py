@@ -43,8 +43,8 @@ N_POINTS = 2**20
 FWD_BYTES_PER_POINT = 4 * D + L * 8 * F * 2 + L * F * 2  # 588
 BWD_BYTES_PER_POINT = 4 * D + L * F * 2 + L * 8 * F * 4  # 1100
 # HBM bytes per forward launch at N = 2^20 measured with rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a 256 MiB copy
-# kernel gives for that counter) + WRITE_SIZE (x1.0): 1694 MB + 67 MB
-FWD_TRAFFIC_BYTES = 1.761e9
+# kernel gives for that counter) + WRITE_SIZE (x1.0): 842 MB + 67 MB
+FWD_TRAFFIC_BYTES = 9.10e8
 
 
 def event_times(fn, reps):
@@ -256,9 +256,9 @@ def main():
     torch.cuda.set_device(0)
 
     h = bench_hash(args.steps, args.warmup)
-    # The forward is one kernel (hash_fwd_tiled_k); the backward is zero + count + offsets + fill + accumulate, each
+    # The forward is one kernel (hash_fwd_sweep_k); the backward is zero + count + offsets + fill + accumulate, each
     # shorter than the forward kernel.
-    dom, dom_ms, dom_bytes = "hash_fwd_tiled_k", h["t_fwd"], FWD_BYTES_PER_POINT * N_POINTS
+    dom, dom_ms, dom_bytes = "hash_fwd_sweep_k", h["t_fwd"], FWD_BYTES_PER_POINT * N_POINTS
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
     bwd_achieved = BWD_BYTES_PER_POINT * N_POINTS / (h["t_bwd"] * 1e-3) / 1e9
     step_bytes = (FWD_BYTES_PER_POINT + BWD_BYTES_PER_POINT) * N_POINTS + h["E"] * F * 4

@@ -67,7 +67,8 @@ typedef struct nf_hash_geom {
 enum {
   NF_HASH_FORCE_GENERIC = 1,   /* use the one-thread-per-(point,level) kernel even where a faster kernel applies */
   NF_HASH_FORCE_ATOMIC = 2,    /* backward: scatter with global atomics even where the LDS-tile kernels apply */
-  NF_HASH_FORCE_PLANES = 4     /* backward: of the two LDS-tile variants take the bit-plane one (smaller workspace) */
+  NF_HASH_FORCE_PLANES = 4,    /* backward: of the two LDS-tile variants take the bit-plane one (smaller workspace) */
+  NF_HASH_FWD_STAGED = 8       /* forward: the LDS-staged tile kernel instead of the register-resident level sweep */
 };
 
 int nf_abi_version(void);

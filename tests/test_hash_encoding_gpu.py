@@ -121,6 +121,30 @@ def test_tiled_and_generic_agree_bitwise(monkeypatch):
     assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("L,hi", [(16, 7006), (8, 512), (4, 64)])
+def test_forward_kernels_agree_bitwise_at_sweep_sizes(L, hi, dtype, monkeypatch):
+    """From 2^18 points on the forward takes the register-resident level sweep; flag 8 selects the LDS-staged
+    tile kernel and flag 1 the per-(point, level) kernel: all three must produce the same bits, also for a ragged
+    last workgroup and a coordinate scale."""
+    hk = _hk()
+    g = GOLDEN["bench"]
+    N = 2**18 + 77
+    torch.manual_seed(2)
+    x = torch.rand(N, 3, device=DEV) * 2.5
+    table = _table(g["T"], L, 3, 16, hi, dtype=dtype, amp=1.0).to(DEV)
+    outs = []
+    for flags in (0, 8, 1):
+        monkeypatch.setattr(hk, "_FLAGS", flags)
+        outs.append(hk.hash_encoding(x, table, None, None, g["T"], 16, hi, L, scale=2.5))
+    assert torch.equal(outs[0], outs[1])
+    assert torch.equal(outs[0], outs[2])
+    idx = torch.randperm(N)[:2048]
+    want = O.encode_forward(x[idx.to(DEV)].cpu() / 2.5, table.float().cpu(), None, g["T"], L, 16, hi)
+    eps = 2.0**-10 if dtype == torch.float16 else 2.0**-7
+    torch.testing.assert_close(outs[0][idx.to(DEV)].cpu().float(), want, rtol=eps, atol=eps * 1e-3)
+
+
 def test_forward_config0_full_size():
     """BASELINE configs[0]: N=65536, L=16, F=2, T=2^19, fp32 table U(-1e-4, 1e-4), seed 0."""
     g = GOLDEN["bench"]

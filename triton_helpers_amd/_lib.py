@@ -23,6 +23,7 @@ NF_EINVAL, NF_EUNSUPPORTED, NF_EALIGN = -1, -2, -3
 NF_HASH_FORCE_GENERIC = 1
 NF_HASH_FORCE_ATOMIC = 2
 NF_HASH_FORCE_PLANES = 4
+NF_HASH_FWD_STAGED = 8
 
 _DTYPE_CODE = {torch.float32: NF_F32, torch.float16: NF_F16, torch.bfloat16: NF_BF16}
 

@@ -232,6 +232,90 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_tiled_k(const void* coo
   }
 }
 
+// Level sweep: the same work with the whole grid resident at once.  A thread keeps the packed results of all its
+// PPT points' levels in registers and stores finished 64-byte rows at the end; nothing is staged in LDS, so
+// a launch of ceil(N / (256 * PPT)) workgroups fits the chip in one round up to about a million points.  Workgroups
+// that start together and do the same work per level stay together: at any moment an XCD's L2 serves the gathers of
+// one or two level tables, not of all of them (a workgroup that runs ahead fetches cold lines and falls back, one
+// that lags finds them warm and catches up).  With workgroups that start at different times, as in the staged
+// kernel's several rounds, every level's table competes for L2 at once.
+template <typename TT, int PPT>
+__global__ __launch_bounds__(TILE_THREADS) void hash_fwd_sweep_k(const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                                 const uint32_t* table, uint16_t* out, int64_t out_stride,
+                                                                 int64_t N, DevGeom g, const int64_t* primes, float scale) {
+  constexpr int P = TILE_THREADS * PPT;
+  constexpr int LMAX = 16;
+  const int t = threadIdx.x;
+  const int64_t p0 = (int64_t)blockIdx.x * P;
+  const int L = g.levels;
+  float x[PPT][3];
+#pragma unroll
+  for (int i = 0; i < PPT; ++i) {
+    int64_t n = p0 + t + TILE_THREADS * i;
+    if (n >= N) n = N - 1;
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+      float v = load_as_f32(coords, n * csn + d * csd, cdt);
+      x[i][d] = scale != 1.0f ? v / scale : v;
+    }
+  }
+  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], (uint32_t)primes[2]};
+  uint32_t enc[PPT][LMAX];
+#pragma unroll
+  for (int l = 0; l < LMAX; ++l) {
+    if (l < L) {
+      const uint32_t res = (uint32_t)g.res[l];
+      const float fres = (float)g.res[l];
+      const bool hashed = l >= g.first_hash;
+      const uint32_t mask = g.rows[l] - 1;
+      const uint32_t* tab = table + g.row_offset[l];
+#pragma unroll
+      for (int i0 = 0; i0 < PPT; i0 += 2) {
+        uint32_t v[2][8];
+        float w[2][8];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          uint32_t c[3];
+          float fr[3];
+#pragma unroll
+          for (int d = 0; d < 3; ++d) {
+            const float pos = x[i0 + i][d] * fres;
+            const float fl = floorf(pos);
+            c[d] = (uint32_t)(int)fl;
+            fr[d] = pos - fl;
+          }
+          const Corner8 r = rows_d3(c, hashed, res, mask, pi);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) v[i][j] = tab[r.row[j]];
+          weights_d3(fr, w[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            a0 = a0 + w[i][j] * TT::to_f32((uint16_t)(v[i][j] & 0xffffu));
+            a1 = a1 + w[i][j] * TT::to_f32((uint16_t)(v[i][j] >> 16));
+          }
+          enc[i0 + i][l] = (uint32_t)TT::from_f32(a0) | ((uint32_t)TT::from_f32(a1) << 16);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) enc[i][l] = 0u;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < PPT; ++i) {
+    const int64_t n = p0 + t + TILE_THREADS * i;
+    if (n >= N) continue;
+    uint4* dst = reinterpret_cast<uint4*>(out + n * out_stride);
+#pragma unroll
+    for (int q = 0; q < LMAX / 4; ++q)
+      if (4 * q < L) dst[q] = make_uint4(enc[i][4 * q], enc[i][4 * q + 1], enc[i][4 * q + 2], enc[i][4 * q + 3]);
+  }
+}
+
 template <typename GT, int PPT>
 __global__ __launch_bounds__(TILE_THREADS) void hash_bwd_tiled_k(const void* coords, int cdt, int64_t csn, int64_t csd,
                                                                  const uint16_t* dout, int64_t dout_stride,
@@ -313,6 +397,8 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_bwd_tiled_k(const void* coo
 // ---------------------------------------------------------------------------
 // below this many points the scattered-atomic kernels are faster than planning + scanning
 constexpr int64_t SCAN_MIN_POINTS = 32768;
+constexpr int SWEEP_PPT = 4;
+constexpr int64_t SWEEP_MIN_POINTS = (int64_t)256 * TILE_THREADS * SWEEP_PPT;
 
 static bool tiled_ok(const nf_hash_geom* g, int table_dt, const void* rows_ptr, int64_t row_stride) {
   if (g->dims != 3 || g->feat != 2 || table_dt == NF_F32) return false;
@@ -367,6 +453,21 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
   NF_REQUIRE(n_points <= ((int64_t)1 << 31) * 256 - 1, NF_EINVAL, "n_points too large");
   hipStream_t s = (hipStream_t)stream;
 
+  // The level sweep wants at least one workgroup per compute unit; below that the staged kernel's smaller tiles
+  // spread the points over more of the chip.
+  if (!(flags & (NF_HASH_FORCE_GENERIC | NF_HASH_FWD_STAGED)) && n_points >= SWEEP_MIN_POINTS &&
+      tiled_ok(geom, table_dtype, out, out_stride_n)) {
+    constexpr int PPT = SWEEP_PPT;
+    constexpr int P = TILE_THREADS * PPT;
+    dim3 grid((unsigned)((n_points + P - 1) / P));
+    if (table_dtype == NF_F16)
+      hipLaunchKernelGGL((hash_fwd_sweep_k<F16, PPT>), grid, dim3(TILE_THREADS), 0, s, coords, coords_dtype, csn, csd,
+                         (const uint32_t*)table, (uint16_t*)out, out_stride_n, n_points, g, primes, scale);
+    else
+      hipLaunchKernelGGL((hash_fwd_sweep_k<BF16, PPT>), grid, dim3(TILE_THREADS), 0, s, coords, coords_dtype, csn, csd,
+                         (const uint32_t*)table, (uint16_t*)out, out_stride_n, n_points, g, primes, scale);
+    return check_launch("hash_fwd_sweep");
+  }
   if (!(flags & NF_HASH_FORCE_GENERIC) && tiled_ok(geom, table_dtype, out, out_stride_n)) {
     constexpr int PPT = 2;
     constexpr int P = TILE_THREADS * PPT;
