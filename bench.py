@@ -245,6 +245,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one out-of-place add over 256 MiB (a copy kernel of known traffic, for scaling "
                          "the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
+    ap.add_argument("--hash-kernel-flags", type=int, default=0,
+                    help="NF_HASH_* flag bits passed to the hash-encoding entry points (profiling the alternative "
+                         "kernels, e.g. 8 = LDS-staged forward); the default 0 is what the bench line is quoted on")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (points are independent, so the work "
@@ -254,11 +257,14 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if args.hash_kernel_flags:
+        from triton_helpers_amd.layers.hash_encoding import kernel as hk
+        hk._FLAGS = args.hash_kernel_flags
 
     h = bench_hash(args.steps, args.warmup)
     # The forward is one kernel (hash_fwd_sweep_k); the backward is zero + count + offsets + fill + accumulate, each
     # shorter than the forward kernel.
-    dom, dom_ms, dom_bytes = "hash_fwd_sweep_k", h["t_fwd"], FWD_BYTES_PER_POINT * N_POINTS
+    dom, dom_ms, dom_bytes = ("hash_fwd_tiled_k" if args.hash_kernel_flags & 8 else "hash_fwd_sweep_k"), h["t_fwd"], FWD_BYTES_PER_POINT * N_POINTS
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
     bwd_achieved = BWD_BYTES_PER_POINT * N_POINTS / (h["t_bwd"] * 1e-3) / 1e9
     step_bytes = (FWD_BYTES_PER_POINT + BWD_BYTES_PER_POINT) * N_POINTS + h["E"] * F * 4
