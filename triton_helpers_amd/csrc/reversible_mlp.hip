@@ -72,6 +72,24 @@ __device__ __forceinline__ void store_tile_packed(uint16_t* base, int64_t stride
   }
 }
 
+// The same tiles when the caller knows that H is the padded width, that every row allows 8-byte accesses and that
+// no chunk is ragged: one address per (tensor, row tile), the column part is an immediate offset.
+template <bool FAST>
+__device__ __forceinline__ uint2 ld_tile(const uint16_t* base, int64_t stride, int64_t row0, int64_t rows, int col0,
+                                         int width, int mt, int lane, bool vec_ok) {
+  if (FAST) return *reinterpret_cast<const uint2*>(base + (row0 + (lane & 15)) * stride + 4 * (lane >> 4) + col0 + 16 * mt);
+  return load_tile_packed(base, stride, row0, rows, col0, width, mt, lane, vec_ok);
+}
+template <bool FAST>
+__device__ __forceinline__ void st_tile(uint16_t* base, int64_t stride, int64_t row0, int64_t rows, int col0, int width,
+                                        int mt, int lane, uint2 v, bool vec_ok) {
+  if (FAST) {
+    *reinterpret_cast<uint2*>(base + (row0 + (lane & 15)) * stride + 4 * (lane >> 4) + col0 + 16 * mt) = v;
+    return;
+  }
+  store_tile_packed(base, stride, row0, rows, col0, width, mt, lane, v, vec_ok);
+}
+
 template <typename T>
 __device__ __forceinline__ f32x4_t unpack4(uint2 v) {
   f32x4_t o = {unpack_lo<T>(v.x), unpack_hi<T>(v.x), unpack_lo<T>(v.y), unpack_hi<T>(v.y)};
@@ -124,7 +142,7 @@ __device__ __forceinline__ void stage_bias_row(float* dst, const uint16_t* b, in
 // Forward: up to FWD_GROUP blocks per launch
 // ---------------------------------------------------------------------------------------
 // ACT >= 0 fixes the activation at compile time (no per-element selection); -1 reads it from the arguments.
-template <typename T, int HP, int ACT>
+template <typename T, int HP, int ACT, bool FAST>
 __global__ __launch_bounds__(768) void rev_fwd_k(RevArgs a) {
   constexpr int MT = HP / 16, KC = HP / 32, LAYER = MT * KC * RFRAG;
   const int act = ACT >= 0 ? ACT : a.act;
@@ -133,7 +151,7 @@ __global__ __launch_bounds__(768) void rev_fwd_k(RevArgs a) {
   const int tid = threadIdx.x, nthreads = blockDim.x, lane = tid & 63, wave = tid >> 6;
   uint16_t* frags = reinterpret_cast<uint16_t*>(smem);  // [nblocks][F.w1, F.w2, G.w1, G.w2][LAYER]
   float* bias = reinterpret_cast<float*>(frags + (size_t)a.nblocks * 4 * LAYER);  // [nblocks][4][HP]
-  const int H = a.half;
+  const int H = FAST ? HP : a.half;
   for (int k = 0; k < a.nblocks; ++k)
     for (int s = 0; s < 2; ++s) {
       const size_t sub = (size_t)(2 * k + s);
@@ -152,8 +170,8 @@ __global__ __launch_bounds__(768) void rev_fwd_k(RevArgs a) {
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        s1[nt][mt] = unpack4<T>(load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in));
-        s2[nt][mt] = unpack4<T>(load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_in));
+        s1[nt][mt] = unpack4<T>(ld_tile<FAST>(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in));
+        s2[nt][mt] = unpack4<T>(ld_tile<FAST>(a.in, a.in_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_in));
       }
     for (int k = 0; k < a.nblocks; ++k) {
 #pragma unroll
@@ -193,8 +211,8 @@ __global__ __launch_bounds__(768) void rev_fwd_k(RevArgs a) {
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        store_tile_packed(a.out, a.out_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, pack4<T>(s1[nt][mt]), a.vec_out);
-        store_tile_packed(a.out, a.out_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, pack4<T>(s2[nt][mt]), a.vec_out);
+        st_tile<FAST>(a.out, a.out_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, pack4<T>(s1[nt][mt]), a.vec_out);
+        st_tile<FAST>(a.out, a.out_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, pack4<T>(s2[nt][mt]), a.vec_out);
       }
   }
 }
@@ -326,13 +344,13 @@ __device__ __forceinline__ void flush_tile(float* dw, int dim, int mt, int nt, i
     if (r0 + r < dim) unsafeAtomicAdd(dw + (size_t)(r0 + r) * dim + c, v[r]);
 }
 
-template <typename T, int HP, int ACT>
+template <typename T, int HP, int ACT, bool FAST>
 __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
   constexpr int MT = HP / 16, KC = HP / 32, LAYER = MT * KC * RFRAG;
   const int act = ACT >= 0 ? ACT : a.act;
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, nthreads = blockDim.x, lane = tid & 63, wave = tid >> 6;
-  const int H = a.half;
+  const int H = FAST ? HP : a.half;
   // weights: forward-form [F.w1, F.w2, G.w1, G.w2], transposed-form the same order
   uint16_t* fw = reinterpret_cast<uint16_t*>(smem);
   uint16_t* tw = fw + 4 * LAYER;
@@ -377,15 +395,15 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          y1[nt][mt] = load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in);
-          d2[nt][mt] = load_tile_packed(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_dy);
+          y1[nt][mt] = ld_tile<FAST>(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in);
+          d2[nt][mt] = ld_tile<FAST>(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_dy);
         }
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          y2[nt][mt] = load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_in);
-          dy1[nt][mt] = load_tile_packed(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_dy);
+          y2[nt][mt] = ld_tile<FAST>(a.in, a.in_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_in);
+          dy1[nt][mt] = ld_tile<FAST>(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_dy);
         }
       // ---- G:  y2 = x2 + G(y1)  =>  x2 = y2 - G(y1),  dy1 += (dG/dy1)^T dy2
       sub_backward<T, MT, KC, ACT>(y1, d2, sout, du, dwG1, dwG2, g2acc, dbG1, dbG2, fw + 2 * LAYER, fw + 3 * LAYER,
@@ -405,8 +423,8 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          y1[nt][mt] = load_tile_packed(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in);
-          d2[nt][mt] = load_tile_packed(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_dy);
+          y1[nt][mt] = ld_tile<FAST>(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in);
+          d2[nt][mt] = ld_tile<FAST>(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_dy);
         }
       // ---- F:  y1 = x1 + F(x2)  =>  x1 = y1 - F(x2),  dx2 = dy2 + (dF/dx2)^T dy1
       sub_backward<T, MT, KC, ACT>(x2, d1, sout, du, dwF1, dwF2, nullptr, dbF1, dbF2, fw, fw + LAYER, tw, tw + LAYER, bias,
@@ -417,10 +435,10 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
         for (int mt = 0; mt < MT; ++mt) {
           const uint2 x1 = pack4<T>(unpack4<T>(y1[nt][mt]) - sout[nt][mt]);
           const uint2 dx2 = pack4<T>(unpack4<T>(d2[nt][mt]) + du[nt][mt]);
-          store_tile_packed(a.out, a.out_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, x1, a.vec_out);
-          store_tile_packed(a.out, a.out_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, x2[nt][mt], a.vec_out);
-          store_tile_packed(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, d1[nt][mt], a.vec_dx);
-          store_tile_packed(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, dx2, a.vec_dx);
+          st_tile<FAST>(a.out, a.out_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, x1, a.vec_out);
+          st_tile<FAST>(a.out, a.out_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, x2[nt][mt], a.vec_out);
+          st_tile<FAST>(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, d1[nt][mt], a.vec_dx);
+          st_tile<FAST>(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, dx2, a.vec_dx);
         }
     }
   }
@@ -532,9 +550,13 @@ static int launch_rev_fwd(RevArgs a, hipStream_t s) {
   int64_t blocks = (chunks + waves - 1) / waves;
   const int64_t cap = (int64_t)rev_cus() * (lds > 80 * 1024 ? 1 : 2);
   if (blocks > cap) blocks = cap;
-  const void* kern = a.act == NF_ACT_GELU   ? (const void*)rev_fwd_k<T, HP, NF_ACT_GELU>
-                     : a.act == NF_ACT_RELU ? (const void*)rev_fwd_k<T, HP, NF_ACT_RELU>
-                                            : (const void*)rev_fwd_k<T, HP, -1>;
+  // full-width, aligned, unragged calls of the two common activations take the variants without per-tile checks
+  const bool fast = a.half == HP && a.rows % 32 == 0 && a.vec_in && a.vec_out;
+  const void* kern = a.act == NF_ACT_GELU   ? (fast ? (const void*)rev_fwd_k<T, HP, NF_ACT_GELU, true>
+                                                    : (const void*)rev_fwd_k<T, HP, NF_ACT_GELU, false>)
+                     : a.act == NF_ACT_RELU ? (fast ? (const void*)rev_fwd_k<T, HP, NF_ACT_RELU, true>
+                                                    : (const void*)rev_fwd_k<T, HP, NF_ACT_RELU, false>)
+                                            : (const void*)rev_fwd_k<T, HP, -1, false>;
   if (lds > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
@@ -557,9 +579,12 @@ static int launch_rev_bwd(RevArgs a, hipStream_t s) {
   // the weight-gradient accumulators take most of the register file: one wave per SIMD
   const int64_t cap = (int64_t)rev_cus();
   if (blocks > cap) blocks = cap;
-  const void* kern = a.act == NF_ACT_GELU   ? (const void*)rev_bwd_block_k<T, HP, NF_ACT_GELU>
-                     : a.act == NF_ACT_RELU ? (const void*)rev_bwd_block_k<T, HP, NF_ACT_RELU>
-                                            : (const void*)rev_bwd_block_k<T, HP, -1>;
+  const bool fast = a.half == HP && a.rows % 32 == 0 && a.vec_in && a.vec_out && a.vec_dy && a.vec_dx;
+  const void* kern = a.act == NF_ACT_GELU   ? (fast ? (const void*)rev_bwd_block_k<T, HP, NF_ACT_GELU, true>
+                                                    : (const void*)rev_bwd_block_k<T, HP, NF_ACT_GELU, false>)
+                     : a.act == NF_ACT_RELU ? (fast ? (const void*)rev_bwd_block_k<T, HP, NF_ACT_RELU, true>
+                                                    : (const void*)rev_bwd_block_k<T, HP, NF_ACT_RELU, false>)
+                                            : (const void*)rev_bwd_block_k<T, HP, -1, false>;
   if (lds > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
