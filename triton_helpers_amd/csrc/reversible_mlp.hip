@@ -4,9 +4,10 @@
 //
 // Forward: one launch runs up to FWD_GROUP coupling blocks with all their weights resident
 // in LDS; the two halves of the residual stream stay in float32 registers between blocks.
-// Backward: one launch per coupling block, last block first.  It takes the block's OUTPUT
-// (y, dy), rebuilds the block's input in-kernel (x2 = y2 - G(y1), x1 = y1 - F(x2)) while it
-// back-propagates, and writes (x, dx), which the next launch reads in place.  No activation
+// Backward: one launch walks the coupling blocks, last block first, a wave keeping its rows.  For
+// each block it takes the block's OUTPUT (y, dy), rebuilds the block's input in-kernel
+// (x2 = y2 - G(y1), x1 = y1 - F(x2)) while it back-propagates, and writes (x, dx), which it reads
+// back in place for the block below after restaging that block's weights.  No activation
 // of the forward pass is ever stored.  The four weight gradients of a block accumulate in
 // float32 registers over the wave's whole row loop; their operands (rows along K) are matrix-core
 // transposes of the row-per-lane fragments, so LDS only holds weights.
@@ -29,8 +30,8 @@ struct RevArgs {
   int64_t dy_stride;
   uint16_t* dx;
   int64_t dx_stride;
-  const uint16_t *w1, *b1, *w2, *b2;  // already offset to the first block of this launch
-  float *dw1, *db1, *dw2, *db2;       // already offset to this block (backward)
+  const uint16_t *w1, *b1, *w2, *b2;  // first coupling of this launch
+  float *dw1, *db1, *dw2, *db2;       // first coupling of this launch (backward)
   int64_t rows;
   int half, nblocks, act;
   int vec_in, vec_out, vec_dy, vec_dx;
@@ -359,15 +360,35 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
   // layer products: at HP = 64 the fourth (G's second layer) lives in LDS, 16 KiB per wave.
   constexpr bool G2_LDS = HP > 32;
   f32x4_t* g2acc = G2_LDS ? reinterpret_cast<f32x4_t*>(bias + 4 * HP) + (size_t)wave * MT * MT * 64 : nullptr;
+  const Frag sel[2] = {sel_frag<T>(0, lane), sel_frag<T>(1, lane)};
+  const f32x4_t zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+  const int64_t n_chunks = (a.rows + 31) / 32;
+
+  // The couplings of the launch, last first.  A wave owns the same rows in every coupling, so it reads (x, dx) of the
+  // coupling above from where it wrote them itself and no workgroup ever waits for another; the weight-gradient
+  // atomics of one coupling drain while the next is being computed.
+  // (Only the variant without per-tile checks loops; the general one is launched once per coupling.)
+  for (int kb = FAST ? a.nblocks - 1 : 0; kb >= 0; --kb) {
+  const bool top = FAST ? kb == a.nblocks - 1 : true;
+  const uint16_t* in_p = top ? a.in : a.out;
+  const int64_t in_s = top ? a.in_stride : a.out_stride;
+  const bool in_v = top ? a.vec_in : a.vec_out;
+  const uint16_t* dy_p = top ? a.dy : a.dx;
+  const int64_t dy_s = top ? a.dy_stride : a.dx_stride;
+  const bool dy_v = top ? a.vec_dy : a.vec_dx;
+  const uint16_t* w1 = a.w1 + (size_t)2 * kb * H * H;
+  const uint16_t* w2 = a.w2 + (size_t)2 * kb * H * H;
+  const uint16_t* b1 = a.b1 ? a.b1 + (size_t)2 * kb * H : nullptr;
+  const uint16_t* b2 = a.b2 ? a.b2 + (size_t)2 * kb * H : nullptr;
   if (G2_LDS)
     for (int i = lane; i < MT * MT * 64; i += 64) g2acc[i] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
   for (int s = 0; s < 2; ++s) {
-    stage_weight_frags<true, false>(fw + (2 * s) * LAYER, a.w1 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
-    stage_weight_frags<true, false>(fw + (2 * s + 1) * LAYER, a.w2 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
-    stage_weight_frags<true, true>(tw + (2 * s) * LAYER, a.w1 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
-    stage_weight_frags<true, true>(tw + (2 * s + 1) * LAYER, a.w2 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
-    stage_bias_row<T>(bias + (2 * s) * HP, a.b1 ? a.b1 + (size_t)s * H : nullptr, H, HP, tid, nthreads);
-    stage_bias_row<T>(bias + (2 * s + 1) * HP, a.b2 ? a.b2 + (size_t)s * H : nullptr, H, HP, tid, nthreads);
+    stage_weight_frags<true, false>(fw + (2 * s) * LAYER, w1 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
+    stage_weight_frags<true, false>(fw + (2 * s + 1) * LAYER, w2 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
+    stage_weight_frags<true, true>(tw + (2 * s) * LAYER, w1 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
+    stage_weight_frags<true, true>(tw + (2 * s + 1) * LAYER, w2 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
+    stage_bias_row<T>(bias + (2 * s) * HP, b1 ? b1 + (size_t)s * H : nullptr, H, HP, tid, nthreads);
+    stage_bias_row<T>(bias + (2 * s + 1) * HP, b2 ? b2 + (size_t)s * H : nullptr, H, HP, tid, nthreads);
   }
   __syncthreads();
 
@@ -375,14 +396,11 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
   // lane (feature, g) of tile i: partial bias gradient of feature 16*i + n over the rows of lane group g
   float dbF1[4] = {0.0f, 0.0f, 0.0f, 0.0f}, dbF2[4] = {0.0f, 0.0f, 0.0f, 0.0f}, dbG1[4] = {0.0f, 0.0f, 0.0f, 0.0f},
         dbG2[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  const Frag sel[2] = {sel_frag<T>(0, lane), sel_frag<T>(1, lane)};
-  const f32x4_t zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) dwF1[i][j] = dwF2[i][j] = dwG1[i][j] = dwG2[i][j] = zero4;
 
-  const int64_t n_chunks = (a.rows + 31) / 32;
   for (int64_t chunk = (int64_t)blockIdx.x * 4 + wave; chunk < n_chunks; chunk += (int64_t)gridDim.x * 4) {
     const int64_t row0 = chunk * 32;
     // The halves of y and dy that a sub-MLP's residual adds need are requested before that sub-MLP runs, so their
@@ -395,15 +413,15 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          y1[nt][mt] = ld_tile<FAST>(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in);
-          d2[nt][mt] = ld_tile<FAST>(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_dy);
+          y1[nt][mt] = ld_tile<FAST>(in_p, in_s, row0 + 16 * nt, a.rows, 0, H, mt, lane, in_v);
+          d2[nt][mt] = ld_tile<FAST>(dy_p, dy_s, row0 + 16 * nt, a.rows, H, H, mt, lane, dy_v);
         }
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          y2[nt][mt] = ld_tile<FAST>(a.in, a.in_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_in);
-          dy1[nt][mt] = ld_tile<FAST>(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_dy);
+          y2[nt][mt] = ld_tile<FAST>(in_p, in_s, row0 + 16 * nt, a.rows, H, H, mt, lane, in_v);
+          dy1[nt][mt] = ld_tile<FAST>(dy_p, dy_s, row0 + 16 * nt, a.rows, 0, H, mt, lane, dy_v);
         }
       // ---- G:  y2 = x2 + G(y1)  =>  x2 = y2 - G(y1),  dy1 += (dG/dy1)^T dy2
       sub_backward<T, MT, KC, ACT>(y1, d2, sout, du, dwG1, dwG2, g2acc, dbG1, dbG2, fw + 2 * LAYER, fw + 3 * LAYER,
@@ -423,8 +441,8 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          y1[nt][mt] = ld_tile<FAST>(a.in, a.in_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, a.vec_in);
-          d2[nt][mt] = ld_tile<FAST>(a.dy, a.dy_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, a.vec_dy);
+          y1[nt][mt] = ld_tile<FAST>(in_p, in_s, row0 + 16 * nt, a.rows, 0, H, mt, lane, in_v);
+          d2[nt][mt] = ld_tile<FAST>(dy_p, dy_s, row0 + 16 * nt, a.rows, H, H, mt, lane, dy_v);
         }
       // ---- F:  y1 = x1 + F(x2)  =>  x1 = y1 - F(x2),  dx2 = dy2 + (dF/dx2)^T dy1
       sub_backward<T, MT, KC, ACT>(x2, d1, sout, du, dwF1, dwF2, nullptr, dbF1, dbF2, fw, fw + LAYER, tw, tw + LAYER, bias,
@@ -487,28 +505,36 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
     }
     __syncthreads();
   }
-  if (wave != 0) return;
+  if (wave == 0) {
   // layer order in dw1 / dw2: sub-MLP F is row block 0, G is row block 1 of this coupling block
+  float* gw1 = a.dw1 + (size_t)2 * kb * H * H;
+  float* gw2 = a.dw2 + (size_t)2 * kb * H * H;
+  float* gb1 = a.db1 ? a.db1 + (size_t)2 * kb * H : nullptr;
+  float* gb2 = a.db2 ? a.db2 + (size_t)2 * kb * H : nullptr;
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
-      flush_tile(a.dw1, H, i, j, lane, dwF1[i][j]);
-      flush_tile(a.dw2, H, i, j, lane, dwF2[i][j]);
-      flush_tile(a.dw1 + (size_t)H * H, H, i, j, lane, dwG1[i][j]);
+      flush_tile(gw1, H, i, j, lane, dwF1[i][j]);
+      flush_tile(gw2, H, i, j, lane, dwF2[i][j]);
+      flush_tile(gw1 + (size_t)H * H, H, i, j, lane, dwG1[i][j]);
       if (G2_LDS) {
         constexpr int PER_WAVE = MT * MT * 64;
         const int at = (i * MT + j) * 64 + lane;  // wave 0's g2acc is the first of the four
         dwG2[i][j] = (g2acc[at] + g2acc[PER_WAVE + at]) + (g2acc[2 * PER_WAVE + at] + g2acc[3 * PER_WAVE + at]);
       }
-      flush_tile(a.dw2 + (size_t)H * H, H, i, j, lane, dwG2[i][j]);
+      flush_tile(gw2 + (size_t)H * H, H, i, j, lane, dwG2[i][j]);
     }
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
-    flush_db_rev(a.db1, H, i, lane, dbF1[i]);
-    flush_db_rev(a.db1 ? a.db1 + H : nullptr, H, i, lane, dbG1[i]);
-    flush_db_rev(a.db2, H, i, lane, dbF2[i]);
-    flush_db_rev(a.db2 ? a.db2 + H : nullptr, H, i, lane, dbG2[i]);
+    flush_db_rev(gb1, H, i, lane, dbF1[i]);
+    flush_db_rev(gb1 ? gb1 + H : nullptr, H, i, lane, dbG1[i]);
+    flush_db_rev(gb2, H, i, lane, dbF2[i]);
+    flush_db_rev(gb2 ? gb2 + H : nullptr, H, i, lane, dbG2[i]);
+  }
+  }
+  // wave 0 has read the other waves' LDS accumulators and the reduction area: both are rewritten for the next coupling
+  __syncthreads();
   }
 }
 
@@ -647,9 +673,15 @@ extern "C" int nf_revmlp_bwd(const void* y, int64_t y_stride, const void* dy, in
   NF_REQUIRE(y_stride >= 2 * half && dy_stride >= 2 * half && dx_stride >= 2 * half && x_rec_stride >= 2 * half, NF_EINVAL,
              "row stride smaller than 2*half");
   hipStream_t s = (hipStream_t)stream;
+  // Full-width, aligned, unragged calls of the two common activations take one launch that walks all couplings, last
+  // first (the first reads (y, dy), the others continue in place on (x_rec, dx)); anything else one launch per coupling.
+  const int hp = half <= 32 ? 32 : 64;
+  const bool fused = half == hp && rows % 32 == 0 && (act == NF_ACT_GELU || act == NF_ACT_RELU) && vec8_ok(y, y_stride, half) &&
+                     vec8_ok(x_rec, x_rec_stride, half) && vec8_ok(dy, dy_stride, half) && vec8_ok(dx, dx_stride, half);
   for (int k = blocks - 1; k >= 0; --k) {
     RevArgs a = {};
     const bool first = k == blocks - 1;
+    const int kw = fused ? 0 : k;  // the fused launch offsets per coupling itself
     a.in = (const uint16_t*)(first ? y : x_rec);
     a.in_stride = first ? y_stride : x_rec_stride;
     a.out = (uint16_t*)x_rec;
@@ -658,17 +690,17 @@ extern "C" int nf_revmlp_bwd(const void* y, int64_t y_stride, const void* dy, in
     a.dy_stride = first ? dy_stride : dx_stride;
     a.dx = (uint16_t*)dx;
     a.dx_stride = dx_stride;
-    a.w1 = (const uint16_t*)w1 + (size_t)2 * k * half * half;
-    a.w2 = (const uint16_t*)w2 + (size_t)2 * k * half * half;
-    a.b1 = b1 ? (const uint16_t*)b1 + (size_t)2 * k * half : nullptr;
-    a.b2 = b2 ? (const uint16_t*)b2 + (size_t)2 * k * half : nullptr;
-    a.dw1 = dw1 + (size_t)2 * k * half * half;
-    a.dw2 = dw2 + (size_t)2 * k * half * half;
-    a.db1 = db1 ? db1 + (size_t)2 * k * half : nullptr;
-    a.db2 = db2 ? db2 + (size_t)2 * k * half : nullptr;
+    a.w1 = (const uint16_t*)w1 + (size_t)2 * kw * half * half;
+    a.w2 = (const uint16_t*)w2 + (size_t)2 * kw * half * half;
+    a.b1 = b1 ? (const uint16_t*)b1 + (size_t)2 * kw * half : nullptr;
+    a.b2 = b2 ? (const uint16_t*)b2 + (size_t)2 * kw * half : nullptr;
+    a.dw1 = dw1 + (size_t)2 * kw * half * half;
+    a.dw2 = dw2 + (size_t)2 * kw * half * half;
+    a.db1 = db1 ? db1 + (size_t)2 * kw * half : nullptr;
+    a.db2 = db2 ? db2 + (size_t)2 * kw * half : nullptr;
     a.rows = rows;
     a.half = half;
-    a.nblocks = 1;
+    a.nblocks = fused ? blocks : 1;
     a.act = act;
     a.vec_in = vec8_ok(a.in, a.in_stride, half);
     a.vec_out = vec8_ok(a.out, a.out_stride, half);
@@ -679,7 +711,7 @@ extern "C" int nf_revmlp_bwd(const void* y, int64_t y_stride, const void* dy, in
       rc = dtype == NF_BF16 ? launch_rev_bwd<BF16, 32>(a, s) : launch_rev_bwd<F16, 32>(a, s);
     else
       rc = dtype == NF_BF16 ? launch_rev_bwd<BF16, 64>(a, s) : launch_rev_bwd<F16, 64>(a, s);
-    if (rc) return rc;
+    if (rc || fused) return rc;
   }
   return 0;
 }
