@@ -43,7 +43,12 @@ def _close(got, want, what, scale_rel=False, blocks=4):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("act", ["gelu", "silu", "none"])
 @pytest.mark.parametrize("bias", [False, True])
-@pytest.mark.parametrize("rows,H,blocks", [(1000, 64, 4), (37, 64, 1), (300, 32, 2), (129, 16, 3), (513, 64, 6), (64, 20, 2)])
+@pytest.mark.parametrize(
+    "rows,H,blocks",
+    [(1000, 64, 4), (37, 64, 1), (300, 32, 2), (129, 16, 3), (513, 64, 6), (64, 20, 2),
+     # unragged full-width shapes: GELU takes the kernels without per-tile checks and one backward launch for all couplings
+     (1024, 64, 4), (96, 64, 1), (640, 64, 6), (512, 32, 3)],
+)
 def test_forward_backward(rows, H, blocks, bias, act, dtype):
     rk = _rk()
     torch.manual_seed(0)
@@ -63,6 +68,55 @@ def test_forward_backward(rows, H, blocks, bias, act, dtype):
     for name, leaf in zip(("dw1", "db1", "dw2", "db2"), leaves):
         if leaf is not None:
             _close(leaf.grad, want[name], name, scale_rel=True, blocks=blocks)
+
+
+def _misaligned(t):
+    """The same values as a view whose rows start 2 bytes off an 8-byte boundary (forces the checked-tile kernels)."""
+    buf = torch.zeros(t.shape[0], t.shape[1] + 4, dtype=t.dtype, device=t.device)
+    view = buf[:, 1 : 1 + t.shape[1]]
+    view.copy_(t)
+    assert view.data_ptr() % 8 != 0
+    return view
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("act", ["gelu", "relu"])
+@pytest.mark.parametrize("rows,H,blocks", [(4096, 64, 4), (1024, 32, 2), (288, 64, 5)])
+def test_unchecked_and_checked_kernels_agree(rows, H, blocks, act, dtype):
+    """Aligned unragged calls run the kernels without per-tile checks (the backward as one launch over all
+    couplings); a misaligned view of the same data runs the checked kernels, one backward launch per coupling.
+    Same arithmetic per row: y and dx must agree bit for bit, the weight gradients up to the order of their float32
+    atomics.  (This is also what covers ReLU's backward, which the oracle comparison leaves out.)"""
+    rk = _rk()
+    torch.manual_seed(1)
+    w1, b1, w2, b2 = (t.to(DEV) for t in _params(blocks, H, True, dtype))
+    x = torch.randn(rows, 2 * H, device=DEV).to(dtype)
+    dy = torch.randn(rows, 2 * H, device=DEV).to(dtype)
+    results = []
+    for variant in (lambda t: t, _misaligned):
+        leaves = [t.clone().requires_grad_(True) for t in (w1, b1, w2, b2)]
+        xv = variant(x).detach().requires_grad_(True)
+        y = rk.reversible_mlp(xv, *leaves, act)
+        y.backward(variant(dy))
+        results.append((y.detach(), xv.grad, [t.grad for t in leaves]))
+    (y0, dx0, g0), (y1, dx1, g1) = results
+    assert torch.equal(y0, y1)
+    assert torch.equal(dx0, dx1)
+    for a, b in zip(g0, g1):
+        scale = float(b.float().abs().max())
+        torch.testing.assert_close(a.float(), b.float(), rtol=1e-2, atol=1e-2 * scale)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,H,blocks", [(1000, 64, 4), (1024, 64, 4), (512, 32, 3)])
+def test_relu_forward(rows, H, blocks, dtype):
+    rk = _rk()
+    torch.manual_seed(0)
+    w1, b1, w2, b2 = _params(blocks, H, True, dtype)
+    x = torch.randn(rows, 2 * H).to(dtype)
+    want_y = R.rev_forward(x, w1, b1, w2, b2, "relu", round_to=dtype, stream_round_every=4).to(dtype)
+    y = rk.reversible_mlp(x.to(DEV), *(t.to(DEV) for t in (w1, b1, w2, b2)), "relu")
+    _close(y, want_y, "y", blocks=blocks)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
