@@ -123,6 +123,19 @@ __device__ __forceinline__ uint32_t wave_rank(uint32_t* cnt, uint32_t bin, bool 
   return rank;
 }
 
+// Largest value of a wave, valid in lane 63: prefix maxima inside each row of 16 lanes, then lane 15 of rows 0 / 2 into
+// rows 1 / 3 and lane 31 into rows 2 / 3 (data-parallel primitives of the vector ALU; nothing goes through LDS).
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t m) {
+  auto step = [](uint32_t v, uint32_t shifted) { return shifted > v ? shifted : v; };
+  m = step(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x111, 0xf, 0xf, false));  // row_shr:1
+  m = step(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x112, 0xf, 0xf, false));  // row_shr:2
+  m = step(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x114, 0xf, 0xf, false));  // row_shr:4
+  m = step(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x118, 0xf, 0xf, false));  // row_shr:8
+  m = step(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x142, 0xa, 0xf, false));  // row_bcast:15 -> rows 1, 3
+  m = step(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x143, 0xc, 0xf, false));  // row_bcast:31 -> rows 2, 3
+  return m;
+}
+
 __global__ void hash_bwd_bin_zero_k(uint32_t* p, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0u;
@@ -239,9 +252,8 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
                                                                    uint3* records) {
   extern __shared__ __align__(16) unsigned char fill_smem[];
   const int NB = bp.binbase[bp.n_levels];
-  uint3* stage = reinterpret_cast<uint3*>(fill_smem);                     // [FILL_RECORDS] records sorted by bin
-  uint16_t* binid = reinterpret_cast<uint16_t*>(stage + FILL_RECORDS);    // bin (within the level) of each staged record
-  uint32_t* cur = reinterpret_cast<uint32_t*>(binid + FILL_RECORDS);      // [NB] next staged position of a bin
+  uint4* stage = reinterpret_cast<uint4*>(fill_smem);                     // [FILL_RECORDS] {record, its place in `records`}, sorted by bin
+  uint32_t* cur = reinterpret_cast<uint32_t*>(stage + FILL_RECORDS);      // [NB] next staged position of a bin
   uint32_t* delta = cur + NB;                                             // [NB] global minus staged position
   uint32_t* totals = delta + NB;                                          // [levels] records of this workgroup per level
   uint32_t* lmax = totals + NF_MAX_LEVELS;                                // [levels] largest |dout| pattern
@@ -313,13 +325,8 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
     {
       // largest |g| of the level: positive 16-bit float patterns order like integers
       const uint32_t pk = packed & 0x7fff7fffu;
-      uint32_t m = (pk & 0xffffu) > (pk >> 16) ? (pk & 0xffffu) : (pk >> 16);
-#pragma unroll
-      for (int d = 1; d < 64; d <<= 1) {
-        const uint32_t o = (uint32_t)__shfl_xor((int)m, d);
-        m = o > m ? o : m;
-      }
-      if (lane == 0 && m) atomicMax(lmax + l, m);
+      const uint32_t m = wave_max_u32((pk & 0xffffu) > (pk >> 16) ? (pk & 0xffffu) : (pk >> 16));
+      if (lane == 63 && m) atomicMax(lmax + l, m);
     }
     {
       const Located3 q = locate(v, (float)g.res[l]);
@@ -336,8 +343,8 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
         else if (nb <= AGG_MAX_BINS) pos = wave_rank(lcur, b0, valid, lane);
         else pos = valid ? atomicAdd(lcur + b0, 1u) : 0u;
         if (valid) {
-          stage[pos] = make_record(r0 & BIN_MASK, (split ? r0 : r1) & BIN_MASK, w[2 * c], split ? 0.0f : w[2 * c + 1], packed);
-          binid[pos] = (uint16_t)b0;
+          const uint3 rec = make_record(r0 & BIN_MASK, (split ? r0 : r1) & BIN_MASK, w[2 * c], split ? 0.0f : w[2 * c + 1], packed);
+          stage[pos] = make_uint4(rec.x, rec.y, rec.z, pos + ldelta[b0]);
         }
         if (nb > 1 && __any(valid && split)) {
           const bool on = valid && split;
@@ -345,15 +352,18 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
           if (nb <= AGG_MAX_BINS) pos1 = wave_rank(lcur, b1, on, lane);
           else pos1 = on ? atomicAdd(lcur + b1, 1u) : 0u;
           if (on) {
-            stage[pos1] = make_record(r1 & BIN_MASK, r1 & BIN_MASK, w[2 * c + 1], 0.0f, packed);
-            binid[pos1] = (uint16_t)b1;
+            const uint3 rec = make_record(r1 & BIN_MASK, r1 & BIN_MASK, w[2 * c + 1], 0.0f, packed);
+            stage[pos1] = make_uint4(rec.x, rec.y, rec.z, pos1 + ldelta[b1]);
           }
         }
       }
     }
     lds_barrier();
     const uint32_t total = totals[l];
-    for (uint32_t i = tid; i < total; i += FILL_POINTS) records[i + ldelta[binid[i]]] = stage[i];
+    for (uint32_t i = tid; i < total; i += FILL_POINTS) {
+      const uint4 e = stage[i];
+      records[e.w] = make_uint3(e.x, e.y, e.z);
+    }
     lds_barrier();  // the next level overwrites the stage
   }
   if (tid < bp.n_levels) {
@@ -532,7 +542,7 @@ int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const 
                      ws.tasks, NB, max_tasks);
   if (int rc = check_launch("hash_bwd_bin_offsets")) return rc;
   {
-    const size_t lds = (size_t)FILL_RECORDS * (sizeof(uint3) + sizeof(uint16_t)) + ((size_t)2 * NB + 2 * NF_MAX_LEVELS) * 4;
+    const size_t lds = (size_t)FILL_RECORDS * sizeof(uint4) + ((size_t)2 * NB + 2 * NF_MAX_LEVELS) * 4;
     hipError_t e = hipFuncSetAttribute((const void*)hash_bwd_bin_fill_k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     hipLaunchKernelGGL(hash_bwd_bin_fill_k, dim3(blocks), dim3(FILL_POINTS), lds, s, coords, cdt, csn, csd,
