@@ -379,7 +379,9 @@ template <typename GT>
 __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const uint3* records, const uint4* tasks,
                                                                     const uint32_t* n_tasks, const uint32_t* gmax, float* dtable,
                                                                     DevGeom g, BinPlan bp) {
-  extern __shared__ unsigned long long acc_tile[];  // [BIN_ROWS][2] fixed-point sums
+  // Fixed-point sums, one plane of BIN_ROWS 64-bit cells per feature: the 64 lanes of an add go to random rows of one
+  // feature, and with 8-byte cells those spread over all 64 banks (interleaved features would leave them half).
+  extern __shared__ unsigned long long acc_tile[];
   if (blockIdx.x >= *n_tasks) return;
   const int tid = threadIdx.x;
   const uint4 task = tasks[blockIdx.x];
@@ -400,7 +402,7 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const uint3*
   }
   // two steps stay inside float range; the weight decode rides on the second
   const float s_lo = nonfinite ? 0.0f : ldexpf(1.0f, se / 2), s_hi = ldexpf(1.0f, se - se / 2) * (1.0f / (float)W_MAX);
-  for (uint32_t i = tid; i < 2u * nrows; i += ACC_THREADS) acc_tile[i] = 0ull;
+  for (uint32_t i = tid; i < 2u * nrows; i += ACC_THREADS) acc_tile[(i & 1u) * BIN_ROWS + (i >> 1)] = 0ull;
   lds_barrier();
   // the next round's records are loaded before this round's adds
   uint3 q[ACC_INFLIGHT];
@@ -437,7 +439,7 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const uint3*
     for (int k = 0; k < ACC_INFLIGHT; ++k)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        if (f[k][j]) atomicAdd(acc_tile + 2u * slot[k][j >> 1] + (uint32_t)(j & 1), (unsigned long long)(long long)f[k][j]);
+        if (f[k][j]) atomicAdd(acc_tile + (uint32_t)(j & 1) * BIN_ROWS + slot[k][j >> 1], (unsigned long long)(long long)f[k][j]);
   }
   lds_barrier();
   float* dst = dtable + (g.row_offset[l] + (int64_t)row0) * 2;
@@ -449,7 +451,7 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const uint3*
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t i = i0 + u * ACC_THREADS + tid;
-      const long long a = i < nvals ? (long long)acc_tile[i] : 0ll;
+      const long long a = i < nvals ? (long long)acc_tile[(i & 1u) * BIN_ROWS + (i >> 1)] : 0ll;
       // |a| < 2^48 is exact in double and so is the division by 2^se: one rounding, to float, at the end
       x[u] = a == 0 ? 0.0f : (float)ldexp((double)a, -se);
       if (nonfinite && a != 0) x[u] = qnan;
