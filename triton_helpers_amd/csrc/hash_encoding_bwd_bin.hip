@@ -445,7 +445,7 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const uint3*
   float* dst = dtable + (g.row_offset[l] + (int64_t)row0) * 2;
   const float qnan = __uint_as_float(0x7fc00000u);
   const uint32_t nvals = 2u * nrows;
-  constexpr int U = 4;  // values per thread whose table reads are in flight together
+  constexpr int U = 16;  // values per thread whose table reads are in flight together (a full bin in one pass)
   for (uint32_t i0 = 0; i0 < nvals; i0 += ACC_THREADS * U) {
     float x[U], old[U];
 #pragma unroll
