@@ -333,27 +333,51 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
       const Corner8 r = rows_d3(q.c, l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi);
       float w[8];
       weights_d3(q.fr, w);
+      // The four x-pairs of the point: their ranks are asked for together, so that a wave waits for LDS once per level
+      // and not once per pair.
+      uint32_t b0[4], b1[4], pos[4], dlt[4];
+      bool split[4];
+      bool any_split = false;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        const uint32_t r0 = r.row[2 * c], r1 = r.row[2 * c + 1];
-        const uint32_t b0 = r0 >> BIN_ROWS_LOG2, b1 = r1 >> BIN_ROWS_LOG2;
-        const bool split = b1 != b0;
-        uint32_t pos;
-        if (nb == 1) pos = (uint32_t)tid * 4u + (uint32_t)c;  // the valid points are the first of the workgroup
-        else if (nb <= AGG_MAX_BINS) pos = wave_rank(lcur, b0, valid, lane);
-        else pos = valid ? atomicAdd(lcur + b0, 1u) : 0u;
-        if (valid) {
-          const uint3 rec = make_record(r0 & BIN_MASK, (split ? r0 : r1) & BIN_MASK, w[2 * c], split ? 0.0f : w[2 * c + 1], packed);
-          stage[pos] = make_uint4(rec.x, rec.y, rec.z, pos + ldelta[b0]);
+        b0[c] = r.row[2 * c] >> BIN_ROWS_LOG2;
+        b1[c] = r.row[2 * c + 1] >> BIN_ROWS_LOG2;
+        split[c] = b1[c] != b0[c];
+        any_split = any_split || split[c];
+      }
+      if (nb == 1) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) pos[c] = (uint32_t)tid * 4u + (uint32_t)c;  // the valid points are the first of the workgroup
+      } else if (nb <= AGG_MAX_BINS) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) pos[c] = wave_rank(lcur, b0[c], valid, lane);
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) pos[c] = valid ? atomicAdd(lcur + b0[c], 1u) : 0u;
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c) dlt[c] = ldelta[b0[c]];
+      if (valid) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const uint32_t r0 = r.row[2 * c], r1 = r.row[2 * c + 1];
+          const uint3 rec = make_record(r0 & BIN_MASK, (split[c] ? r0 : r1) & BIN_MASK, w[2 * c], split[c] ? 0.0f : w[2 * c + 1], packed);
+          stage[pos[c]] = make_uint4(rec.x, rec.y, rec.z, pos[c] + dlt[c]);
         }
-        if (nb > 1 && __any(valid && split)) {
-          const bool on = valid && split;
+      }
+      // a pair that straddles two bins leaves its second corner as a record of its own (rare)
+      if (nb > 1 && __any(valid && any_split)) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const bool on = valid && split[c];
+          if (!__any(on)) continue;
           uint32_t pos1;
-          if (nb <= AGG_MAX_BINS) pos1 = wave_rank(lcur, b1, on, lane);
-          else pos1 = on ? atomicAdd(lcur + b1, 1u) : 0u;
+          if (nb <= AGG_MAX_BINS) pos1 = wave_rank(lcur, b1[c], on, lane);
+          else pos1 = on ? atomicAdd(lcur + b1[c], 1u) : 0u;
           if (on) {
+            const uint32_t r1 = r.row[2 * c + 1];
             const uint3 rec = make_record(r1 & BIN_MASK, r1 & BIN_MASK, w[2 * c + 1], 0.0f, packed);
-            stage[pos1] = make_uint4(rec.x, rec.y, rec.z, pos1 + ldelta[b1]);
+            stage[pos1] = make_uint4(rec.x, rec.y, rec.z, pos1 + ldelta[b1[c]]);
           }
         }
       }
