@@ -232,13 +232,14 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_tiled_k(const void* coo
   }
 }
 
-// Level sweep: the same work with the whole grid resident at once.  A thread keeps the packed results of all its
-// PPT points' levels in registers and stores finished 64-byte rows at the end; nothing is staged in LDS, so
-// a launch of ceil(N / (256 * PPT)) workgroups fits the chip in one round up to about a million points.  Workgroups
+// Level sweep: the same work with (nearly) the whole grid resident at once.  A thread keeps the packed results of all
+// its PPT points' levels in registers and stores finished 64-byte rows at the end; nothing is staged in LDS, so three
+// or four workgroups fit a CU and a million points take little more than one round of workgroups.  Workgroups
 // that start together and do the same work per level stay together: at any moment an XCD's L2 serves the gathers of
-// one or two level tables, not of all of them (a workgroup that runs ahead fetches cold lines and falls back, one
+// a few level tables, not of all of them (a workgroup that runs ahead fetches cold lines and falls back, one
 // that lags finds them warm and catches up).  With workgroups that start at different times, as in the staged
-// kernel's several rounds, every level's table competes for L2 at once.
+// kernel's several rounds, every level's table competes for L2 at once.  (Perfect lock-step is not the aim: one
+// workgroup per CU, all in the same phase of the same level, lets the memory pipeline drain at every level.)
 template <typename TT, int PPT>
 __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_sweep_k(const void* coords, int cdt, int64_t csn, int64_t csd,
                                                                  const uint32_t* table, uint16_t* out, int64_t out_stride,
