@@ -105,6 +105,50 @@ def test_forward_backward(shape, d_in, d_hidden, d_out, depth, bias, act, dtype)
         _close(leaves[k].grad, want["d" + k], "d" + k, scale_rel=True, depth=depth)
 
 
+@pytest.mark.parametrize("act", ["relu", "silu", "none"])
+@pytest.mark.parametrize("shape,d_in,d_hidden,d_out,depth", [((3, 40), 1, 32, 5, 1), ((2, 2), 8, 16, 4, 3), ((1, 1000), 32, 64, 16, 2)])
+def test_float32_storage(shape, d_in, d_hidden, d_out, depth, act):
+    """float32 tensors: the reference multiplies them in TF32 (10-bit mantissa) and its tests allow 1e-3 forward,
+    1e-2 backward (tests/test_layers/test_fully_fused_mlp.py:42-46, 235-239); this build multiplies float16 roundings
+    of the same values with float32 accumulation and returns float32.  Checked against the float32 oracle on the
+    unrounded values at those tolerances (relative to each tensor's scale), and the results must be float32."""
+    mk = _mk()
+    torch.manual_seed(0)
+    p = _params(d_in, d_hidden, d_out, depth, True, torch.float32)
+    x = torch.randn(*shape, d_in)
+    dy = torch.randn(*shape, d_out)
+    if act == "relu":
+        # a unit within float16 rounding of zero switches its gate and moves dx by a whole weight: compare with the
+        # oracle evaluated at the same rounding points (float16 operands), as the 16-bit tests do
+        h = {k: (None if v is None else v.half()) for k, v in p.items()}
+        args = (h["w_in"], h["b_in"], h["w_out"], h["b_out"], h["w_hid"], h["b_hid"], act)
+        want_y = M.mlp_forward(x.half().float().view(-1, d_in), *args, round_to=torch.float16)
+        want = M.mlp_backward(x.half().view(-1, d_in), dy.half().view(-1, d_out), *args, round_to=torch.float16)
+    else:
+        args = (p["w_in"], p["b_in"], p["w_out"], p["b_out"], p["w_hid"], p["b_hid"], act)
+        want_y = M.mlp_forward(x.view(-1, d_in), *args)
+        want = M.mlp_backward(x.view(-1, d_in), dy.view(-1, d_out), *args)
+    leaves = {k: (None if v is None else v.to(DEV).requires_grad_(True)) for k, v in p.items()}
+    xd = x.to(DEV).requires_grad_(True)
+    y = mk.fully_fused_mlp(xd, leaves["w_in"], leaves["b_in"], leaves["w_out"], leaves["b_out"], leaves["w_hid"], leaves["b_hid"], act)
+    assert y.dtype == torch.float32 and y.shape == (*shape, d_out)
+
+    def close(got, ref, tol, what):
+        ref = ref.float()
+        scale = max(1.0, float(ref.abs().max()))
+        tol = max(tol, 1e-2) if act == "relu" else tol
+        torch.testing.assert_close(got.detach().cpu(), ref, rtol=tol, atol=tol * scale, msg=lambda m: f"{what}: {m}")
+
+    close(y.view(-1, d_out), want_y, 2e-3 * depth, "y")
+    y.backward(dy.to(DEV))
+    assert xd.grad.dtype == torch.float32
+    close(xd.grad.view(-1, d_in), want["dx"], 1e-2, "dx")
+    for k in ("w_in", "b_in", "w_out", "b_out", "w_hid", "b_hid"):
+        if leaves[k] is not None:
+            assert leaves[k].grad.dtype == torch.float32
+            close(leaves[k].grad, want["d" + k], 1e-2, "d" + k)
+
+
 def test_config2_sample_vs_oracle():
     """BASELINE configs[2] (32->64->64->16, ReLU, bf16, no bias) on 65536 rows against the oracle."""
     mk = _mk()
@@ -231,7 +275,9 @@ def test_argument_errors():
     with pytest.raises(ValueError):
         mk.fully_fused_mlp(x[0], p["w_in"], p["b_in"], p["w_out"], p["b_out"])  # x must be 3-D
     with pytest.raises(NotImplementedError):
-        mk.fully_fused_mlp(x.float(), *(p[k].float() for k in ("w_in", "b_in", "w_out", "b_out")))
+        mk.fully_fused_mlp(x.double(), *(p[k].double() for k in ("w_in", "b_in", "w_out", "b_out")))
+    with pytest.raises(AssertionError):
+        mk.fully_fused_mlp(x, *(p[k].float() for k in ("w_in", "b_in", "w_out", "b_out")))  # float32 parameters, 16-bit input
     w24 = torch.zeros(24, 8, device=DEV).half()
     with pytest.raises(AssertionError):
         mk.fully_fused_mlp(x, w24, None, torch.zeros(4, 24, device=DEV).half(), None)  # hidden not a power of 2

@@ -155,6 +155,30 @@ def test_full_size_config3_properties():
     _close(xg.grad[idx], want["dx"], "dx sample")
 
 
+def test_float32_storage():
+    """float32 tensors run with float16 operands and float32 accumulation; everything comes back as float32."""
+    rk = _rk()
+    torch.manual_seed(0)
+    w1, b1, w2, b2 = _params(3, 64, True, torch.float32)
+    x = torch.randn(500, 128)
+    dy = torch.randn(500, 128)
+    want_y = R.rev_forward(x, w1, b1, w2, b2, "gelu")
+    want = R.rev_backward(x, dy, w1, b1, w2, b2, "gelu")
+    leaves = [t.to(DEV).requires_grad_(True) for t in (w1, b1, w2, b2)]
+    xd = x.to(DEV).requires_grad_(True)
+    y = rk.reversible_mlp(xd, *leaves, "gelu")
+    assert y.dtype == torch.float32
+    _close(y, want_y, "y")
+    y.backward(dy.to(DEV))
+    assert xd.grad.dtype == torch.float32 and all(t.grad.dtype == torch.float32 for t in leaves)
+    _close(xd.grad, want["dx"], "dx")
+    for name, leaf in zip(("dw1", "db1", "dw2", "db2"), leaves):
+        _close(leaf.grad, want[name], name, scale_rel=True)
+    xr = rk.reversible_mlp_inverse(y.detach(), *(t.detach() for t in leaves))
+    assert xr.dtype == torch.float32
+    torch.testing.assert_close(xr.cpu(), x, rtol=2.0**-7, atol=2.0**-7)
+
+
 def test_module_and_errors():
     from triton_helpers_amd.layers.reversible_mlp import ReversibleMLP
 
@@ -174,4 +198,8 @@ def test_module_and_errors():
     with pytest.raises(AssertionError):
         rk.reversible_mlp(torch.zeros(4, 128, device=DEV).half(), w[:100], None, w[:100], None)
     with pytest.raises(NotImplementedError):
-        rk.reversible_mlp(torch.zeros(4, 128, device=DEV), w.float(), None, w.float(), None)
+        rk.reversible_mlp(torch.zeros(4, 128, device=DEV).double(), w.double(), None, w.double(), None)
+    # a float32 module without autocast runs too (float16 operands inside) and returns float32
+    y32 = layer(x.detach())
+    assert y32.dtype == torch.float32
+    torch.testing.assert_close(y32, y.detach().float(), rtol=2e-2, atol=1e-2)

@@ -11,8 +11,11 @@ Supersets / differences:
   * weight gradients are accumulated in float32 inside the kernel and rounded once
     (the reference sums per-program partials in the storage dtype, kernel.py:599-633);
   * ``fp16_acc`` is accepted and ignored: accumulation is always float32 (MFMA);
-  * storage dtypes are float16 and bfloat16 (what autocast produces); float32 tensors
-    raise ``NotImplementedError`` -- cast them, or run the module under autocast.
+  * storage dtypes of the kernels are float16 and bfloat16 (what autocast produces).  float32 tensors
+    (the reference feeds them to ``tl.dot``, which multiplies in TF32: 10-bit mantissa, float32
+    accumulation) are run with float16 operands -- the same 10-bit mantissa, float32 accumulation;
+    operands beyond +-65504 overflow, which TF32's 8-bit exponent would not -- and the output, ``dx`` and
+    the weight gradients (straight from the float32 accumulators) come back as float32.
 """
 from __future__ import annotations
 
@@ -82,13 +85,17 @@ def feedforward_bwd_dx(w: Tensor, dz: Tensor, DTYPE: torch.dtype = torch.float32
 
 # ---------------------------------------------------------------------------
 def _check_storage(x: Tensor, w_in: Tensor, *others: Optional[Tensor]) -> None:
-    """Parameters share one 16-bit dtype; ``x`` may be in the other 16-bit dtype (an fp16 encoder output in front of
-    bf16 weights): the kernels convert it while loading, exactly as a cast in front would."""
-    for t in (x, w_in):
-        if t.dtype not in (torch.float16, torch.bfloat16):
-            raise NotImplementedError(
-                f"fully_fused_mlp runs on float16 / bfloat16 storage, got {t.dtype}; cast the tensors or use autocast"
-            )
+    """Parameters share one dtype.  With 16-bit parameters ``x`` may be in the other 16-bit dtype (an fp16 encoder
+    output in front of bf16 weights): the kernels convert it while loading, exactly as a cast in front would.
+    float32 runs as a whole (``x`` and parameters) with float16 operands."""
+    if w_in.dtype == torch.float32:
+        assert x.dtype == torch.float32, f"float32 parameters take a float32 input, got {x.dtype}"
+    else:
+        for t in (x, w_in):
+            if t.dtype not in (torch.float16, torch.bfloat16):
+                raise NotImplementedError(
+                    f"fully_fused_mlp runs on float16 / bfloat16 / float32 storage, got {t.dtype}; cast the tensors or use autocast"
+                )
     for t in others:
         assert t is None or t.dtype == w_in.dtype, f"All parameters must share one dtype, got {w_in.dtype} and {t.dtype}"
     for t in (w_in, *others):
@@ -101,6 +108,10 @@ def _rows2d(t: Tensor, width: int) -> Tensor:
     if t2.stride(1) != 1:
         t2 = t2.contiguous()
     return t2
+
+
+def _half(t: Optional[Tensor]) -> Optional[Tensor]:
+    return None if t is None else t.to(torch.float16)
 
 
 def _c(t: Optional[Tensor]) -> Optional[Tensor]:
@@ -147,6 +158,13 @@ class _fully_fused_mlp(Function):
         assert activation in _ACTIVATIONS, f"Invalid activation function: {activation}"
         _check_storage(x, w_in, b_in, w_out, b_out, w_hid, b_hid)
 
+        ctx.save_for_backward(x, w_in, b_in, w_out, b_out, w_hid, b_hid)
+        ctx.activation = activation
+        ctx.fp16_acc = fp16_acc
+        ctx.depth = depth
+        wide = w_in.dtype == torch.float32
+        if wide:  # float16 operands, float32 accumulation and results
+            x, w_in, b_in, w_out, b_out, w_hid, b_hid = (_half(t) for t in (x, w_in, b_in, w_out, b_out, w_hid, b_hid))
         w_in, b_in, w_out, b_out, w_hid, b_hid = (_c(t) for t in (w_in, b_in, w_out, b_out, w_hid, b_hid))
         x2 = _rows2d(x, D_in)
         o = x.new_empty((B, L, D_out), dtype=w_in.dtype)
@@ -159,12 +177,7 @@ class _fully_fused_mlp(Function):
             _lib.dtype_code(x.dtype), _lib.current_stream(x.device),
         )
         _lib.check(rc, "nf_mlp_fwd")
-
-        ctx.save_for_backward(x, w_in, b_in, w_out, b_out, w_hid, b_hid)
-        ctx.activation = activation
-        ctx.fp16_acc = fp16_acc
-        ctx.depth = depth
-        return o
+        return o.float() if wide else o
 
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
@@ -174,6 +187,9 @@ class _fully_fused_mlp(Function):
         B, L, D_in = x.shape
         D_hidden = w_in.shape[0]
         D_out = w_out.shape[0]
+        wide = w_in.dtype == torch.float32
+        if wide:
+            x, w_in, b_in, w_out, b_out, w_hid, b_hid = (_half(t) for t in (x, w_in, b_in, w_out, b_out, w_hid, b_hid))
         if do.dtype != w_in.dtype:
             do = do.to(w_in.dtype)
         if x.dtype != w_in.dtype and not (ctx.depth == 2 and D_hidden > 32 and ctx.activation == "relu"):
@@ -200,7 +216,9 @@ class _fully_fused_mlp(Function):
             break
         _lib.check(rc, "nf_mlp_bwd")
         # float32 accumulators, rounded once to the parameters' dtype (one kernel for all of them)
-        dw_in, db_in, dw_out, db_out, dw_hid, db_hid = grads.rounded(w_in.dtype)
+        dw_in, db_in, dw_out, db_out, dw_hid, db_hid = grads.rounded(torch.float32 if wide else w_in.dtype)
+        if wide and dx is not None:
+            dx = dx.float()
         return dx, dw_in, db_in, dw_out, db_out, dw_hid, db_hid, None, None
 
 

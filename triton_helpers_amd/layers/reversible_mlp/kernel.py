@@ -39,8 +39,8 @@ def _validate(x: Tensor, w1: Tensor, b1: Optional[Tensor], w2: Tensor, b2: Optio
     for b in (b1, b2):
         assert b is None or b.shape == (2 * blocks, H), "biases must be (blocks*2, H)"
     assert activation in _ACTIVATIONS, f"Invalid activation function: {activation}"
-    if x.dtype not in (torch.float16, torch.bfloat16):
-        raise NotImplementedError(f"reversible_mlp runs on float16 / bfloat16 storage, got {x.dtype}")
+    if x.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        raise NotImplementedError(f"reversible_mlp runs on float16 / bfloat16 / float32 storage, got {x.dtype}")
     for t in (w1, b1, w2, b2):
         assert t is None or (t.dtype == x.dtype and t.device == x.device), "All tensors must share dtype and device"
     assert x.device.type == "cuda", "All tensors must be on a GPU device"
@@ -57,6 +57,10 @@ class _reversible_mlp(Function):
     @torch.no_grad()
     def forward(ctx, x: Tensor, w1: Tensor, b1: Optional[Tensor], w2: Tensor, b2: Optional[Tensor], activation: str = "gelu") -> Tensor:
         H, blocks = _validate(x, w1, b1, w2, b2, activation)
+        # float32 tensors run with float16 operands (float32 accumulation) and come back as float32, like the fused MLP
+        wide = x.dtype == torch.float32
+        if wide:
+            x, w1, b1, w2, b2 = (None if t is None else t.to(torch.float16) for t in (x, w1, b1, w2, b2))
         w1, b1, w2, b2 = (_c(t) for t in (w1, b1, w2, b2))
         x2 = _rows2d(x, 2 * H)
         y = x.new_empty(x.shape)
@@ -71,7 +75,8 @@ class _reversible_mlp(Function):
         ctx.activation = activation
         ctx.half = H
         ctx.blocks = blocks
-        return y
+        ctx.wide = wide
+        return y.float() if wide else y
 
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
@@ -96,8 +101,8 @@ class _reversible_mlp(Function):
             y2.shape[0], H, ctx.blocks, _lib.NF_ACT[ctx.activation], _lib.dtype_code(y.dtype), _lib.current_stream(y.device),
         )
         _lib.check(rc, "nf_revmlp_bwd")
-        dw1, db1, dw2, db2 = grads.rounded(w1.dtype)
-        return dx, dw1, db1, dw2, db2, None
+        dw1, db1, dw2, db2 = grads.rounded(torch.float32 if ctx.wide else w1.dtype)
+        return (dx.float() if ctx.wide else dx), dw1, db1, dw2, db2, None
 
 
 def reversible_mlp(x: Tensor, w1: Tensor, b1: Optional[Tensor], w2: Tensor, b2: Optional[Tensor], activation: str = "gelu") -> Tensor:
@@ -115,6 +120,9 @@ def reversible_mlp(x: Tensor, w1: Tensor, b1: Optional[Tensor], w2: Tensor, b2: 
 def reversible_mlp_inverse(y: Tensor, w1: Tensor, b1: Optional[Tensor], w2: Tensor, b2: Optional[Tensor], activation: str = "gelu") -> Tensor:
     """Input reconstructed from the output by the backward kernel's in-kernel inverse."""
     H, blocks = _validate(y, w1, b1, w2, b2, activation)
+    wide = y.dtype == torch.float32
+    if wide:
+        y, w1, b1, w2, b2 = (None if t is None else t.to(torch.float16) for t in (y, w1, b1, w2, b2))
     w1, b1, w2, b2 = (_c(t) for t in (w1, b1, w2, b2))
     y2 = _rows2d(y, 2 * H)
     zeros = torch.zeros_like(y2)
@@ -129,4 +137,4 @@ def reversible_mlp_inverse(y: Tensor, w1: Tensor, b1: Optional[Tensor], w2: Tens
         y2.shape[0], H, blocks, _lib.NF_ACT[activation], _lib.dtype_code(y.dtype), _lib.current_stream(y.device),
     )
     _lib.check(rc, "nf_revmlp_bwd")
-    return x_rec
+    return x_rec.float() if wide else x_rec
