@@ -516,7 +516,7 @@ extern "C" int nf_hash_encode_bwd(const void* coords, int coords_dtype, int64_t 
 
   // large batches: accumulate in LDS tiles (needs the caller's workspace for the sorted records or the bit-planes)
   if (!(flags & (NF_HASH_FORCE_GENERIC | NF_HASH_FORCE_ATOMIC)) && n_points >= SCAN_MIN_POINTS && workspace != nullptr &&
-      ((uintptr_t)dout % 4 == 0) && (dout_stride_n % 2 == 0) && ((uintptr_t)workspace % 4 == 0)) {
+      ((uintptr_t)dout % (dout_dtype == NF_F32 ? 8 : 4) == 0) && (dout_stride_n % 2 == 0) && ((uintptr_t)workspace % 4 == 0)) {
     const int64_t need_bin = bwd_bin_workspace_bytes(n_points, geom, dout_dtype);
     if (!(flags & NF_HASH_FORCE_PLANES) && need_bin > 0 && workspace_bytes >= need_bin && ((uintptr_t)workspace % 16 == 0))
       return launch_bwd_bin(coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, geom, g, primes,

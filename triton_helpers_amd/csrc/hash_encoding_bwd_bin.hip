@@ -63,7 +63,7 @@ struct BinWs {
   uint32_t* n_tasks;
   uint4* tasks;
   uint32_t* wg_counts;
-  uint3* records;
+  uint32_t* records;  // 3 words per record (16-bit gradient) or 4 (float32 gradient)
   uint32_t max_tasks;
 };
 
@@ -245,15 +245,23 @@ __global__ __launch_bounds__(1024) void hash_bwd_bin_offsets_k(const uint32_t* h
 // ---------------------------------------------------------------------------------------
 // fill
 // ---------------------------------------------------------------------------------------
+// G32 = false: 16-bit upstream gradient, 12-byte records {.., .., packed pair}.  G32 = true: float32 upstream gradient,
+// 16-byte records {.., .., g0, g1}; a staged entry then names the point instead of carrying the pair, and the copy-out
+// takes the pair from the workgroup's per-level gradient table in LDS (the stage has no room for 20-byte entries).
+template <bool G32>
 __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* coords, int cdt, int64_t csn, int64_t csd,
-                                                                   const uint16_t* dout, int64_t dout_stride, int64_t N,
+                                                                   const void* dout_v, int64_t dout_stride, int64_t N,
                                                                    DevGeom g, BinPlan bp, const int64_t* primes, float scale,
                                                                    const uint32_t* wg_counts, uint32_t* cursor, uint32_t* gmax,
-                                                                   uint3* records) {
+                                                                   uint32_t* records_v) {
   extern __shared__ __align__(16) unsigned char fill_smem[];
   const int NB = bp.binbase[bp.n_levels];
+  const uint16_t* dout = reinterpret_cast<const uint16_t*>(dout_v);
+  uint3* records = reinterpret_cast<uint3*>(records_v);
+  uint4* records4 = reinterpret_cast<uint4*>(records_v);
   uint4* stage = reinterpret_cast<uint4*>(fill_smem);                     // [FILL_RECORDS] {record, its place in `records`}, sorted by bin
-  uint32_t* cur = reinterpret_cast<uint32_t*>(stage + FILL_RECORDS);      // [NB] next staged position of a bin
+  uint2* gtab = reinterpret_cast<uint2*>(stage + FILL_RECORDS);           // G32: [FILL_POINTS] this level's gradient pair of every point
+  uint32_t* cur = reinterpret_cast<uint32_t*>(gtab + (G32 ? FILL_POINTS : 0));  // [NB] next staged position of a bin
   uint32_t* delta = cur + NB;                                             // [NB] global minus staged position
   uint32_t* totals = delta + NB;                                          // [levels] records of this workgroup per level
   uint32_t* lmax = totals + NF_MAX_LEVELS;                                // [levels] largest |dout| pattern
@@ -272,10 +280,11 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
   float v[3] = {0.0f, 0.0f, 0.0f};
   if (valid) load_point(coords, cdt, csn, csd, n, scale, v);
   const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], (uint32_t)primes[2]};
-  // this point's gradient row, read once (up to 16 levels live in registers)
+  // this point's gradient row, read once (up to 16 levels live in registers); float32 rows are read level by level
   const uint32_t* grow = reinterpret_cast<const uint32_t*>(dout + (valid ? n : 0) * dout_stride);
+  const uint2* grow32 = reinterpret_cast<const uint2*>(reinterpret_cast<const float*>(dout_v) + (valid ? n : 0) * dout_stride);
   uint32_t gr[16];
-  const bool row_vec = bp.n_levels <= 16 && (bp.n_levels & 3) == 0 && ((uintptr_t)dout & 15u) == 0 && (dout_stride & 7) == 0;
+  const bool row_vec = !G32 && bp.n_levels <= 16 && (bp.n_levels & 3) == 0 && ((uintptr_t)dout & 15u) == 0 && (dout_stride & 7) == 0;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     uint4 t = make_uint4(0u, 0u, 0u, 0u);
@@ -314,15 +323,23 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
     const int nb = bp.nbins[l];
     uint32_t* lcur = cur + bp.binbase[l];
     const uint32_t* ldelta = delta + bp.binbase[l];
-    uint32_t packed = 0u;
-    if (row_vec) {
-      packed = gr[0];
+    uint32_t packed = 0u;  // 16-bit: the pair; float32: the point's index in the workgroup (its pair goes to gtab)
+    if (G32) {
+      const uint2 pair = valid ? grow32[l] : make_uint2(0u, 0u);
+      gtab[tid] = pair;
+      packed = (uint32_t)tid;
+      // largest |g| of the level: positive float patterns order like integers
+      const uint32_t a0 = pair.x & 0x7fffffffu, a1 = pair.y & 0x7fffffffu;
+      const uint32_t m = wave_max_u32(a0 > a1 ? a0 : a1);
+      if (lane == 63 && m) atomicMax(lmax + l, m);
+    } else {
+      if (row_vec) {
+        packed = gr[0];
 #pragma unroll
-      for (int i = 1; i < 16; ++i) packed = (l == i) ? gr[i] : packed;
-    } else if (valid) {
-      packed = grow[l];
-    }
-    {
+        for (int i = 1; i < 16; ++i) packed = (l == i) ? gr[i] : packed;
+      } else if (valid) {
+        packed = grow[l];
+      }
       // largest |g| of the level: positive 16-bit float patterns order like integers
       const uint32_t pk = packed & 0x7fff7fffu;
       const uint32_t m = wave_max_u32((pk & 0xffffu) > (pk >> 16) ? (pk & 0xffffu) : (pk >> 16));
@@ -362,7 +379,7 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
         for (int c = 0; c < 4; ++c) {
           const uint32_t r0 = r.row[2 * c], r1 = r.row[2 * c + 1];
           const uint3 rec = make_record(r0 & BIN_MASK, (split[c] ? r0 : r1) & BIN_MASK, w[2 * c], split[c] ? 0.0f : w[2 * c + 1], packed);
-          stage[pos[c]] = make_uint4(rec.x, rec.y, rec.z, pos[c] + dlt[c]);
+          stage[pos[c]] = G32 ? make_uint4(rec.x, rec.y, pos[c] + dlt[c], rec.z) : make_uint4(rec.x, rec.y, rec.z, pos[c] + dlt[c]);
         }
       }
       // a pair that straddles two bins leaves its second corner as a record of its own (rare)
@@ -377,7 +394,8 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
           if (on) {
             const uint32_t r1 = r.row[2 * c + 1];
             const uint3 rec = make_record(r1 & BIN_MASK, r1 & BIN_MASK, w[2 * c + 1], 0.0f, packed);
-            stage[pos1] = make_uint4(rec.x, rec.y, rec.z, pos1 + ldelta[b1[c]]);
+            const uint32_t gp = pos1 + ldelta[b1[c]];
+            stage[pos1] = G32 ? make_uint4(rec.x, rec.y, gp, rec.z) : make_uint4(rec.x, rec.y, rec.z, gp);
           }
         }
       }
@@ -386,7 +404,12 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
     const uint32_t total = totals[l];
     for (uint32_t i = tid; i < total; i += FILL_POINTS) {
       const uint4 e = stage[i];
-      records[e.w] = make_uint3(e.x, e.y, e.z);
+      if (G32) {
+        const uint2 pair = gtab[e.w];
+        records4[e.z] = make_uint4(e.x, e.y, pair.x, pair.y);
+      } else {
+        records[e.w] = make_uint3(e.x, e.y, e.z);
+      }
     }
     lds_barrier();  // the next level overwrites the stage
   }
@@ -399,10 +422,29 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
 // ---------------------------------------------------------------------------------------
 // accumulate
 // ---------------------------------------------------------------------------------------
+// record type and gradient decode per upstream-gradient dtype
 template <typename GT>
-__global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const uint3* records, const uint4* tasks,
+struct BinRec {
+  typedef uint3 type;
+  __device__ static __forceinline__ type zero() { return make_uint3(0u, 0u, 0u); }
+  __device__ static __forceinline__ float g0(const type& q) { return GT::to_f32((uint16_t)(q.z & 0xffffu)); }
+  __device__ static __forceinline__ float g1(const type& q) { return GT::to_f32((uint16_t)(q.z >> 16)); }
+  __device__ static __forceinline__ float level_max(uint32_t pattern) { return GT::to_f32((uint16_t)pattern); }
+};
+template <>
+struct BinRec<F32> {
+  typedef uint4 type;
+  __device__ static __forceinline__ type zero() { return make_uint4(0u, 0u, 0u, 0u); }
+  __device__ static __forceinline__ float g0(const type& q) { return __uint_as_float(q.z); }
+  __device__ static __forceinline__ float g1(const type& q) { return __uint_as_float(q.w); }
+  __device__ static __forceinline__ float level_max(uint32_t pattern) { return __uint_as_float(pattern); }
+};
+
+template <typename GT>
+__global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const typename BinRec<GT>::type* records, const uint4* tasks,
                                                                     const uint32_t* n_tasks, const uint32_t* gmax, float* dtable,
                                                                     DevGeom g, BinPlan bp) {
+  typedef typename BinRec<GT>::type Rec;
   // Fixed-point sums, one plane of BIN_ROWS 64-bit cells per feature: the 64 lanes of an add go to random rows of one
   // feature, and with 8-byte cells those spread over all 64 banks (interleaved features would leave them half).
   extern __shared__ unsigned long long acc_tile[];
@@ -415,7 +457,7 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const uint3*
   const uint32_t left = g.rows[l] - row0;
   const uint32_t nrows = left < (uint32_t)BIN_ROWS ? left : (uint32_t)BIN_ROWS;
   // fixed-point scale 2^se of the level:  |w * g| * 2^se < 2^30
-  const float gm = GT::to_f32((uint16_t)gmax[l]);
+  const float gm = BinRec<GT>::level_max(gmax[l]);
   const bool nonfinite = !(gm <= 3.0e38f);
   int se = 0;
   if (!nonfinite && gm > 0.0f) {
@@ -429,18 +471,18 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const uint3*
   for (uint32_t i = tid; i < 2u * nrows; i += ACC_THREADS) acc_tile[(i & 1u) * BIN_ROWS + (i >> 1)] = 0ull;
   lds_barrier();
   // the next round's records are loaded before this round's adds
-  uint3 q[ACC_INFLIGHT];
+  Rec q[ACC_INFLIGHT];
 #pragma unroll
   for (int k = 0; k < ACC_INFLIGHT; ++k) {
     const uint32_t i = task.y + k * ACC_THREADS + tid;
-    q[k] = i < task.z ? records[i] : make_uint3(0u, 0u, 0u);
+    q[k] = i < task.z ? records[i] : BinRec<GT>::zero();
   }
   for (uint32_t i0 = task.y; i0 < task.z; i0 += ACC_THREADS * ACC_INFLIGHT) {
     uint32_t slot[ACC_INFLIGHT][2];
     int32_t f[ACC_INFLIGHT][4];
 #pragma unroll
     for (int k = 0; k < ACC_INFLIGHT; ++k) {
-      const float g0 = GT::to_f32((uint16_t)(q[k].z & 0xffffu)) * s_lo, g1 = GT::to_f32((uint16_t)(q[k].z >> 16)) * s_lo;
+      const float g0 = BinRec<GT>::g0(q[k]) * s_lo, g1 = BinRec<GT>::g1(q[k]) * s_lo;
       // records past the end: zero weights
       const float w0 = (float)(q[k].y & W_MAX), w1 = (float)((q[k].x >> 26) << 13 | q[k].y >> W_BITS);
       slot[k][0] = q[k].x & BIN_MASK;
@@ -457,7 +499,7 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const uint3*
 #pragma unroll
     for (int k = 0; k < ACC_INFLIGHT; ++k) {
       const uint32_t i = i0 + ACC_THREADS * ACC_INFLIGHT + k * ACC_THREADS + tid;
-      q[k] = i < task.z ? records[i] : make_uint3(0u, 0u, 0u);
+      q[k] = i < task.z ? records[i] : BinRec<GT>::zero();
     }
 #pragma unroll
     for (int k = 0; k < ACC_INFLIGHT; ++k)
@@ -496,7 +538,7 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const uint3*
 // Host side
 // ---------------------------------------------------------------------------------------
 static bool bin_plan(int64_t N, const nf_hash_geom* geom, int dout_dtype, BinPlan* bp, int64_t* records, uint32_t* max_tasks) {
-  if (geom->dims != 3 || geom->feat != 2 || dout_dtype == NF_F32 || N <= 0) return false;
+  if (geom->dims != 3 || geom->feat != 2 || N <= 0) return false;
   bp->n_levels = geom->levels;
   int nb_total = 0;
   for (int l = 0; l < geom->levels; ++l) {
@@ -520,7 +562,7 @@ static bool bin_plan(int64_t N, const nf_hash_geom* geom, int dout_dtype, BinPla
 
 static int64_t wg_count_words(int64_t N, int NB) { return (((N + FILL_POINTS - 1) / FILL_POINTS) * NB + 3) & ~(int64_t)3; }
 
-static int64_t bin_ws(void* workspace, const BinPlan& bp, int64_t N, int64_t R, uint32_t max_tasks, BinWs* ws) {
+static int64_t bin_ws(void* workspace, const BinPlan& bp, int64_t N, int64_t R, int rec_words, uint32_t max_tasks, BinWs* ws) {
   uint32_t* p = (uint32_t*)workspace;
   const int NB = bp.binbase[bp.n_levels];
   const int NBp = (NB + 3) & ~3;
@@ -531,7 +573,8 @@ static int64_t bin_ws(void* workspace, const BinPlan& bp, int64_t N, int64_t R, 
   ws->n_tasks = p + o; o += 4;
   ws->tasks = reinterpret_cast<uint4*>(p + o); o += 4 * (int64_t)max_tasks;
   ws->wg_counts = p + o; o += wg_count_words(N, NB);
-  ws->records = reinterpret_cast<uint3*>(p + o); o += 3 * R;
+  o = (o + 3) & ~(int64_t)3;  // 16-byte records start on a 16-byte boundary
+  ws->records = p + o; o += (int64_t)rec_words * R;
   ws->max_tasks = max_tasks;
   return o * 4;
 }
@@ -542,7 +585,7 @@ int64_t bwd_bin_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int 
   uint32_t max_tasks;
   if (!bin_plan(n_points, geom, dout_dtype, &bp, &R, &max_tasks)) return 0;
   BinWs ws;
-  return bin_ws(nullptr, bp, n_points, R, max_tasks, &ws);
+  return bin_ws(nullptr, bp, n_points, R, dout_dtype == NF_F32 ? 4 : 3, max_tasks, &ws);
 }
 
 int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const void* dout, int ddt, int64_t dout_stride,
@@ -553,8 +596,9 @@ int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const 
   uint32_t max_tasks;
   NF_REQUIRE(bin_plan(N, geom, ddt, &bp, &R, &max_tasks), NF_EUNSUPPORTED, "binned backward does not cover this geometry");
   NF_REQUIRE(((uintptr_t)workspace & 15u) == 0, NF_EALIGN, "workspace must be 16-byte aligned");
+  const bool g32 = ddt == NF_F32;
   BinWs ws;
-  bin_ws(workspace, bp, N, R, max_tasks, &ws);
+  bin_ws(workspace, bp, N, R, g32 ? 4 : 3, max_tasks, &ws);
   const int NB = bp.binbase[bp.n_levels];
   const int NBp = (NB + 3) & ~3;
   const unsigned blocks = (unsigned)((N + FILL_POINTS - 1) / FILL_POINTS);
@@ -568,20 +612,26 @@ int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const 
                      ws.tasks, NB, max_tasks);
   if (int rc = check_launch("hash_bwd_bin_offsets")) return rc;
   {
-    const size_t lds = (size_t)FILL_RECORDS * sizeof(uint4) + ((size_t)2 * NB + 2 * NF_MAX_LEVELS) * 4;
-    hipError_t e = hipFuncSetAttribute((const void*)hash_bwd_bin_fill_k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    const size_t lds = (size_t)FILL_RECORDS * sizeof(uint4) + (g32 ? (size_t)FILL_POINTS * sizeof(uint2) : 0) +
+                       ((size_t)2 * NB + 2 * NF_MAX_LEVELS) * 4;
+    const void* kern = g32 ? (const void*)hash_bwd_bin_fill_k<true> : (const void*)hash_bwd_bin_fill_k<false>;
+    hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    hipLaunchKernelGGL(hash_bwd_bin_fill_k, dim3(blocks), dim3(FILL_POINTS), lds, s, coords, cdt, csn, csd,
-                       (const uint16_t*)dout, dout_stride, N, g, bp, primes, scale, (const uint32_t*)ws.wg_counts, ws.cursor,
-                       ws.gmax, ws.records);
+    const uint32_t* wc = ws.wg_counts;
+    void* args[] = {(void*)&coords, (void*)&cdt,   (void*)&csn,    (void*)&csd,   (void*)&dout, (void*)&dout_stride, (void*)&N, (void*)&g,
+                    (void*)&bp,     (void*)&primes, (void*)&scale, (void*)&wc,    (void*)&ws.cursor, (void*)&ws.gmax, (void*)&ws.records};
+    e = hipLaunchKernel(kern, dim3(blocks), dim3(FILL_POINTS), args, lds, s);
+    if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(hash_bwd_bin_fill): %s", hipGetErrorString(e));
     if (int rc = check_launch("hash_bwd_bin_fill")) return rc;
   }
   {
     const size_t lds = (size_t)BIN_ROWS * 2 * sizeof(unsigned long long);
-    const void* kern = ddt == NF_F16 ? (const void*)hash_bwd_bin_accum_k<F16> : (const void*)hash_bwd_bin_accum_k<BF16>;
+    const void* kern = ddt == NF_F16    ? (const void*)hash_bwd_bin_accum_k<F16>
+                       : ddt == NF_BF16 ? (const void*)hash_bwd_bin_accum_k<BF16>
+                                        : (const void*)hash_bwd_bin_accum_k<F32>;
     hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    const uint3* rc_ = ws.records;
+    const uint32_t* rc_ = ws.records;
     const uint4* tk = ws.tasks;
     const uint32_t* nt = ws.n_tasks;
     const uint32_t* gm = ws.gmax;
