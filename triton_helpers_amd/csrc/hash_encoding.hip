@@ -317,6 +317,82 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_sweep_k(const void* coo
   }
 }
 
+// The level sweep for float32 tables (a row is one 8-byte pair, an output row 32 floats): same walk, same operation
+// order as the per-(point, level) kernel, the results of a thread's PPT points held as float pairs.
+template <int PPT>
+__global__ __launch_bounds__(TILE_THREADS) void hash_fwd_sweep32_k(const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                                   const float2* table, float* out, int64_t out_stride,
+                                                                   int64_t N, DevGeom g, const int64_t* primes, float scale) {
+  constexpr int P = TILE_THREADS * PPT;
+  constexpr int LMAX = 16;
+  const int t = threadIdx.x;
+  const int64_t p0 = (int64_t)blockIdx.x * P;
+  const int L = g.levels;
+  float x[PPT][3];
+#pragma unroll
+  for (int i = 0; i < PPT; ++i) {
+    int64_t n = p0 + t + TILE_THREADS * i;
+    if (n >= N) n = N - 1;
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+      float v = load_as_f32(coords, n * csn + d * csd, cdt);
+      x[i][d] = scale != 1.0f ? v / scale : v;
+    }
+  }
+  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], (uint32_t)primes[2]};
+  float2 enc[PPT][LMAX];
+#pragma unroll
+  for (int l = 0; l < LMAX; ++l) {
+    if (l < L) {
+      const uint32_t res = (uint32_t)g.res[l];
+      const float fres = (float)g.res[l];
+      const bool hashed = l >= g.first_hash;
+      const uint32_t mask = g.rows[l] - 1;
+      const float2* tab = table + g.row_offset[l];
+      float2 v[PPT][8];
+      float w[PPT][8];
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) {
+        uint32_t c[3];
+        float fr[3];
+#pragma unroll
+        for (int d = 0; d < 3; ++d) {
+          const float pos = x[i][d] * fres;
+          const float fl = floorf(pos);
+          c[d] = (uint32_t)(int)fl;
+          fr[d] = pos - fl;
+        }
+        const Corner8 r = rows_d3(c, hashed, res, mask, pi);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[i][j] = tab[r.row[j]];
+        weights_d3(fr, w[i]);
+      }
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) {
+        float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          a0 = a0 + w[i][j] * v[i][j].x;
+          a1 = a1 + w[i][j] * v[i][j].y;
+        }
+        enc[i][l] = make_float2(a0, a1);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) enc[i][l] = make_float2(0.0f, 0.0f);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < PPT; ++i) {
+    const int64_t n = p0 + t + TILE_THREADS * i;
+    if (n >= N) continue;
+    float4* dst = reinterpret_cast<float4*>(out + n * out_stride);
+#pragma unroll
+    for (int q = 0; q < LMAX / 2; ++q)
+      if (2 * q < L) dst[q] = make_float4(enc[i][2 * q].x, enc[i][2 * q].y, enc[i][2 * q + 1].x, enc[i][2 * q + 1].y);
+  }
+}
+
 template <typename GT, int PPT>
 __global__ __launch_bounds__(TILE_THREADS) void hash_bwd_tiled_k(const void* coords, int cdt, int64_t csn, int64_t csd,
                                                                  const uint16_t* dout, int64_t dout_stride,
@@ -413,6 +489,16 @@ static bool tiled_ok(const nf_hash_geom* g, int table_dt, const void* rows_ptr, 
   return true;
 }
 
+static bool sweep32_ok(const nf_hash_geom* g, const void* table, const void* rows_ptr, int64_t row_stride) {
+  if (g->dims != 3 || g->feat != 2 || g->levels % 2 != 0 || g->levels > 16) return false;
+  for (int l = g->first_hash_level; l < g->levels; ++l) {
+    if (l < 0) return false;
+    const int64_t r = g->rows[l];
+    if ((r & (r - 1)) != 0) return false;
+  }
+  return ((uintptr_t)table & 7u) == 0 && ((uintptr_t)rows_ptr & 15u) == 0 && row_stride % 4 == 0;
+}
+
 template <int D, typename TT>
 static void launch_fwd_generic(const void* coords, int cdt, int64_t csn, int64_t csd, const void* table, void* out,
                                int64_t out_stride, int64_t N, const DevGeom& g, const int64_t* primes, float scale,
@@ -454,6 +540,16 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
   NF_REQUIRE(n_points <= ((int64_t)1 << 31) * 256 - 1, NF_EINVAL, "n_points too large");
   hipStream_t s = (hipStream_t)stream;
 
+  // float32 tables: the same sweep on 8-byte rows
+  if (!(flags & (NF_HASH_FORCE_GENERIC | NF_HASH_FWD_STAGED)) && n_points >= SWEEP_MIN_POINTS && table_dtype == NF_F32 &&
+      sweep32_ok(geom, table, out, out_stride_n)) {
+    constexpr int PPT = 2;
+    constexpr int P = TILE_THREADS * PPT;
+    dim3 grid((unsigned)((n_points + P - 1) / P));
+    hipLaunchKernelGGL((hash_fwd_sweep32_k<PPT>), grid, dim3(TILE_THREADS), 0, s, coords, coords_dtype, csn, csd,
+                       (const float2*)table, (float*)out, out_stride_n, n_points, g, primes, scale);
+    return check_launch("hash_fwd_sweep32");
+  }
   // The level sweep wants at least one workgroup per compute unit; below that the staged kernel's smaller tiles
   // spread the points over more of the chip.
   if (!(flags & (NF_HASH_FORCE_GENERIC | NF_HASH_FWD_STAGED)) && n_points >= SWEEP_MIN_POINTS &&
