@@ -114,7 +114,7 @@ __device__ __forceinline__ float normal_cdf_pdf(float z, float* pdf) {
 __device__ __forceinline__ float act_fwd(float z, int act) {
   switch (act) {
     case NF_ACT_RELU: return z < 0.0f ? 0.0f : z;
-    case NF_ACT_SILU: return z / (1.0f + __expf(-z));
+    case NF_ACT_SILU: return z * __builtin_amdgcn_rcpf(1.0f + __expf(-z));  // v_rcp_f32 (1 ulp) instead of a full division
     case NF_ACT_RELU2: return fmaxf(z, 0.0f) * z;
     case NF_ACT_GELU: return z * normal_cdf(z);
     default: return z;
@@ -125,7 +125,7 @@ __device__ __forceinline__ float act_grad(float z, int act) {
   switch (act) {
     case NF_ACT_RELU: return z > 0.0f ? 1.0f : 0.0f;
     case NF_ACT_SILU: {
-      const float s = 1.0f / (1.0f + __expf(-z));
+      const float s = __builtin_amdgcn_rcpf(1.0f + __expf(-z));
       return s * (z * (1.0f - s) + 1.0f);
     }
     case NF_ACT_RELU2: return z > 0.0f ? 2.0f * z : 0.0f;
