@@ -415,6 +415,300 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// The same kernel for deeper ReLU nets: NH hidden-to-hidden layers (depth = NH + 1), 32-row chunks.  Every
+// hidden activation of the chunk stays in registers (they are the gates as well), every weight gradient in float32
+// accumulators over the wave's row loop; the weights of all layers, in both forms, are resident in LDS.
+// ---------------------------------------------------------------------------------------
+template <typename T, int KIN, int HP, int OUTP, int NH, bool FAST>
+__global__ __launch_bounds__(256) void mlp_bwdn_k(MlpArgs a) {
+  constexpr int KC_IN = KIN / 32, KC_H = HP / 32, MT_H = HP / 16, MT_I = KIN / 16, MT_O = OUTP / 16;
+  constexpr int KC_O = (OUTP + 31) / 32;
+  constexpr int NT = 2;
+  constexpr int HID = MT_H * KC_H * FRAG_ELEMS;  // one hidden layer's fragments
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int lane = tid & 63, wave = tid >> 6;
+
+  uint16_t* f_in = reinterpret_cast<uint16_t*>(smem);          // W_in      [MT_H][KC_IN]
+  uint16_t* f_hid = f_in + MT_H * KC_IN * FRAG_ELEMS;          // W_hid[k]  [NH][MT_H][KC_H]
+  uint16_t* t_in = f_hid + NH * HID;                           // W_in^T    [MT_I][KC_H]
+  uint16_t* t_hid = t_in + MT_I * KC_H * FRAG_ELEMS;           // W_hid[k]^T
+  uint16_t* t_out = t_hid + NH * HID;                          // W_out^T   [MT_H][KC_O]
+  float* bias_in = reinterpret_cast<float*>(t_out + MT_H * KC_O * FRAG_ELEMS);
+  float* bias_hid = bias_in + HP;                              // [NH][HP]
+
+  const size_t hh = (size_t)a.d_hidden * a.d_hidden;
+  stage_weight_frags<true, false>(f_in, a.w_in, a.d_hidden, a.d_in, MT_H, KC_IN, tid, nthreads);
+  stage_weight_frags<true, true>(t_in, a.w_in, a.d_hidden, a.d_in, MT_I, KC_H, tid, nthreads);
+  stage_weight_frags<true, true>(t_out, a.w_out, a.d_out, a.d_hidden, MT_H, KC_O, tid, nthreads);
+  stage_bias<T>(bias_in, a.b_in, a.d_hidden, HP, tid, nthreads);
+  for (int k = 0; k < NH; ++k) {
+    stage_weight_frags<true, false>(f_hid + k * HID, a.w_hid + k * hh, a.d_hidden, a.d_hidden, MT_H, KC_H, tid, nthreads);
+    stage_weight_frags<true, true>(t_hid + k * HID, a.w_hid + k * hh, a.d_hidden, a.d_hidden, MT_H, KC_H, tid, nthreads);
+    stage_bias<T>(bias_hid + k * HP, a.b_hid ? a.b_hid + (size_t)k * a.d_hidden : nullptr, a.d_hidden, HP, tid, nthreads);
+  }
+  __syncthreads();
+
+  f32x4_t dw_in[MT_H][MT_I], dw_hid[NH][MT_H][MT_H], dw_out[MT_O][MT_H];
+  float db_in[MT_H], db_hid[NH][MT_H], db_out[MT_O];
+  const f32x4_t zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int i = 0; i < MT_H; ++i) {
+#pragma unroll
+    for (int j = 0; j < MT_I; ++j) dw_in[i][j] = zero4;
+    db_in[i] = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NH; ++k) {
+#pragma unroll
+      for (int j = 0; j < MT_H; ++j) dw_hid[k][i][j] = zero4;
+      db_hid[k][i] = 0.0f;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MT_O; ++i) {
+#pragma unroll
+    for (int j = 0; j < MT_H; ++j) dw_out[i][j] = zero4;
+    db_out[i] = 0.0f;
+  }
+  const Frag sel[2] = {sel_frag<T>(0, lane), sel_frag<T>(1, lane)};
+
+  constexpr int ROWS = 16 * NT;
+  const int64_t n_chunks = (a.rows + ROWS - 1) / ROWS;
+  const int64_t wave_stride = (int64_t)gridDim.x * 4;
+  const int64_t first_chunk = (int64_t)blockIdx.x * 4 + wave;
+  Frag nx[NT][KC_IN], ndy[NT][KC_O];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+    for (int kc = 0; kc < KC_IN; ++kc)
+      nx[nt][kc] = load_chain<FAST>(a.x, a.x_stride, first_chunk * ROWS + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+#pragma unroll
+    for (int kc = 0; kc < KC_O; ++kc)
+      ndy[nt][kc] = load_chain<FAST>(a.dy, a.dy_stride, first_chunk * ROWS + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
+  }
+
+  for (int64_t chunk = first_chunk; chunk < n_chunks; chunk += wave_stride) {
+    const int64_t row0 = chunk * ROWS;
+    Frag in[NT][2], h[NH + 1][NT][2], dz[NT][2];
+    f32x4_t acc[NT][4];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+      for (int kc = 0; kc < KC_IN; ++kc) {
+        in[nt][kc] = nx[nt][kc];
+        nx[nt][kc] = load_chain<FAST>(a.x, a.x_stride, (chunk + wave_stride) * ROWS + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+      }
+#pragma unroll
+      for (int kc = 0; kc < KC_O; ++kc) {
+        dz[nt][kc] = ndy[nt][kc];
+        ndy[nt][kc] = load_chain<FAST>(a.dy, a.dy_stride, (chunk + wave_stride) * ROWS + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
+      }
+    }
+    // ---- forward recompute: h[0] = relu(W_in x + b), h[k] = relu(W_hid[k-1] h[k-1] + b) ----
+    layer_nt<T, NT, MT_H, KC_IN>(acc, in, f_in, bias_in, lane);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT_H; ++mt) {
+        h[0][nt][mt >> 1].w[2 * (mt & 1)] = relu_pk(pack2<T>(acc[nt][mt][0], acc[nt][mt][1]));
+        h[0][nt][mt >> 1].w[2 * (mt & 1) + 1] = relu_pk(pack2<T>(acc[nt][mt][2], acc[nt][mt][3]));
+      }
+#pragma unroll
+    for (int k = 1; k <= NH; ++k) {
+      layer_nt<T, NT, MT_H, KC_H>(acc, h[k - 1], f_hid + (k - 1) * HID, bias_hid + (k - 1) * HP, lane);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT_H; ++mt) {
+          h[k][nt][mt >> 1].w[2 * (mt & 1)] = relu_pk(pack2<T>(acc[nt][mt][0], acc[nt][mt][1]));
+          h[k][nt][mt >> 1].w[2 * (mt & 1) + 1] = relu_pk(pack2<T>(acc[nt][mt][2], acc[nt][mt][3]));
+        }
+    }
+    // ---- output layer: dW_out += dy^T h[NH], db_out += sum dy ; dh = W_out^T dy ----
+    {
+      Frag hb[MT_H];
+#pragma unroll
+      for (int j = 0; j < MT_H; ++j) hb[j] = transpose_tile<T>(h[NH][0][j >> 1], h[NH][1][j >> 1], sel[j & 1]);
+#pragma unroll
+      for (int i = 0; i < MT_O; ++i) {
+        const Frag da = transpose_tile<T>(dz[0][i >> 1], dz[1][i >> 1], sel[i & 1]);
+#pragma unroll
+        for (int j = 0; j < MT_H; ++j) dw_out[i][j] = mfma16<T>(da, hb[j], dw_out[i][j]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) db_out[i] = dot2_ones<T>(da.w[q], db_out[i]);
+      }
+    }
+    layer_nt<T, NT, MT_H, KC_O>(acc, dz, t_out, nullptr, lane);
+    // ---- hidden layers, last first: dz_k = dh_k gated by h[k] ; dW_hid[k-1] += dz_k^T h[k-1] ; dh_{k-1} = W_hid[k-1]^T dz_k
+#pragma unroll
+    for (int k = NH; k >= 1; --k) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT_H; ++mt) {
+          dz[nt][mt >> 1].w[2 * (mt & 1)] = relu_gate_pk(pack2<T>(acc[nt][mt][0], acc[nt][mt][1]), h[k][nt][mt >> 1].w[2 * (mt & 1)]);
+          dz[nt][mt >> 1].w[2 * (mt & 1) + 1] =
+              relu_gate_pk(pack2<T>(acc[nt][mt][2], acc[nt][mt][3]), h[k][nt][mt >> 1].w[2 * (mt & 1) + 1]);
+        }
+      {
+        Frag hb[MT_H];
+#pragma unroll
+        for (int j = 0; j < MT_H; ++j) hb[j] = transpose_tile<T>(h[k - 1][0][j >> 1], h[k - 1][1][j >> 1], sel[j & 1]);
+#pragma unroll
+        for (int i = 0; i < MT_H; ++i) {
+          const Frag da = transpose_tile<T>(dz[0][i >> 1], dz[1][i >> 1], sel[i & 1]);
+#pragma unroll
+          for (int j = 0; j < MT_H; ++j) dw_hid[k - 1][i][j] = mfma16<T>(da, hb[j], dw_hid[k - 1][i][j]);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) db_hid[k - 1][i] = dot2_ones<T>(da.w[q], db_hid[k - 1][i]);
+        }
+      }
+      layer_nt<T, NT, MT_H, KC_H>(acc, dz, t_hid + (k - 1) * HID, nullptr, lane);
+    }
+    // ---- input layer: dz_0 = dh_0 gated by h[0] ; dW_in += dz_0^T x ; dx = W_in^T dz_0 ----
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT_H; ++mt) {
+        dz[nt][mt >> 1].w[2 * (mt & 1)] = relu_gate_pk(pack2<T>(acc[nt][mt][0], acc[nt][mt][1]), h[0][nt][mt >> 1].w[2 * (mt & 1)]);
+        dz[nt][mt >> 1].w[2 * (mt & 1) + 1] =
+            relu_gate_pk(pack2<T>(acc[nt][mt][2], acc[nt][mt][3]), h[0][nt][mt >> 1].w[2 * (mt & 1) + 1]);
+      }
+    {
+      Frag xb[MT_I];
+#pragma unroll
+      for (int j = 0; j < MT_I; ++j) xb[j] = transpose_tile<T>(in[0][j >> 1], in[1][j >> 1], sel[j & 1]);
+#pragma unroll
+      for (int i = 0; i < MT_H; ++i) {
+        const Frag da = transpose_tile<T>(dz[0][i >> 1], dz[1][i >> 1], sel[i & 1]);
+#pragma unroll
+        for (int j = 0; j < MT_I; ++j) dw_in[i][j] = mfma16<T>(da, xb[j], dw_in[i][j]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) db_in[i] = dot2_ones<T>(da.w[q], db_in[i]);
+      }
+    }
+    if (a.dx != nullptr) {
+      layer_nt<T, NT, MT_I, KC_H>(acc, dz, t_in, nullptr, lane);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT_I; ++mt) store_dx<T, FAST>(a, row0 + 16 * nt, mt, lane, acc[nt][mt]);
+    }
+  }
+
+  // ---- reduce the gradients over the four waves through LDS (the weight fragments are dead by now), then
+  // one pass of atomics per workgroup ----
+  __syncthreads();
+  constexpr int N_TILES = MT_H * (MT_I + NH * MT_H) + MT_O * MT_H;
+  f32x4_t* red = reinterpret_cast<f32x4_t*>(smem) + lane;
+  float* redb = reinterpret_cast<float*>(smem) + (size_t)N_TILES * 256 + lane;
+  for (int w = 1; w < 4; ++w) {
+    if (wave == w) {
+      int t = 0, u = 0;
+#pragma unroll
+      for (int i = 0; i < MT_H; ++i) {
+#pragma unroll
+        for (int j = 0; j < MT_I; ++j) red[64 * (t++)] = dw_in[i][j];
+        redb[64 * (u++)] = db_in[i];
+#pragma unroll
+        for (int k = 0; k < NH; ++k) {
+#pragma unroll
+          for (int j = 0; j < MT_H; ++j) red[64 * (t++)] = dw_hid[k][i][j];
+          redb[64 * (u++)] = db_hid[k][i];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < MT_O; ++i) {
+#pragma unroll
+        for (int j = 0; j < MT_H; ++j) red[64 * (t++)] = dw_out[i][j];
+        redb[64 * (u++)] = db_out[i];
+      }
+    }
+    __syncthreads();
+    if (wave == 0) {
+      int t = 0, u = 0;
+#pragma unroll
+      for (int i = 0; i < MT_H; ++i) {
+#pragma unroll
+        for (int j = 0; j < MT_I; ++j) dw_in[i][j] += red[64 * (t++)];
+        db_in[i] += redb[64 * (u++)];
+#pragma unroll
+        for (int k = 0; k < NH; ++k) {
+#pragma unroll
+          for (int j = 0; j < MT_H; ++j) dw_hid[k][i][j] += red[64 * (t++)];
+          db_hid[k][i] += redb[64 * (u++)];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < MT_O; ++i) {
+#pragma unroll
+        for (int j = 0; j < MT_H; ++j) dw_out[i][j] += red[64 * (t++)];
+        db_out[i] += redb[64 * (u++)];
+      }
+    }
+    __syncthreads();
+  }
+  if (wave != 0) return;
+#pragma unroll
+  for (int i = 0; i < MT_H; ++i) {
+#pragma unroll
+    for (int j = 0; j < MT_I; ++j) flush_dw_tile(a.dw_in, a.d_hidden, a.d_in, i, j, lane, dw_in[i][j]);
+    flush_db(a.db_in, a.d_hidden, i, lane, db_in[i]);
+#pragma unroll
+    for (int k = 0; k < NH; ++k) {
+#pragma unroll
+      for (int j = 0; j < MT_H; ++j) flush_dw_tile(a.dw_hid + k * hh, a.d_hidden, a.d_hidden, i, j, lane, dw_hid[k][i][j]);
+      flush_db(a.db_hid ? a.db_hid + (size_t)k * a.d_hidden : nullptr, a.d_hidden, i, lane, db_hid[k][i]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MT_O; ++i) {
+#pragma unroll
+    for (int j = 0; j < MT_H; ++j) flush_dw_tile(a.dw_out, a.d_out, a.d_hidden, i, j, lane, dw_out[i][j]);
+    flush_db(a.db_out, a.d_out, i, lane, db_out[i]);
+  }
+}
+
+template <typename T, int KIN, int HP, int OUTP, int NH>
+static int launchn(const MlpArgs& a0, hipStream_t s) {
+  MlpArgs a = a0;
+  constexpr int KC_O = (OUTP + 31) / 32;
+  constexpr int MT_H = HP / 16, MT_I = KIN / 16, MT_O = OUTP / 16;
+  constexpr size_t W_BYTES = ((size_t)MT_H * (KIN / 32) + (size_t)MT_I * (HP / 32) + 2 * (size_t)NH * MT_H * (HP / 32) + (size_t)MT_H * KC_O) * 1024 +
+                             (size_t)(1 + NH) * HP * 4;
+  constexpr size_t RED = (size_t)(MT_H * (MT_I + NH * MT_H) + MT_O * MT_H) * 1024 + (size_t)((1 + NH) * MT_H + MT_O) * 256;
+  constexpr size_t LDS = W_BYTES > RED ? W_BYTES : RED;
+  static_assert(LDS <= 160 * 1024, "LDS budget");
+  a.waves = 4;
+  a.x_vec = ((uintptr_t)a.x % 8 == 0) && (a.x_stride % 4 == 0);
+  a.dy_vec = ((uintptr_t)a.dy % 8 == 0) && (a.dy_stride % 4 == 0);
+  const int64_t chunks = (a.rows + 31) / 32;
+  int64_t blocks = (chunks + 3) / 4;
+  const int64_t cap = (int64_t)device_cus();
+  if (blocks > cap) blocks = cap;
+  const bool fast = a.x_vec && a.dy_vec && a.d_in % 4 == 0 && a.d_out % 4 == 0 &&
+                    (a.dx == nullptr || ((uintptr_t)a.dx % 8 == 0 && a.dx_stride % 4 == 0));
+  const void* kern = fast ? (const void*)mlp_bwdn_k<T, KIN, HP, OUTP, NH, true> : (const void*)mlp_bwdn_k<T, KIN, HP, OUTP, NH, false>;
+  if (LDS > 64 * 1024) {
+    const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
+    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  }
+  void* args[] = {(void*)&a};
+  const hipError_t e = hipLaunchKernel(kern, dim3((unsigned)blocks), dim3(256), args, LDS, s);
+  if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(mlp_bwdn): %s", hipGetErrorString(e));
+  return check_launch("mlp_bwdn");
+}
+
+template <typename T, int NH>
+static int dispatchn(const MlpArgs& a, hipStream_t s) {
+  const int kin = (a.d_in + 31) / 32 * 32, outp = a.d_out <= 16 ? 16 : 64;
+  if (kin == 32 && outp == 16) return launchn<T, 32, 64, 16, NH>(a, s);
+  if (kin == 32) return launchn<T, 32, 64, 64, NH>(a, s);
+  if (outp == 16) return launchn<T, 64, 64, 16, NH>(a, s);
+  return launchn<T, 64, 64, 64, NH>(a, s);
+}
+
 template <typename T, int KIN, int HP, int OUTP>
 static int launch2(const MlpArgs& a0, hipStream_t s) {
   MlpArgs a = a0;
@@ -472,8 +766,13 @@ static int dispatch2(const MlpArgs& a, hipStream_t s, bool* handled) {
 
 int launch_mlp_bwd2(const MlpArgs& a, int dtype, hipStream_t s, bool* handled) {
   *handled = false;
-  if (a.depth != 2) return 0;
-  return dtype == NF_BF16 ? dispatch2<BF16>(a, s, handled) : dispatch2<F16>(a, s, handled);
+  if (a.depth == 2) return dtype == NF_BF16 ? dispatch2<BF16>(a, s, handled) : dispatch2<F16>(a, s, handled);
+  // two hidden-to-hidden layers: the register-resident kernel covers wide ReLU nets with x in the parameters' dtype
+  if (a.depth == 3 && a.d_hidden > 32 && a.act == NF_ACT_RELU && a.x_conv == 0) {
+    *handled = true;
+    return dtype == NF_BF16 ? dispatchn<BF16, 2>(a, s) : dispatchn<F16, 2>(a, s);
+  }
+  return 0;
 }
 
 }  // namespace nf
