@@ -74,7 +74,8 @@ SHAPES = [
     ((1, 4097), 32, 64, 4, 2),   # BASELINE configs[4] geometry, ragged rows
     ((5, 77), 64, 64, 64, 4),
     ((2, 33), 17, 32, 33, 2),
-    # two hidden-to-hidden layers of width 64: ReLU takes the register-resident backward for deeper nets
+    # two or three hidden-to-hidden layers of width 64: ReLU takes the register-resident backward for deeper nets
+    ((1, 1000), 32, 64, 16, 4),
     ((1, 1000), 32, 64, 16, 3),
     ((3, 100), 64, 64, 64, 3),
     ((2, 77), 40, 64, 20, 3),

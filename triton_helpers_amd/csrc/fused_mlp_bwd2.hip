@@ -420,6 +420,14 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
 // hidden activation of the chunk stays in registers (they are the gates as well), every weight gradient in float32
 // accumulators over the wave's row loop; the weights of all layers, in both forms, are resident in LDS.
 // ---------------------------------------------------------------------------------------
+// hidden-to-hidden weight gradients that accumulate in LDS instead of registers
+// (measured on the compiler: with two in registers the two-layer kernels spill where the input or output layer is 64
+// wide, the three-layer kernels, whose third accumulator is in LDS anyway, do not)
+constexpr int bwdn_lds_layers(int kin, int outp, int nh) {
+  if (nh >= 3) return nh - 2;
+  return (kin == 32 && outp == 16) ? 0 : 1;
+}
+
 template <typename T, int KIN, int HP, int OUTP, int NH, bool FAST>
 __global__ __launch_bounds__(256) void mlp_bwdn_k(MlpArgs a) {
   constexpr int KC_IN = KIN / 32, KC_H = HP / 32, MT_H = HP / 16, MT_I = KIN / 16, MT_O = OUTP / 16;
@@ -437,6 +445,15 @@ __global__ __launch_bounds__(256) void mlp_bwdn_k(MlpArgs a) {
   uint16_t* t_out = t_hid + NH * HID;                          // W_out^T   [MT_H][KC_O]
   float* bias_in = reinterpret_cast<float*>(t_out + MT_H * KC_O * FRAG_ELEMS);
   float* bias_hid = bias_in + HP;                              // [NH][HP]
+  // One or two 64x64 hidden accumulators stay in registers next to the rest; the others live in LDS, 16 KiB per
+  // wave and layer (the layers of highest index).
+  constexpr int LA = bwdn_lds_layers(KIN, OUTP, NH), NREG = NH - LA;
+  constexpr size_t W_BYTES = ((size_t)MT_H * KC_IN + (size_t)MT_I * KC_H + 2 * (size_t)NH * MT_H * KC_H + (size_t)MT_H * KC_O) * 1024 +
+                             (size_t)(1 + NH) * HP * 4;
+  constexpr size_t RED_BYTES = (size_t)(MT_H * (MT_I + NREG * MT_H) + MT_O * MT_H) * 1024 + (size_t)((1 + NH) * MT_H + MT_O) * 256;
+  constexpr size_t LACC_AT = W_BYTES > RED_BYTES ? W_BYTES : RED_BYTES;  // behind the weights and the closing reduction's area
+  f32x4_t* lacc = reinterpret_cast<f32x4_t*>(smem + LACC_AT) + (size_t)wave * (LA * MT_H * MT_H * 64);
+  for (int i = lane; i < LA * MT_H * MT_H * 64; i += 64) lacc[i] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
   const size_t hh = (size_t)a.d_hidden * a.d_hidden;
   stage_weight_frags<true, false>(f_in, a.w_in, a.d_hidden, a.d_in, MT_H, KC_IN, tid, nthreads);
@@ -450,7 +467,7 @@ __global__ __launch_bounds__(256) void mlp_bwdn_k(MlpArgs a) {
   }
   __syncthreads();
 
-  f32x4_t dw_in[MT_H][MT_I], dw_hid[NH][MT_H][MT_H], dw_out[MT_O][MT_H];
+  f32x4_t dw_in[MT_H][MT_I], dw_hid[NREG][MT_H][MT_H], dw_out[MT_O][MT_H];
   float db_in[MT_H], db_hid[NH][MT_H], db_out[MT_O];
   const f32x4_t zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -460,8 +477,10 @@ __global__ __launch_bounds__(256) void mlp_bwdn_k(MlpArgs a) {
     db_in[i] = 0.0f;
 #pragma unroll
     for (int k = 0; k < NH; ++k) {
+      if (k < NREG) {
 #pragma unroll
-      for (int j = 0; j < MT_H; ++j) dw_hid[k][i][j] = zero4;
+        for (int j = 0; j < MT_H; ++j) dw_hid[k < NREG ? k : 0][i][j] = zero4;
+      }
       db_hid[k][i] = 0.0f;
     }
   }
@@ -558,8 +577,17 @@ __global__ __launch_bounds__(256) void mlp_bwdn_k(MlpArgs a) {
 #pragma unroll
         for (int i = 0; i < MT_H; ++i) {
           const Frag da = transpose_tile<T>(dz[0][i >> 1], dz[1][i >> 1], sel[i & 1]);
+          if (k - 1 < NREG) {
 #pragma unroll
-          for (int j = 0; j < MT_H; ++j) dw_hid[k - 1][i][j] = mfma16<T>(da, hb[j], dw_hid[k - 1][i][j]);
+            for (int j = 0; j < MT_H; ++j)
+              dw_hid[k - 1 < NREG ? k - 1 : 0][i][j] = mfma16<T>(da, hb[j], dw_hid[k - 1 < NREG ? k - 1 : 0][i][j]);
+          } else {
+#pragma unroll
+            for (int j = 0; j < MT_H; ++j) {
+              f32x4_t* slot = lacc + (((k - 1 - NREG) * MT_H + i) * MT_H + j) * 64 + lane;
+              *slot = mfma16<T>(da, hb[j], *slot);
+            }
+          }
 #pragma unroll
           for (int q = 0; q < 4; ++q) db_hid[k - 1][i] = dot2_ones<T>(da.w[q], db_hid[k - 1][i]);
         }
@@ -600,7 +628,7 @@ __global__ __launch_bounds__(256) void mlp_bwdn_k(MlpArgs a) {
   // ---- reduce the gradients over the four waves through LDS (the weight fragments are dead by now), then
   // one pass of atomics per workgroup ----
   __syncthreads();
-  constexpr int N_TILES = MT_H * (MT_I + NH * MT_H) + MT_O * MT_H;
+  constexpr int N_TILES = MT_H * (MT_I + NREG * MT_H) + MT_O * MT_H;
   f32x4_t* red = reinterpret_cast<f32x4_t*>(smem) + lane;
   float* redb = reinterpret_cast<float*>(smem) + (size_t)N_TILES * 256 + lane;
   for (int w = 1; w < 4; ++w) {
@@ -613,8 +641,10 @@ __global__ __launch_bounds__(256) void mlp_bwdn_k(MlpArgs a) {
         redb[64 * (u++)] = db_in[i];
 #pragma unroll
         for (int k = 0; k < NH; ++k) {
+          if (k < NREG) {
 #pragma unroll
-          for (int j = 0; j < MT_H; ++j) red[64 * (t++)] = dw_hid[k][i][j];
+            for (int j = 0; j < MT_H; ++j) red[64 * (t++)] = dw_hid[k < NREG ? k : 0][i][j];
+          }
           redb[64 * (u++)] = db_hid[k][i];
         }
       }
@@ -635,8 +665,10 @@ __global__ __launch_bounds__(256) void mlp_bwdn_k(MlpArgs a) {
         db_in[i] += redb[64 * (u++)];
 #pragma unroll
         for (int k = 0; k < NH; ++k) {
+          if (k < NREG) {
 #pragma unroll
-          for (int j = 0; j < MT_H; ++j) dw_hid[k][i][j] += red[64 * (t++)];
+            for (int j = 0; j < MT_H; ++j) dw_hid[k < NREG ? k : 0][i][j] += red[64 * (t++)];
+          }
           db_hid[k][i] += redb[64 * (u++)];
         }
       }
@@ -658,7 +690,17 @@ __global__ __launch_bounds__(256) void mlp_bwdn_k(MlpArgs a) {
 #pragma unroll
     for (int k = 0; k < NH; ++k) {
 #pragma unroll
-      for (int j = 0; j < MT_H; ++j) flush_dw_tile(a.dw_hid + k * hh, a.d_hidden, a.d_hidden, i, j, lane, dw_hid[k][i][j]);
+      for (int j = 0; j < MT_H; ++j) {
+        f32x4_t v;
+        if (k < NREG) {
+          v = dw_hid[k < NREG ? k : 0][i][j];
+        } else {  // wave 0's LDS tiles are the first of the four waves'
+          constexpr int PER_WAVE = LA * MT_H * MT_H * 64;
+          const int at = (((k - NREG) * MT_H + i) * MT_H + j) * 64 + lane;
+          v = (lacc[at] + lacc[PER_WAVE + at]) + (lacc[2 * PER_WAVE + at] + lacc[3 * PER_WAVE + at]);
+        }
+        flush_dw_tile(a.dw_hid + k * hh, a.d_hidden, a.d_hidden, i, j, lane, v);
+      }
       flush_db(a.db_hid ? a.db_hid + (size_t)k * a.d_hidden : nullptr, a.d_hidden, i, lane, db_hid[k][i]);
     }
   }
@@ -677,8 +719,9 @@ static int launchn(const MlpArgs& a0, hipStream_t s) {
   constexpr int MT_H = HP / 16, MT_I = KIN / 16, MT_O = OUTP / 16;
   constexpr size_t W_BYTES = ((size_t)MT_H * (KIN / 32) + (size_t)MT_I * (HP / 32) + 2 * (size_t)NH * MT_H * (HP / 32) + (size_t)MT_H * KC_O) * 1024 +
                              (size_t)(1 + NH) * HP * 4;
-  constexpr size_t RED = (size_t)(MT_H * (MT_I + NH * MT_H) + MT_O * MT_H) * 1024 + (size_t)((1 + NH) * MT_H + MT_O) * 256;
-  constexpr size_t LDS = W_BYTES > RED ? W_BYTES : RED;
+  constexpr int LA = bwdn_lds_layers(KIN, OUTP, NH);  // hidden accumulators kept in LDS, behind the weights
+  constexpr size_t RED = (size_t)(MT_H * (MT_I + (NH - LA) * MT_H) + MT_O * MT_H) * 1024 + (size_t)((1 + NH) * MT_H + MT_O) * 256;
+  constexpr size_t LDS = (W_BYTES > RED ? W_BYTES : RED) + (size_t)4 * LA * MT_H * MT_H * 1024;
   static_assert(LDS <= 160 * 1024, "LDS budget");
   a.waves = 4;
   a.x_vec = ((uintptr_t)a.x % 8 == 0) && (a.x_stride % 4 == 0);
@@ -771,6 +814,10 @@ int launch_mlp_bwd2(const MlpArgs& a, int dtype, hipStream_t s, bool* handled) {
   if (a.depth == 3 && a.d_hidden > 32 && a.act == NF_ACT_RELU && a.x_conv == 0) {
     *handled = true;
     return dtype == NF_BF16 ? dispatchn<BF16, 2>(a, s) : dispatchn<F16, 2>(a, s);
+  }
+  if (a.depth == 4 && a.d_hidden > 32 && a.act == NF_ACT_RELU && a.x_conv == 0) {
+    *handled = true;
+    return dtype == NF_BF16 ? dispatchn<BF16, 3>(a, s) : dispatchn<F16, 3>(a, s);
   }
   return 0;
 }
