@@ -213,6 +213,29 @@ def test_backward_lds_tile_path(N, T, L, lo, hi, do_dtype, variant):
 
 
 @pytest.mark.parametrize("do_dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("N,T,L,lo,hi", [(40000, 2**14, 16, 16, 512), (70001, 2**19, 8, 16, 4096), (33000, 2**12, 4, 8, 64)])
+def test_backward_binned_two_dimensions(N, T, L, lo, hi, do_dtype):
+    """2-D coordinates take the binned backward too (two x-pairs per point and level): against the oracle and the
+    scattered-atomic kernel, with points on the cell borders."""
+    hk = _hk()
+    torch.manual_seed(4)
+    x = torch.rand(N, 2)
+    x[:5] = torch.tensor([[0.0, 0.0], [1.0, 1.0], [1.0, 0.0], [0.999999, 0.5], [0.5, 1.0]])
+    E = O.level_row_offsets(L, T, 2, lo, hi)[-1]
+    do = torch.randn(N, L * 2).to(do_dtype)
+    want = O.encode_backward(x, do, E, 2, None, T, L, lo, hi)
+    got = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, 2, None, T, lo, hi, L)
+    hk._FLAGS = 2
+    try:
+        ref = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, 2, None, T, lo, hi, L)
+    finally:
+        hk._FLAGS = 0
+    scale = max(1.0, float(want.abs().max()))
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-3, atol=1e-4 * scale)
+    torch.testing.assert_close(got, ref, rtol=1e-3, atol=1e-4 * scale)
+
+
+@pytest.mark.parametrize("do_dtype", [torch.float16, torch.float32])
 def test_backward_binned_clustered_points(do_dtype):
     """Clustered input: a few cells receive everything, so their bins are cut into several accumulation tasks
     (atomic flush), and x = 8191 sits on a bin border of the dense levels / has 13 trailing ones on hashed levels, so

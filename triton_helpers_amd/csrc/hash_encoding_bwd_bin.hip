@@ -105,6 +105,59 @@ __device__ __forceinline__ void load_point(const void* coords, int cdt, int64_t 
   }
 }
 
+// Table rows (and trilinear / bilinear weights) of the 2^D corners of a point's cell, corner j = bit pattern of its
+// offsets with x in bit 0, so that corners 2c and 2c+1 are an x-pair.  D = 3 or 2.
+template <int D>
+__device__ __forceinline__ void cell_rows(const float (&v)[3], float fres, bool hashed, uint32_t res, uint32_t mask,
+                                          const uint32_t (&pi)[3], uint32_t (&row)[1 << D], float* w) {
+  if (D == 3) {
+    const Located3 q = locate(v, fres);
+    const Corner8 r = rows_d3(q.c, hashed, res, mask, pi);
+#pragma unroll
+    for (int j = 0; j < (1 << D); ++j) row[j] = r.row[j];
+    if (w != nullptr) weights_d3(q.fr, w);
+  } else {
+    uint32_t c[2];
+    float fr[2];
+#pragma unroll
+    for (int d = 0; d < 2; ++d) {
+      const float pos = v[d] * fres;
+      const float fl = floorf(pos);
+      c[d] = (uint32_t)(int)fl;
+      fr[d] = pos - fl;
+    }
+    if (hashed) {
+      const uint32_t x0 = c[0] * pi[0], x1 = x0 + pi[0], y0 = c[1] * pi[1], y1 = y0 + pi[1];
+      row[0] = (x0 ^ y0) & mask;
+      row[1] = (x1 ^ y0) & mask;
+      row[2] = (x0 ^ y1) & mask;
+      row[3] = (x1 ^ y1) & mask;
+    } else {
+      const uint32_t b = c[0] + c[1] * res;
+      row[0] = b;
+      row[1] = b + 1;
+      row[2] = b + res;
+      row[3] = b + res + 1;
+    }
+    if (w != nullptr) {
+      const float gx = 1.0f - fr[0], gy = 1.0f - fr[1];
+      w[0] = gx * gy;
+      w[1] = fr[0] * gy;
+      w[2] = gx * fr[1];
+      w[3] = fr[0] * fr[1];
+    }
+  }
+}
+template <int D>
+__device__ __forceinline__ void load_point_d(const void* coords, int cdt, int64_t csn, int64_t csd, int64_t n, float scale,
+                                             float (&v)[3]) {
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    v[d] = load_as_f32(coords, n * csn + d * csd, cdt);
+    if (scale != 1.0f) v[d] = v[d] / scale;
+  }
+}
+
 // Position of every active lane among the wave's lanes with the same bin, on top of one LDS add per distinct bin.
 __device__ __forceinline__ uint32_t wave_rank(uint32_t* cnt, uint32_t bin, bool active, int lane) {
   uint32_t rank = 0;
@@ -144,6 +197,7 @@ __global__ void hash_bwd_bin_zero_k(uint32_t* p, int n) {
 // ---------------------------------------------------------------------------------------
 // count
 // ---------------------------------------------------------------------------------------
+template <int D>
 __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_count_k(const void* coords, int cdt, int64_t csn, int64_t csd,
                                                                     int64_t N, DevGeom g, BinPlan bp, const int64_t* primes,
                                                                     float scale, uint32_t* hist, uint32_t* wg_counts) {
@@ -155,23 +209,24 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_count_k(const void* 
   const int64_t n = (int64_t)blockIdx.x * FILL_POINTS + tid;
   const bool valid = n < N;
   float v[3] = {0.0f, 0.0f, 0.0f};
-  if (valid) load_point(coords, cdt, csn, csd, n, scale, v);
-  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], (uint32_t)primes[2]};
+  constexpr int PAIRS = 1 << (D - 1);
+  if (valid) load_point_d<D>(coords, cdt, csn, csd, n, scale, v);
+  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], D > 2 ? (uint32_t)primes[D > 2 ? 2 : 0] : 0u};
   for (int l = 0; l < bp.n_levels; ++l) {
     uint32_t* cnt = lh + bp.binbase[l];
     const int nb = bp.nbins[l];
     if (nb == 1) {
       if (valid) {
         const unsigned long long m = __ballot(true);
-        if (lane == __ffsll((long long)m) - 1) atomicAdd(cnt, 4u * (uint32_t)__popcll(m));
+        if (lane == __ffsll((long long)m) - 1) atomicAdd(cnt, (uint32_t)PAIRS * (uint32_t)__popcll(m));
       }
       continue;
     }
-    const Located3 q = locate(v, (float)g.res[l]);
-    const Corner8 r = rows_d3(q.c, l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi);
+    uint32_t row[1 << D];
+    cell_rows<D>(v, (float)g.res[l], l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi, row, nullptr);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const uint32_t b0 = r.row[2 * c] >> BIN_ROWS_LOG2, b1 = r.row[2 * c + 1] >> BIN_ROWS_LOG2;
+    for (int c = 0; c < PAIRS; ++c) {
+      const uint32_t b0 = row[2 * c] >> BIN_ROWS_LOG2, b1 = row[2 * c + 1] >> BIN_ROWS_LOG2;
       if (nb <= AGG_MAX_BINS) {
         wave_rank(cnt, b0, valid, lane);
         if (__any(valid && b1 != b0)) wave_rank(cnt, b1, valid && b1 != b0, lane);
@@ -248,7 +303,7 @@ __global__ __launch_bounds__(1024) void hash_bwd_bin_offsets_k(const uint32_t* h
 // G32 = false: 16-bit upstream gradient, 12-byte records {.., .., packed pair}.  G32 = true: float32 upstream gradient,
 // 16-byte records {.., .., g0, g1}; a staged entry then names the point instead of carrying the pair, and the copy-out
 // takes the pair from the workgroup's per-level gradient table in LDS (the stage has no room for 20-byte entries).
-template <bool G32>
+template <bool G32, int D>
 __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* coords, int cdt, int64_t csn, int64_t csd,
                                                                    const void* dout_v, int64_t dout_stride, int64_t N,
                                                                    DevGeom g, BinPlan bp, const int64_t* primes, float scale,
@@ -278,8 +333,9 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
   }
   if (tid < NF_MAX_LEVELS) lmax[tid] = 0u;
   float v[3] = {0.0f, 0.0f, 0.0f};
-  if (valid) load_point(coords, cdt, csn, csd, n, scale, v);
-  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], (uint32_t)primes[2]};
+  constexpr int PAIRS = 1 << (D - 1);
+  if (valid) load_point_d<D>(coords, cdt, csn, csd, n, scale, v);
+  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], D > 2 ? (uint32_t)primes[D > 2 ? 2 : 0] : 0u};
   // this point's gradient row, read once (up to 16 levels live in registers); float32 rows are read level by level
   const uint32_t* grow = reinterpret_cast<const uint32_t*>(dout + (valid ? n : 0) * dout_stride);
   const uint2* grow32 = reinterpret_cast<const uint2*>(reinterpret_cast<const float*>(dout_v) + (valid ? n : 0) * dout_stride);
@@ -346,38 +402,37 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
       if (lane == 63 && m) atomicMax(lmax + l, m);
     }
     {
-      const Located3 q = locate(v, (float)g.res[l]);
-      const Corner8 r = rows_d3(q.c, l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi);
-      float w[8];
-      weights_d3(q.fr, w);
-      // The four x-pairs of the point: their ranks are asked for together, so that a wave waits for LDS once per level
-      // and not once per pair.
-      uint32_t b0[4], b1[4], pos[4], dlt[4];
-      bool split[4];
+      uint32_t row[1 << D];
+      float w[1 << D];
+      cell_rows<D>(v, (float)g.res[l], l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi, row, w);
+      // The x-pairs of the point (four in 3-D, two in 2-D): their ranks are asked for together, so that a wave waits
+      // for LDS once per level and not once per pair.
+      uint32_t b0[PAIRS], b1[PAIRS], pos[PAIRS], dlt[PAIRS];
+      bool split[PAIRS];
       bool any_split = false;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        b0[c] = r.row[2 * c] >> BIN_ROWS_LOG2;
-        b1[c] = r.row[2 * c + 1] >> BIN_ROWS_LOG2;
+      for (int c = 0; c < PAIRS; ++c) {
+        b0[c] = row[2 * c] >> BIN_ROWS_LOG2;
+        b1[c] = row[2 * c + 1] >> BIN_ROWS_LOG2;
         split[c] = b1[c] != b0[c];
         any_split = any_split || split[c];
       }
       if (nb == 1) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) pos[c] = (uint32_t)tid * 4u + (uint32_t)c;  // the valid points are the first of the workgroup
+        for (int c = 0; c < PAIRS; ++c) pos[c] = (uint32_t)tid * (uint32_t)PAIRS + (uint32_t)c;  // the valid points are the first of the workgroup
       } else if (nb <= AGG_MAX_BINS) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) pos[c] = wave_rank(lcur, b0[c], valid, lane);
+        for (int c = 0; c < PAIRS; ++c) pos[c] = wave_rank(lcur, b0[c], valid, lane);
       } else {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) pos[c] = valid ? atomicAdd(lcur + b0[c], 1u) : 0u;
+        for (int c = 0; c < PAIRS; ++c) pos[c] = valid ? atomicAdd(lcur + b0[c], 1u) : 0u;
       }
 #pragma unroll
-      for (int c = 0; c < 4; ++c) dlt[c] = ldelta[b0[c]];
+      for (int c = 0; c < PAIRS; ++c) dlt[c] = ldelta[b0[c]];
       if (valid) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const uint32_t r0 = r.row[2 * c], r1 = r.row[2 * c + 1];
+        for (int c = 0; c < PAIRS; ++c) {
+          const uint32_t r0 = row[2 * c], r1 = row[2 * c + 1];
           const uint3 rec = make_record(r0 & BIN_MASK, (split[c] ? r0 : r1) & BIN_MASK, w[2 * c], split[c] ? 0.0f : w[2 * c + 1], packed);
           stage[pos[c]] = G32 ? make_uint4(rec.x, rec.y, pos[c] + dlt[c], rec.z) : make_uint4(rec.x, rec.y, rec.z, pos[c] + dlt[c]);
         }
@@ -385,14 +440,14 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
       // a pair that straddles two bins leaves its second corner as a record of its own (rare)
       if (nb > 1 && __any(valid && any_split)) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
+        for (int c = 0; c < PAIRS; ++c) {
           const bool on = valid && split[c];
           if (!__any(on)) continue;
           uint32_t pos1;
           if (nb <= AGG_MAX_BINS) pos1 = wave_rank(lcur, b1[c], on, lane);
           else pos1 = on ? atomicAdd(lcur + b1[c], 1u) : 0u;
           if (on) {
-            const uint32_t r1 = r.row[2 * c + 1];
+            const uint32_t r1 = row[2 * c + 1];
             const uint3 rec = make_record(r1 & BIN_MASK, r1 & BIN_MASK, w[2 * c + 1], 0.0f, packed);
             const uint32_t gp = pos1 + ldelta[b1[c]];
             stage[pos1] = G32 ? make_uint4(rec.x, rec.y, gp, rec.z) : make_uint4(rec.x, rec.y, rec.z, gp);
@@ -538,7 +593,7 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const typena
 // Host side
 // ---------------------------------------------------------------------------------------
 static bool bin_plan(int64_t N, const nf_hash_geom* geom, int dout_dtype, BinPlan* bp, int64_t* records, uint32_t* max_tasks) {
-  if (geom->dims != 3 || geom->feat != 2 || N <= 0) return false;
+  if ((geom->dims != 3 && geom->dims != 2) || geom->feat != 2 || N <= 0) return false;
   bp->n_levels = geom->levels;
   int nb_total = 0;
   for (int l = 0; l < geom->levels; ++l) {
@@ -553,7 +608,7 @@ static bool bin_plan(int64_t N, const nf_hash_geom* geom, int dout_dtype, BinPla
   bp->binbase[geom->levels] = nb_total;
   if (nb_total > MAX_BINS_TOTAL) return false;
   // room for every pair to be split in two; normally half of it is used
-  const int64_t R = N * geom->levels * 8;
+  const int64_t R = N * geom->levels * (geom->dims == 3 ? 8 : 4);
   if (R >= ((int64_t)1 << 32) - 4 * ACC_THREADS * ACC_INFLIGHT) return false;  // 32-bit record positions
   *records = R;
   *max_tasks = (uint32_t)(nb_total + R / SPLIT_RECORDS + 1);
@@ -605,8 +660,12 @@ int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const 
 
   hipLaunchKernelGGL(hash_bwd_bin_zero_k, dim3((unsigned)((NBp + 32 + 255) / 256)), dim3(256), 0, s, ws.hist, NBp + 32);
   if (int rc = check_launch("hash_bwd_bin_zero")) return rc;
-  hipLaunchKernelGGL(hash_bwd_bin_count_k, dim3(blocks), dim3(FILL_POINTS), (size_t)NB * 4, s, coords, cdt, csn, csd, N, g, bp,
-                     primes, scale, ws.hist, ws.wg_counts);
+  if (g.dims == 3)
+    hipLaunchKernelGGL(hash_bwd_bin_count_k<3>, dim3(blocks), dim3(FILL_POINTS), (size_t)NB * 4, s, coords, cdt, csn, csd, N, g, bp,
+                       primes, scale, ws.hist, ws.wg_counts);
+  else
+    hipLaunchKernelGGL(hash_bwd_bin_count_k<2>, dim3(blocks), dim3(FILL_POINTS), (size_t)NB * 4, s, coords, cdt, csn, csd, N, g, bp,
+                       primes, scale, ws.hist, ws.wg_counts);
   if (int rc = check_launch("hash_bwd_bin_count")) return rc;
   hipLaunchKernelGGL(hash_bwd_bin_offsets_k, dim3(1), dim3(1024), 0, s, (const uint32_t*)ws.hist, ws.cursor, ws.n_tasks,
                      ws.tasks, NB, max_tasks);
@@ -614,7 +673,8 @@ int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const 
   {
     const size_t lds = (size_t)FILL_RECORDS * sizeof(uint4) + (g32 ? (size_t)FILL_POINTS * sizeof(uint2) : 0) +
                        ((size_t)2 * NB + 2 * NF_MAX_LEVELS) * 4;
-    const void* kern = g32 ? (const void*)hash_bwd_bin_fill_k<true> : (const void*)hash_bwd_bin_fill_k<false>;
+    const void* kern = g.dims == 3 ? (g32 ? (const void*)hash_bwd_bin_fill_k<true, 3> : (const void*)hash_bwd_bin_fill_k<false, 3>)
+                                   : (g32 ? (const void*)hash_bwd_bin_fill_k<true, 2> : (const void*)hash_bwd_bin_fill_k<false, 2>);
     hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     const uint32_t* wc = ws.wg_counts;
