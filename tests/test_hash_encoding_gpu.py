@@ -184,6 +184,7 @@ def test_backward_vs_oracle(N, D, F, T, L, lo, hi, scale, do_dtype, flags, monke
         (50001, 2**16, 8, 16, 2048),    # 4 tiles per hashed level, ragged point count
         (40000, 2**19, 4, 4096, 30000), # resolutions above the tile size: the x corner moves the tile id
         (45000, 2**12, 4, 8, 64),       # hashed levels smaller than a tile
+        (40000, 12345, 8, 16, 512),     # hashed level size not a power of two: exact 64-bit remainder
     ],
 )
 @pytest.mark.parametrize("variant", [0, 4])  # 0: binned records, 4: bit-planes (NF_HASH_FORCE_PLANES)
@@ -213,7 +214,8 @@ def test_backward_lds_tile_path(N, T, L, lo, hi, do_dtype, variant):
 
 
 @pytest.mark.parametrize("do_dtype", [torch.float16, torch.float32])
-@pytest.mark.parametrize("N,T,L,lo,hi", [(40000, 2**14, 16, 16, 512), (70001, 2**19, 8, 16, 4096), (33000, 2**12, 4, 8, 64)])
+@pytest.mark.parametrize("N,T,L,lo,hi", [(40000, 2**14, 16, 16, 512), (70001, 2**19, 8, 16, 4096), (33000, 2**12, 4, 8, 64),
+                                        (40000, 5000, 4, 8, 256)])
 def test_backward_binned_two_dimensions(N, T, L, lo, hi, do_dtype):
     """2-D coordinates take the binned backward too (two x-pairs per point and level): against the oracle and the
     scattered-atomic kernel, with points on the cell borders."""

@@ -107,9 +107,42 @@ __device__ __forceinline__ void load_point(const void* coords, int cdt, int64_t 
 
 // Table rows (and trilinear / bilinear weights) of the 2^D corners of a point's cell, corner j = bit pattern of its
 // offsets with x in bit 0, so that corners 2c and 2c+1 are an x-pair.  D = 3 or 2.
+// A hashed level whose size is not a power of two takes the exact remainder of the 64-bit hash (the reference's
+// CPU form) instead of the 32-bit wrap-around and mask.
 template <int D>
 __device__ __forceinline__ void cell_rows(const float (&v)[3], float fres, bool hashed, uint32_t res, uint32_t mask,
-                                          const uint32_t (&pi)[3], uint32_t (&row)[1 << D], float* w) {
+                                          const uint32_t (&pi)[3], const int64_t* primes, uint32_t (&row)[1 << D], float* w) {
+  const uint32_t n_rows = mask + 1u;
+  if (hashed && (n_rows & mask) != 0u) {
+    uint32_t c[D];
+    float fr[3] = {0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const float pos = v[d] * fres;
+      const float fl = floorf(pos);
+      c[d] = (uint32_t)(int)fl;
+      fr[d] = pos - fl;
+    }
+#pragma unroll
+    for (int j = 0; j < (1 << D); ++j) {
+      uint64_t h = 0;
+#pragma unroll
+      for (int d = 0; d < D; ++d) h ^= (uint64_t)(c[d] + ((j >> d) & 1)) * (uint64_t)primes[d];
+      row[j] = (uint32_t)(h % (uint64_t)n_rows);
+    }
+    if (w != nullptr) {
+      if (D == 3) {
+        weights_d3(fr, w);
+      } else {
+        const float gx = 1.0f - fr[0], gy = 1.0f - fr[1];
+        w[0] = gx * gy;
+        w[1] = fr[0] * gy;
+        w[2] = gx * fr[1];
+        w[3] = fr[0] * fr[1];
+      }
+    }
+    return;
+  }
   if (D == 3) {
     const Located3 q = locate(v, fres);
     const Corner8 r = rows_d3(q.c, hashed, res, mask, pi);
@@ -223,7 +256,7 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_count_k(const void* 
       continue;
     }
     uint32_t row[1 << D];
-    cell_rows<D>(v, (float)g.res[l], l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi, row, nullptr);
+    cell_rows<D>(v, (float)g.res[l], l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi, primes, row, nullptr);
 #pragma unroll
     for (int c = 0; c < PAIRS; ++c) {
       const uint32_t b0 = row[2 * c] >> BIN_ROWS_LOG2, b1 = row[2 * c + 1] >> BIN_ROWS_LOG2;
@@ -404,7 +437,7 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
     {
       uint32_t row[1 << D];
       float w[1 << D];
-      cell_rows<D>(v, (float)g.res[l], l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi, row, w);
+      cell_rows<D>(v, (float)g.res[l], l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi, primes, row, w);
       // The x-pairs of the point (four in 3-D, two in 2-D): their ranks are asked for together, so that a wave waits
       // for LDS once per level and not once per pair.
       uint32_t b0[PAIRS], b1[PAIRS], pos[PAIRS], dlt[PAIRS];
@@ -598,7 +631,6 @@ static bool bin_plan(int64_t N, const nf_hash_geom* geom, int dout_dtype, BinPla
   int nb_total = 0;
   for (int l = 0; l < geom->levels; ++l) {
     const int64_t r = geom->rows[l];
-    if (l >= geom->first_hash_level && (r & (r - 1)) != 0) return false;  // hashed levels: power-of-two sizes
     const int64_t nb = (r + BIN_ROWS - 1) / BIN_ROWS;
     if (nb > MAX_BINS_PER_LEVEL) return false;
     bp->nbins[l] = (int)nb;
