@@ -20,13 +20,16 @@ namespace nf {
 // activation + rounding of a hidden layer; the packed tiles become the next layer's B fragments
 template <typename T, int KC_H, bool RELU>
 __device__ __forceinline__ void hidden_epilogue(const f32x4_t (&acc)[2][4], Frag (&in)[2][2], int act) {
+  with_act(RELU ? NF_ACT_RELU : act, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt)
+    for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-    for (int kc = 0; kc < KC_H; ++kc) {
-      act_pack<T, RELU>(acc[nt][2 * kc], act, in[nt][kc].w[0], in[nt][kc].w[1]);
-      act_pack<T, RELU>(acc[nt][2 * kc + 1], act, in[nt][kc].w[2], in[nt][kc].w[3]);
-    }
+      for (int kc = 0; kc < KC_H; ++kc) {
+        act_pack<T, RELU>(acc[nt][2 * kc], ACT, in[nt][kc].w[0], in[nt][kc].w[1]);
+        act_pack<T, RELU>(acc[nt][2 * kc + 1], ACT, in[nt][kc].w[2], in[nt][kc].w[3]);
+      }
+  });
 }
 
 // ---------------------------------------------------------------------------------------
@@ -111,19 +114,22 @@ __global__ __launch_bounds__(256) void mlp_fwd_k(MlpArgs a) {
 template <typename T, int MT_H, bool RELU>
 __device__ __forceinline__ void recompute_epilogue(const f32x4_t (&acc)[2][4], Frag (&in)[2][2], uint16_t* panel, uint32_t* im,
                                                    int act, int lane) {
+  with_act(RELU ? NF_ACT_RELU : act, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt)
+    for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-    for (int mt = 0; mt < MT_H; ++mt) {
-      uint32_t h01, h23, g01, g23;
-      act_pack<T, RELU>(acc[nt][mt], act, h01, h23);
-      gate_pack<T, RELU>(acc[nt][mt], act, h01, h23, g01, g23);
-      in[nt][mt >> 1].w[2 * (mt & 1)] = h01;
-      in[nt][mt >> 1].w[2 * (mt & 1) + 1] = h23;
-      park_tile_T(panel, mt, nt, lane, h01, h23);
-      im[((mt * 2 + nt) * 2 + 0) * 64 + lane] = g01;
-      im[((mt * 2 + nt) * 2 + 1) * 64 + lane] = g23;
-    }
+      for (int mt = 0; mt < MT_H; ++mt) {
+        uint32_t h01, h23, g01, g23;
+        act_pack<T, RELU>(acc[nt][mt], ACT, h01, h23);
+        gate_pack<T, RELU>(acc[nt][mt], ACT, h01, h23, g01, g23);
+        in[nt][mt >> 1].w[2 * (mt & 1)] = h01;
+        in[nt][mt >> 1].w[2 * (mt & 1) + 1] = h23;
+        park_tile_T(panel, mt, nt, lane, h01, h23);
+        im[((mt * 2 + nt) * 2 + 0) * 64 + lane] = g01;
+        im[((mt * 2 + nt) * 2 + 1) * 64 + lane] = g23;
+      }
+  });
 }
 
 template <typename T, int KIN, int HP, int OUTP, int REG_HIDDEN>

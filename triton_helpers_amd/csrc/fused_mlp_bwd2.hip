@@ -226,43 +226,57 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
 
     // ---- forward recompute: h1 = act(W_in x + b), h2 = act(W_hid h1 + b) ----
     layer_nt<T, NT, MT_H, KC_IN>(acc, in, f_in, bias_in, lane);
+    if (RELU) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
+      for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-      for (int mt = 0; mt < MT_H; ++mt) {
-        uint32_t p01, p23;
-        if (RELU) {
-          p01 = relu_pk(pack2<T>(acc[nt][mt][0], acc[nt][mt][1]));
-          p23 = relu_pk(pack2<T>(acc[nt][mt][2], acc[nt][mt][3]));
-        } else {
-          uint32_t q01, q23;
-          act_pack<T, false>(acc[nt][mt], a.act, p01, p23);
-          gate_pack<T, false>(acc[nt][mt], a.act, p01, p23, q01, q23);
-          g1[nt][mt >> 1].w[2 * (mt & 1)] = q01;
-          g1[nt][mt >> 1].w[2 * (mt & 1) + 1] = q23;
+        for (int mt = 0; mt < MT_H; ++mt) {
+          h1[nt][mt >> 1].w[2 * (mt & 1)] = relu_pk(pack2<T>(acc[nt][mt][0], acc[nt][mt][1]));
+          h1[nt][mt >> 1].w[2 * (mt & 1) + 1] = relu_pk(pack2<T>(acc[nt][mt][2], acc[nt][mt][3]));
         }
-        h1[nt][mt >> 1].w[2 * (mt & 1)] = p01;
-        h1[nt][mt >> 1].w[2 * (mt & 1) + 1] = p23;
-      }
+    } else {
+      with_act(a.act, [&](auto act_c) {
+        constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+          for (int mt = 0; mt < MT_H; ++mt) {
+            uint32_t p01, p23, q01, q23;
+            act_pack<T, false>(acc[nt][mt], ACT, p01, p23);
+            gate_pack<T, false>(acc[nt][mt], ACT, p01, p23, q01, q23);
+            g1[nt][mt >> 1].w[2 * (mt & 1)] = q01;
+            g1[nt][mt >> 1].w[2 * (mt & 1) + 1] = q23;
+            h1[nt][mt >> 1].w[2 * (mt & 1)] = p01;
+            h1[nt][mt >> 1].w[2 * (mt & 1) + 1] = p23;
+          }
+      });
+    }
     layer_nt<T, NT, MT_H, KC_H>(acc, h1, f_hid, bias_hid, lane);
+    if (RELU) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
+      for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-      for (int mt = 0; mt < MT_H; ++mt) {
-        uint32_t p01, p23;
-        if (RELU) {
-          p01 = relu_pk(pack2<T>(acc[nt][mt][0], acc[nt][mt][1]));
-          p23 = relu_pk(pack2<T>(acc[nt][mt][2], acc[nt][mt][3]));
-        } else {
-          uint32_t q01, q23;
-          act_pack<T, false>(acc[nt][mt], a.act, p01, p23);
-          gate_pack<T, false>(acc[nt][mt], a.act, p01, p23, q01, q23);
-          g2[nt][mt >> 1].w[2 * (mt & 1)] = q01;
-          g2[nt][mt >> 1].w[2 * (mt & 1) + 1] = q23;
+        for (int mt = 0; mt < MT_H; ++mt) {
+          h2[nt][mt >> 1].w[2 * (mt & 1)] = relu_pk(pack2<T>(acc[nt][mt][0], acc[nt][mt][1]));
+          h2[nt][mt >> 1].w[2 * (mt & 1) + 1] = relu_pk(pack2<T>(acc[nt][mt][2], acc[nt][mt][3]));
         }
-        h2[nt][mt >> 1].w[2 * (mt & 1)] = p01;
-        h2[nt][mt >> 1].w[2 * (mt & 1) + 1] = p23;
-      }
+    } else {
+      with_act(a.act, [&](auto act_c) {
+        constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+          for (int mt = 0; mt < MT_H; ++mt) {
+            uint32_t p01, p23, q01, q23;
+            act_pack<T, false>(acc[nt][mt], ACT, p01, p23);
+            gate_pack<T, false>(acc[nt][mt], ACT, p01, p23, q01, q23);
+            g2[nt][mt >> 1].w[2 * (mt & 1)] = q01;
+            g2[nt][mt >> 1].w[2 * (mt & 1) + 1] = q23;
+            h2[nt][mt >> 1].w[2 * (mt & 1)] = p01;
+            h2[nt][mt >> 1].w[2 * (mt & 1) + 1] = p23;
+          }
+      });
+    }
 
     // ---- output layer: dW_out += dy^T h2, db_out += sum dy ; dh2 = W_out^T dy ----
 #pragma unroll

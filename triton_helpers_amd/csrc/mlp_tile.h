@@ -18,6 +18,7 @@
 // 16 bytes, lane (m, g) holding W[16*mt + m][k(kc, g, 0..7)].
 #pragma once
 
+#include <type_traits>
 #include "nf_common.h"
 
 namespace nf {
@@ -134,7 +135,22 @@ __device__ __forceinline__ float act_grad(float z, int act) {
   }
 }
 
-// h = act(z) packed to 16 bit.  RELU = true is the branch-free fast path; otherwise `act` selects at run time.
+// Runs body(std::integral_constant<int, ACT>) under one wave-uniform branch on `act`, so that everything inside
+// sees the activation as a compile-time constant.  A switch evaluated per element gets flattened into
+// "compute every activation, then select", which doubles the cost of a layer epilogue.
+template <typename Body>
+__device__ __forceinline__ void with_act(int act, Body&& body) {
+  switch (act) {
+    case NF_ACT_RELU: body(std::integral_constant<int, NF_ACT_RELU>{}); break;
+    case NF_ACT_SILU: body(std::integral_constant<int, NF_ACT_SILU>{}); break;
+    case NF_ACT_RELU2: body(std::integral_constant<int, NF_ACT_RELU2>{}); break;
+    case NF_ACT_GELU: body(std::integral_constant<int, NF_ACT_GELU>{}); break;
+    default: body(std::integral_constant<int, NF_ACT_NONE>{}); break;
+  }
+}
+
+// h = act(z) packed to 16 bit.  RELU = true is the branch-free fast path; otherwise `act` selects (pass a constant,
+// see with_act, wherever the call sits in a loop).
 template <typename T, bool RELU>
 __device__ __forceinline__ void act_pack(const f32x4_t z, int act, uint32_t& p01, uint32_t& p23) {
   if (RELU) {

@@ -191,15 +191,18 @@ __global__ __launch_bounds__(768) void rev_fwd_k(RevArgs a) {
           for (int mt = 0; mt < MT; ++mt) p[nt][mt] = pack4<T>(src[nt][mt]);
         tiles_to_frags<MT>(p, u);
         rev_layer<T, MT, KC>(acc, u, fw1, bb1, lane);
+        with_act(act, [&](auto act_c) {
+          constexpr int A = decltype(act_c)::value;
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
+          for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            f32x4_t z = acc[nt][mt];
+            for (int mt = 0; mt < MT; ++mt) {
+              f32x4_t z = acc[nt][mt];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) z[r] = act_fwd(z[r], act);
-            p[nt][mt] = pack4<T>(z);
-          }
+              for (int r = 0; r < 4; ++r) z[r] = act_fwd(z[r], A);
+              p[nt][mt] = pack4<T>(z);
+            }
+        });
         tiles_to_frags<MT>(p, t);
         rev_layer<T, MT, KC>(acc, t, fw1 + LAYER, bb1 + HP, lane);
 #pragma unroll
@@ -223,7 +226,7 @@ __global__ __launch_bounds__(768) void rev_fwd_k(RevArgs a) {
 // ---------------------------------------------------------------------------------------
 // Activation and its derivative from one pre-activation (GELU shares the exponential between the two).
 template <int ACT>
-__device__ __forceinline__ void act_both(float z, int act, float& h, float& g) {
+__device__ __forceinline__ void act_both(float z, float& h, float& g) {
   if (ACT == NF_ACT_GELU) {
     float pdf;
     const float cdf = normal_cdf_pdf(z, &pdf);
@@ -233,8 +236,8 @@ __device__ __forceinline__ void act_both(float z, int act, float& h, float& g) {
     h = fmaxf(z, 0.0f);
     g = z > 0.0f ? 1.0f : 0.0f;
   } else {
-    h = act_fwd(z, act);
-    g = act_grad(z, act);
+    h = act_fwd(z, ACT);
+    g = act_grad(z, ACT);
   }
 }
 
@@ -257,21 +260,24 @@ __device__ __forceinline__ void sub_backward(const uint2 (&u)[2][4], const uint2
   tiles_to_frags<MT>(d, df);
   // recompute hidden activation t = act(W1 u + b1) and act'(z)
   rev_layer<T, MT, KC>(acc, uf, fw1, b1, lane);
+  with_act(act, [&](auto act_c) {
+    constexpr int A = decltype(act_c)::value;
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt)
+    for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      f32x4_t h, g;
+      for (int mt = 0; mt < MT; ++mt) {
+        f32x4_t h, g;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float hv, gv;
-        act_both<ACT>(acc[nt][mt][r], act, hv, gv);
-        h[r] = hv;
-        g[r] = gv;
+        for (int r = 0; r < 4; ++r) {
+          float hv, gv;
+          act_both<A>(acc[nt][mt][r], hv, gv);
+          h[r] = hv;
+          g[r] = gv;
+        }
+        tp[nt][mt] = pack4<T>(h);
+        gp[nt][mt] = pack4<T>(g);
       }
-      tp[nt][mt] = pack4<T>(h);
-      gp[nt][mt] = pack4<T>(g);
-    }
+  });
   tiles_to_frags<MT>(tp, tf);
   // S(u) = W2 t + b2
   rev_layer<T, MT, KC>(sout, tf, fw2, b2, lane);
