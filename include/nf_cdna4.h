@@ -112,7 +112,16 @@ int nf_hash_encode_indices(const void* coords, int coords_dtype, int64_t coords_
  * may each be NULL.  depth >= 1 counts the input layer plus the hidden layers. */
 int nf_mlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_stride, const void* w_in, const void* b_in,
                const void* w_hid, const void* b_hid, const void* w_out, const void* b_out, int64_t rows, int d_in,
-               int d_hidden, int d_out, int depth, int act, int dtype, int x_dtype, void* stream);
+               int d_hidden, int d_out, int depth, int act, int dtype, int x_dtype, void* workspace,
+               int64_t workspace_bytes, void* stream);
+
+/* Networks deeper than one launch holds on chip (forward: about 18 layers at d_hidden = 64; backward: 4 hidden-to-
+ * hidden layers with ReLU, 2 with other activations at d_hidden = 64, 8 at d_hidden <= 32) run as a chain of
+ * launches that hand 16-bit pre-activations [rows, d_hidden] to each other through `workspace` (16-byte aligned
+ * device memory of at least this many bytes; contents are scratch).  0: one launch, workspace may be NULL.  (The
+ * reference loops over the layers inside one kernel, triton_helpers/layers/fully_fused_mlp/kernel.py:139-178,
+ * 264-304, re-reading every weight per program.) */
+int64_t nf_mlp_workspace_bytes(int64_t rows, int d_hidden, int depth, int act, int backward);
 
 /* x_dtype may be the other 16-bit type than `dtype` (an fp16 encoder output feeding bf16 weights): the rows are
  * converted while they are loaded, as a cast kernel in front would, and the backward writes dx in x_dtype.
@@ -125,7 +134,7 @@ int nf_mlp_bwd(const void* x, int64_t x_stride, const void* dy, int64_t dy_strid
                const void* w_in, const void* b_in, const void* w_hid, const void* b_hid, const void* w_out,
                const void* b_out, float* dw_in, float* db_in, float* dw_hid, float* db_hid, float* dw_out,
                float* db_out, int64_t rows, int d_in, int d_hidden, int d_out, int depth, int act, int dtype,
-               int x_dtype, void* stream);
+               int x_dtype, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Reversible MLP of `blocks` additive couplings over rows of width 2*half:
  *   y1 = x1 + F_k(x2),  y2 = x2 + G_k(y1),  F/G(u) = act(u W1^T + b1) W2^T + b2.

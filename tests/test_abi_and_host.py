@@ -48,16 +48,43 @@ def test_argument_validation_without_gpu():
     geom.dims = 7
     rc = lib.nf_hash_encode_fwd(None, 0, 3, 1, None, 0, None, 32, 10, geom, None, 1.0, 0, None)
     assert rc == -1 and b"dims" in lib.nf_last_error()
-    rc = lib.nf_mlp_fwd(None, 32, None, 16, None, None, None, None, None, None, 8, 32, 24, 16, 2, 1, _lib.NF_BF16, _lib.NF_BF16, None)
+    rc = lib.nf_mlp_fwd(None, 32, None, 16, None, None, None, None, None, None, 8, 32, 24, 16, 2, 1, _lib.NF_BF16, _lib.NF_BF16, None, 0, None)
     assert rc == -1 and b"d_hidden" in lib.nf_last_error()
-    rc = lib.nf_mlp_fwd(None, 32, None, 16, None, None, None, None, None, None, 8, 32, 64, 16, 2, 1, _lib.NF_F32, _lib.NF_BF16, None)
+    rc = lib.nf_mlp_fwd(None, 32, None, 16, None, None, None, None, None, None, 8, 32, 64, 16, 2, 1, _lib.NF_F32, _lib.NF_BF16, None, 0, None)
     assert rc == -2
     rc = lib.nf_revmlp_fwd(None, 128, None, 128, None, None, None, None, 8, 65, 4, 4, _lib.NF_BF16, None)
     assert rc == -1
     with pytest.raises(RuntimeError):
         _lib.check(rc, "nf_revmlp_fwd")
     # zero rows is a no-op that needs no device
-    assert lib.nf_mlp_fwd(None, 32, None, 16, None, None, None, None, None, None, 0, 32, 64, 16, 2, 1, _lib.NF_BF16, _lib.NF_BF16, None) == 0
+    assert lib.nf_mlp_fwd(None, 32, None, 16, None, None, None, None, None, None, 0, 32, 64, 16, 2, 1, _lib.NF_BF16, _lib.NF_BF16, None, 0, None) == 0
+
+
+def test_mlp_workspace_sizes_without_gpu():
+    """One launch needs no workspace; a chain of n launches keeps two hand-over buffers in the forward and
+    n - 1 of them plus two gradient buffers in the backward, each rows * d_hidden 16-bit values (256-byte rounded)."""
+    from triton_helpers_amd import _lib
+
+    if not _lib.LIB_PATH.exists():
+        pytest.skip("libnf_cdna4.so not built")
+    lib = _lib.load()
+    relu, silu = _lib.NF_ACT["relu"], _lib.NF_ACT["silu"]
+    rows = 1000
+    buf = (rows * 64 * 2 + 255) // 256 * 256
+    for depth in (1, 2, 4):
+        assert lib.nf_mlp_workspace_bytes(rows, 64, depth, relu, 0) == 0
+        assert lib.nf_mlp_workspace_bytes(rows, 64, depth, relu, 1) == 0
+    assert lib.nf_mlp_workspace_bytes(rows, 64, 2, silu, 1) == 0
+    assert lib.nf_mlp_workspace_bytes(rows, 64, 8, relu, 0) == 0           # 9 layers of weights fit LDS
+    assert lib.nf_mlp_workspace_bytes(rows, 64, 8, relu, 1) == (1 + 2) * buf  # 9 linear layers = 5 + 4
+    assert lib.nf_mlp_workspace_bytes(rows, 64, 5, silu, 1) == (1 + 2) * buf  # 6 linear layers = 3 + 3
+    assert lib.nf_mlp_workspace_bytes(rows, 64, 32, relu, 0) == 2 * buf
+    assert lib.nf_mlp_workspace_bytes(rows, 32, 8, relu, 1) == 0
+    assert lib.nf_mlp_workspace_bytes(0, 64, 32, relu, 1) == 0
+    # a deep call without the workspace is refused before anything is launched
+    rc = lib.nf_mlp_bwd(1, 32, 1, 16, None, 32, 1, None, 1, None, 1, None, 1, None, 1, None, 1, None,
+                        rows, 32, 64, 16, 8, relu, _lib.NF_BF16, _lib.NF_BF16, None, 0, None)
+    assert rc == -1 and b"workspace" in lib.nf_last_error()
 
 
 @pytest.mark.parametrize("name", ["bench", "default"])

@@ -27,11 +27,11 @@ def _mk():
     return kernel
 
 
-def _params(d_in, d_hidden, d_out, depth, bias, dtype, seed=0):
+def _params(d_in, d_hidden, d_out, depth, bias, dtype, seed=0, gain=1.0):
     g = torch.Generator().manual_seed(seed)
 
     def u(shape, fan_in):
-        return ((torch.rand(*shape, generator=g) * 2 - 1) / fan_in**0.5).to(dtype)
+        return ((torch.rand(*shape, generator=g) * 2 - 1) * gain / fan_in**0.5).to(dtype)
 
     p = dict(w_in=u((d_hidden, d_in), d_in), w_out=u((d_out, d_hidden), d_hidden))
     p["b_in"] = u((d_hidden,), d_in) if bias else None
@@ -79,6 +79,12 @@ SHAPES = [
     ((1, 1000), 32, 64, 16, 3),
     ((3, 100), 64, 64, 64, 3),
     ((2, 77), 40, 64, 20, 3),
+    # deeper than one launch covers: a chain of launches handing pre-activations over through the workspace
+    ((1, 300), 32, 64, 16, 5),
+    ((2, 100), 64, 64, 64, 8),
+    ((1, 203), 32, 64, 3, 12),
+    ((1, 100), 8, 32, 4, 12),
+    ((1, 64), 32, 64, 16, 32),   # the forward, too, splits (the weights of 33 layers do not fit LDS)
 ]
 
 
@@ -108,6 +114,50 @@ def test_forward_backward(shape, d_in, d_hidden, d_out, depth, bias, act, dtype)
         if leaves[k] is None:
             continue
         _close(leaves[k].grad, want["d" + k], "d" + k, scale_rel=True, depth=depth)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize(
+    "act,gain,d_in,d_hidden,d_out,depth",
+    [
+        ("relu", 6**0.5, 32, 64, 16, 5),
+        ("relu", 6**0.5, 32, 64, 16, 9),
+        ("relu", 6**0.5, 64, 64, 3, 12),
+        ("relu", 6**0.5, 16, 32, 8, 11),
+        ("silu", 3.0, 32, 64, 16, 3),
+        ("silu", 3.0, 32, 64, 16, 6),
+        ("none", 3**0.5, 32, 64, 16, 7),
+    ],
+)
+def test_chained_launches_keep_signal(act, gain, d_in, d_hidden, d_out, depth, dtype):
+    """Deep nets with variance-preserving weights: activations and gradients stay O(1) through every launch
+    boundary, so a wrong hand-over (activation applied twice or not at all, a missing act'(x) on the gradient,
+    a weight slice off by one layer) shows at full size instead of drowning in a shrinking signal."""
+    mk = _mk()
+    rows = 777
+    torch.manual_seed(1)
+    p = _params(d_in, d_hidden, d_out, depth, True, dtype, seed=3, gain=gain)
+    x = torch.randn(1, rows, d_in).to(dtype)
+    dy = torch.randn(1, rows, d_out).to(dtype)
+    want_y = M.mlp_forward(x.float().view(-1, d_in), p["w_in"], p["b_in"], p["w_out"], p["b_out"], p["w_hid"], p["b_hid"], act, round_to=dtype)
+    want = M.mlp_backward(x.view(-1, d_in), dy.view(-1, d_out), p["w_in"], p["b_in"], p["w_out"], p["b_out"], p["w_hid"], p["b_hid"], act, round_to=dtype)
+    assert float(want_y.abs().mean()) > 0.05 and float(want["dx"].abs().mean()) > 0.05, "the signal must survive the depth"
+    leaves = {k: v.to(DEV).requires_grad_(True) for k, v in p.items()}
+    xd = x.to(DEV).requires_grad_(True)
+    y = mk.fully_fused_mlp(xd, leaves["w_in"], leaves["b_in"], leaves["w_out"], leaves["b_out"], leaves["w_hid"], leaves["b_hid"], act)
+    y.backward(dy.to(DEV))
+
+    def rel(got, ref):  # error relative to the tensor's scale: deep 16-bit chains accumulate rounding layer by layer
+        got, ref = got.detach().cpu().float(), ref.float()
+        return float((got - ref).abs().max() / ref.abs().max())
+
+    tol = RTOL * max(1.0, depth / 4)
+    assert rel(y.view(-1, d_out), want_y) <= tol
+    # ReLU: rows whose gate flips on a rounding difference move by a whole weight; compare the bulk
+    dxe = (xd.grad.view(-1, d_in).cpu().float() - want["dx"].float()).abs() / want["dx"].float().abs().max()
+    assert float((dxe > tol).float().mean()) <= (2e-3 if act == "relu" else 0.0), f"dx: max rel {float(dxe.max()):.3g}"
+    for k in ("w_in", "b_in", "w_out", "b_out", "w_hid", "b_hid"):
+        assert rel(leaves[k].grad, want["d" + k]) <= tol, k
 
 
 @pytest.mark.parametrize("act", ["relu", "silu", "none"])

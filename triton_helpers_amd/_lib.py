@@ -36,6 +36,7 @@ EXPORTS = (
     "nf_hash_encode_indices",
     "nf_mlp_fwd",
     "nf_mlp_bwd",
+    "nf_mlp_workspace_bytes",
     "nf_revmlp_fwd",
     "nf_revmlp_bwd",
 )
@@ -85,9 +86,11 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.nf_hash_encode_indices.restype = c_int
     lib.nf_hash_encode_indices.argtypes = [P, I, I64, I64, P, P, I64, POINTER(HashGeom), P, c_float, P]
     lib.nf_mlp_fwd.restype = c_int
-    lib.nf_mlp_fwd.argtypes = [P, I64, P, I64, P, P, P, P, P, P, I64, I, I, I, I, I, I, I, P]
+    lib.nf_mlp_fwd.argtypes = [P, I64, P, I64, P, P, P, P, P, P, I64, I, I, I, I, I, I, I, P, I64, P]
+    lib.nf_mlp_workspace_bytes.restype = I64
+    lib.nf_mlp_workspace_bytes.argtypes = [I64, I, I, I, I]
     lib.nf_mlp_bwd.restype = c_int
-    lib.nf_mlp_bwd.argtypes = [P, I64, P, I64, P, I64, P, P, P, P, P, P, P, P, P, P, P, P, I64, I, I, I, I, I, I, I, P]
+    lib.nf_mlp_bwd.argtypes = [P, I64, P, I64, P, I64, P, P, P, P, P, P, P, P, P, P, P, P, I64, I, I, I, I, I, I, I, P, I64, P]
     lib.nf_revmlp_fwd.restype = c_int
     lib.nf_revmlp_fwd.argtypes = [P, I64, P, I64, P, P, P, P, I64, I, I, I, I, P]
     lib.nf_revmlp_bwd.restype = c_int

@@ -20,6 +20,7 @@ struct MlpArgs {
   int d_in, d_hidden, d_out, depth, act;
   int x_vec, y_vec, dy_vec, dx_vec;
   int waves;  // waves per workgroup
+  int in_act; // activation applied to x as it is loaded (x holds pre-activations of a layer in front); dx = d/dx of that
   int x_conv; // 0: x / dx stored like the weights; 1: stored as float16 (weights bfloat16); 2: stored as bfloat16 (weights float16)
 };
 

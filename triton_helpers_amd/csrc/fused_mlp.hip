@@ -13,6 +13,8 @@
 // float32 registers over the wave's whole row loop (up to REG_HIDDEN hidden layers), are
 // reduced across the workgroup through LDS and leave with one coalesced atomic add per
 // 64-byte segment; deeper nets add the hidden-layer partials to memory chunk by chunk.
+#include <vector>
+
 #include "fused_mlp.h"
 
 namespace nf {
@@ -37,7 +39,7 @@ __device__ __forceinline__ void hidden_epilogue(const f32x4_t (&acc)[2][4], Frag
 // ---------------------------------------------------------------------------------------
 // XC: how x is stored (MlpArgs::x_conv), fixed at compile time.
 template <typename T, int KIN, int HP, int OUTP, int XC>
-__global__ __launch_bounds__(256) void mlp_fwd_k(MlpArgs a) {
+__global__ __launch_bounds__(512) void mlp_fwd_k(MlpArgs a) {
   constexpr int KC_IN = KIN / 32, KC_H = HP / 32, MT_H = HP / 16, MT_O = OUTP / 16;
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, nthreads = blockDim.x;
@@ -83,6 +85,7 @@ __global__ __launch_bounds__(256) void mlp_fwd_k(MlpArgs a) {
 #pragma unroll
       for (int kc = 0; kc < KC_IN; ++kc) {
         in[nt][kc] = XC == 0 ? nxt[nt][kc] : convert_frag(nxt[nt][kc], XC);
+        if (a.in_act != NF_ACT_NONE) in[nt][kc] = act_frag<T>(in[nt][kc], a.in_act);
         nxt[nt][kc] = load_rows_frag(a.x, a.x_stride, (chunk + wave_stride) * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
       }
 
@@ -228,6 +231,7 @@ __global__ __launch_bounds__(256) void mlp_bwd_k(MlpArgs a) {
 #pragma unroll
       for (int kc = 0; kc < KC_IN; ++kc) {
         in[nt][kc] = nx[nt][kc];
+        if (a.in_act != NF_ACT_NONE) in[nt][kc] = act_frag<T>(in[nt][kc], a.in_act);
         nx[nt][kc] = load_rows_frag(a.x, a.x_stride, (chunk + wave_stride) * 32 + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
         park_frag_T(xT, kc, nt, lane, in[nt][kc]);
       }
@@ -341,6 +345,13 @@ __global__ __launch_bounds__(256) void mlp_bwd_k(MlpArgs a) {
               const Frag wa = lds_frag(t_in, mt * KC_H + kc, lane);
               o0 = mfma16<T>(wa, dz[0][kc], o0);
               o1 = mfma16<T>(wa, dz[1][kc], o1);
+            }
+            if (a.in_act != NF_ACT_NONE) {
+              // the stored x of these positions (just read by this wave: a cache hit) gives act'(x)
+              const uint2 x0 = load_rows_tile(a.x, a.x_stride, row0, a.rows, a.d_in, mt, lane, a.x_vec != 0);
+              const uint2 x1 = load_rows_tile(a.x, a.x_stride, row0 + 16, a.rows, a.d_in, mt, lane, a.x_vec != 0);
+              o0 = input_gate<T>(o0, x0.x, x0.y, a.in_act);
+              o1 = input_gate<T>(o1, x1.x, x1.y, a.in_act);
             }
             store_rows_tile<T>(a.dx, a.dx_stride, row0, a.rows, a.d_in, mt, lane, o0, a.dx_vec);
             store_rows_tile<T>(a.dx, a.dx_stride, row0 + 16, a.rows, a.d_in, mt, lane, o1, a.dx_vec);
@@ -532,10 +543,11 @@ static int launch_fwd(const MlpArgs& a0, hipStream_t s) {
   const size_t lds = ((size_t)(HP / 16) * (KIN / 32) + (size_t)n_hid * (HP / 16) * (HP / 32) + (size_t)(OUTP / 16) * (HP / 32)) * 1024 +
                      ((size_t)HP + (size_t)n_hid * HP + OUTP) * 4;
   NF_REQUIRE(lds <= LDS_LIMIT, NF_EUNSUPPORTED, "weights of depth %d need %zu B of LDS (limit %zu)", a.depth, lds, LDS_LIMIT);
-  a.waves = 4;
+  // weights beyond half of LDS leave room for one workgroup per CU: give it eight waves to keep two per SIMD
+  a.waves = lds > 76 * 1024 ? 8 : 4;
   const int64_t chunks = (a.rows + 31) / 32;
   int64_t blocks = (chunks + a.waves - 1) / a.waves;
-  const int64_t cap = (int64_t)device_cus() * (lds > 64 * 1024 ? 1 : (lds > 40 * 1024 ? 2 : 3));
+  const int64_t cap = (int64_t)device_cus() * (lds > 76 * 1024 ? 1 : (lds > 40 * 1024 ? 2 : 3));
   if (blocks > cap) blocks = cap;
   constexpr int XC_OTHER = T::code == NF_BF16 ? 1 : 2;
   const void* kern = a.x_conv == 0 ? (const void*)mlp_fwd_k<T, KIN, HP, OUTP, 0> : (const void*)mlp_fwd_k<T, KIN, HP, OUTP, XC_OTHER>;
@@ -620,13 +632,116 @@ static int dispatch_bwd(const MlpArgs& a, hipStream_t s) {
   return a.depth - 1 <= 1 ? dispatch_bwd2<T, 1>(a, s) : dispatch_bwd2<T, 0>(a, s);
 }
 
+// ---------------------------------------------------------------------------------------
+// Networks deeper than one launch covers
+// ---------------------------------------------------------------------------------------
+// A launch keeps every weight of its layers in LDS and (backward) every activation of a chunk on chip, which bounds
+// the layers it can take.  Deeper networks run as a chain of launches over consecutive linear layers l0 .. l1-1
+// (0 = input layer, depth = output layer).  The value handed from one launch to the next is the PRE-activation of layer
+// l1-1, rounded to 16 bit: the launch behind applies the activation as it loads its rows (MlpArgs::in_act) and, in
+// the backward, multiplies its dx by act'(x), so every launch is an ordinary "input layer, hidden layers, linear
+// output layer" network and no elementwise pass runs in between.  The backward first replays the forward up to the
+// last boundary, keeping each boundary's rows (rows * d_hidden * 2 bytes), then walks the launches last to first.
+
+static int fwd_one(const MlpArgs& a, int dtype, hipStream_t s) {
+  return dtype == NF_BF16 ? dispatch_fwd<BF16>(a, s) : dispatch_fwd<F16>(a, s);
+}
+
+static int bwd_one(const MlpArgs& a, int dtype, hipStream_t s) {
+  bool handled = false;
+  const int rc = launch_mlp_bwd2(a, dtype, s, &handled);
+  if (rc != 0 || handled) return rc;
+  NF_REQUIRE(a.x_conv == 0, NF_EUNSUPPORTED, "x_dtype != dtype needs depth == 2 and d_hidden > 32 in the backward");
+  return dtype == NF_BF16 ? dispatch_bwd<BF16>(a, s) : dispatch_bwd<F16>(a, s);
+}
+
+// Most linear layers one forward launch holds in LDS (input and output layers priced at their widest).
+static int fwd_max_linear(int d_hidden) {
+  const int hp = d_hidden <= 32 ? 32 : 64;
+  auto fits = [&](int n_linear) {
+    const int n_hid = n_linear - 2;
+    const size_t lds = ((size_t)(hp / 16) * 2 + (size_t)n_hid * (hp / 16) * (hp / 32) + (size_t)4 * (hp / 32)) * 1024 +
+                       ((size_t)hp + (size_t)n_hid * hp + 64) * 4;
+    return lds <= LDS_LIMIT;
+  };
+  int m = 2;
+  while (fits(m + 1)) ++m;
+  return m;
+}
+
+// Most linear layers one backward launch takes: the register-resident kernels of the 64-wide nets reach five (ReLU)
+// or three; the general kernel takes nine at width 16 / 32.
+static int bwd_max_linear(int d_hidden, int act) {
+  if (d_hidden > 32) return act == NF_ACT_RELU ? 5 : 3;
+  return 9;
+}
+
+// Boundaries of the launches: n_linear layers in ceil(n_linear / max_per_launch) runs of near-equal length (each >= 2).
+static std::vector<int> plan_launches(int n_linear, int max_per_launch) {
+  const int n = (n_linear + max_per_launch - 1) / max_per_launch;
+  std::vector<int> first(n + 1, 0);
+  for (int k = 0; k <= n; ++k) first[k] = (int)((int64_t)n_linear * k / n);
+  return first;
+}
+
+static size_t boundary_bytes(int64_t rows, int d_hidden) { return ((size_t)rows * d_hidden * 2 + 255) / 256 * 256; }
+
+// Arguments of the launch over linear layers l0 .. l1-1 of network `a` (x / y / dy / dx are left to the caller).
+static MlpArgs launch_args(const MlpArgs& a, int l0, int l1) {
+  MlpArgs g = a;
+  const int H = a.d_hidden, last = a.depth;
+  const size_t hh = (size_t)H * H;
+  auto W = [&](int l) { return l == 0 ? a.w_in : l == last ? a.w_out : a.w_hid + (size_t)(l - 1) * hh; };
+  auto B = [&](int l) -> const uint16_t* {
+    return l == 0 ? a.b_in : l == last ? a.b_out : (a.b_hid ? a.b_hid + (size_t)(l - 1) * H : nullptr);
+  };
+  auto DW = [&](int l) -> float* {
+    if (a.dw_in == nullptr) return nullptr;  // forward
+    return l == 0 ? a.dw_in : l == last ? a.dw_out : a.dw_hid + (size_t)(l - 1) * hh;
+  };
+  auto DB = [&](int l) -> float* {
+    return l == 0 ? a.db_in : l == last ? a.db_out : (a.db_hid ? a.db_hid + (size_t)(l - 1) * H : nullptr);
+  };
+  const bool has_hid = l1 - l0 > 2;
+  g.w_in = W(l0); g.b_in = B(l0); g.dw_in = DW(l0); g.db_in = DB(l0);
+  g.w_out = W(l1 - 1); g.b_out = B(l1 - 1); g.dw_out = DW(l1 - 1); g.db_out = DB(l1 - 1);
+  g.w_hid = has_hid ? W(l0 + 1) : nullptr; g.b_hid = has_hid ? B(l0 + 1) : nullptr;
+  g.dw_hid = has_hid ? DW(l0 + 1) : nullptr; g.db_hid = has_hid ? DB(l0 + 1) : nullptr;
+  g.d_in = l0 == 0 ? a.d_in : H;
+  g.d_out = l1 - 1 == last ? a.d_out : H;
+  g.depth = l1 - l0 - 1;
+  g.in_act = l0 == 0 ? NF_ACT_NONE : a.act;
+  g.x_conv = l0 == 0 ? a.x_conv : 0;
+  return g;
+}
+
+static void set_rows(MlpArgs& g, const uint16_t* x, int64_t x_stride, uint16_t* y, int64_t y_stride, const uint16_t* dy,
+                     int64_t dy_stride, uint16_t* dx, int64_t dx_stride) {
+  g.x = x; g.x_stride = x_stride; g.y = y; g.y_stride = y_stride;
+  g.dy = dy; g.dy_stride = dy_stride; g.dx = dx; g.dx_stride = dx_stride;
+  g.x_vec = vec_load_ok(x, x_stride, g.d_in);
+  g.y_vec = y ? vec_store_ok(y, y_stride, g.d_out) : 0;
+  g.dy_vec = dy ? vec_load_ok(dy, dy_stride, g.d_out) : 0;
+  g.dx_vec = dx ? vec_store_ok(dx, dx_stride, g.d_in) : 0;
+}
+
 }  // namespace nf
 
 using namespace nf;
 
+extern "C" int64_t nf_mlp_workspace_bytes(int64_t rows, int d_hidden, int depth, int act, int backward) {
+  if (rows <= 0 || depth < 1 || d_hidden < 1) return 0;
+  const int n_linear = depth + 1;
+  const int n = (int)plan_launches(n_linear, backward ? bwd_max_linear(d_hidden, act) : fwd_max_linear(d_hidden)).size() - 1;
+  if (n <= 1) return 0;
+  // forward: two boundaries alive at a time; backward: every boundary plus two gradient buffers
+  return (int64_t)boundary_bytes(rows, d_hidden) * (backward ? (n - 1) + 2 : 2);
+}
+
 extern "C" int nf_mlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_stride, const void* w_in, const void* b_in,
                           const void* w_hid, const void* b_hid, const void* w_out, const void* b_out, int64_t rows,
-                          int d_in, int d_hidden, int d_out, int depth, int act, int dtype, int x_dtype, void* stream) {
+                          int d_in, int d_hidden, int d_out, int depth, int act, int dtype, int x_dtype, void* workspace,
+                          int64_t workspace_bytes, void* stream) {
   if (int rc = validate(rows, d_in, d_hidden, d_out, depth, act, dtype)) return rc;
   NF_REQUIRE(x_dtype == NF_F16 || x_dtype == NF_BF16, NF_EUNSUPPORTED, "x_dtype code %d: float16 or bfloat16", x_dtype);
   if (rows == 0) return 0;
@@ -634,22 +749,36 @@ extern "C" int nf_mlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_st
   NF_REQUIRE(depth == 1 || w_hid, NF_EINVAL, "w_hid is NULL but depth=%d", depth);
   NF_REQUIRE(x_stride >= d_in && y_stride >= d_out, NF_EINVAL, "row stride smaller than row width");
   MlpArgs a = {};
-  a.x = (const uint16_t*)x; a.x_stride = x_stride; a.y = (uint16_t*)y; a.y_stride = y_stride;
   a.w_in = (const uint16_t*)w_in; a.b_in = (const uint16_t*)b_in; a.w_hid = (const uint16_t*)w_hid;
   a.b_hid = (const uint16_t*)b_hid; a.w_out = (const uint16_t*)w_out; a.b_out = (const uint16_t*)b_out;
   a.rows = rows; a.d_in = d_in; a.d_hidden = d_hidden; a.d_out = d_out; a.depth = depth; a.act = act;
-  a.x_vec = vec_load_ok(x, x_stride, d_in);
-  a.y_vec = vec_store_ok(y, y_stride, d_out);
+  a.in_act = NF_ACT_NONE;
   a.x_conv = x_dtype == dtype ? 0 : (x_dtype == NF_F16 ? 1 : 2);
+  set_rows(a, (const uint16_t*)x, x_stride, (uint16_t*)y, y_stride, nullptr, 0, nullptr, 0);
   hipStream_t s = (hipStream_t)stream;
-  return dtype == NF_BF16 ? dispatch_fwd<BF16>(a, s) : dispatch_fwd<F16>(a, s);
+  const std::vector<int> first = plan_launches(depth + 1, fwd_max_linear(d_hidden));
+  const int n = (int)first.size() - 1;
+  if (n == 1) return fwd_one(a, dtype, s);
+  const size_t buf = boundary_bytes(rows, d_hidden);
+  NF_REQUIRE(workspace != nullptr && workspace_bytes >= (int64_t)(2 * buf), NF_EINVAL,
+             "forward of depth %d runs as %d launches and needs a workspace of %zu bytes (nf_mlp_workspace_bytes)", depth, n,
+             2 * buf);
+  NF_REQUIRE((uintptr_t)workspace % 16 == 0, NF_EINVAL, "workspace must be 16-byte aligned");
+  uint16_t* bound[2] = {(uint16_t*)workspace, (uint16_t*)((char*)workspace + buf)};
+  for (int k = 0; k < n; ++k) {
+    MlpArgs g = launch_args(a, first[k], first[k + 1]);
+    set_rows(g, k == 0 ? a.x : bound[(k - 1) & 1], k == 0 ? a.x_stride : d_hidden, k == n - 1 ? a.y : bound[k & 1],
+             k == n - 1 ? a.y_stride : d_hidden, nullptr, 0, nullptr, 0);
+    if (int rc = fwd_one(g, dtype, s)) return rc;
+  }
+  return 0;
 }
 
 extern "C" int nf_mlp_bwd(const void* x, int64_t x_stride, const void* dy, int64_t dy_stride, void* dx, int64_t dx_stride,
                           const void* w_in, const void* b_in, const void* w_hid, const void* b_hid, const void* w_out,
                           const void* b_out, float* dw_in, float* db_in, float* dw_hid, float* db_hid, float* dw_out,
                           float* db_out, int64_t rows, int d_in, int d_hidden, int d_out, int depth, int act, int dtype,
-                          int x_dtype, void* stream) {
+                          int x_dtype, void* workspace, int64_t workspace_bytes, void* stream) {
   if (int rc = validate(rows, d_in, d_hidden, d_out, depth, act, dtype)) return rc;
   NF_REQUIRE(x_dtype == NF_F16 || x_dtype == NF_BF16, NF_EUNSUPPORTED, "x_dtype code %d: float16 or bfloat16", x_dtype);
   if (rows == 0) return 0;
@@ -658,20 +787,38 @@ extern "C" int nf_mlp_bwd(const void* x, int64_t x_stride, const void* dy, int64
   NF_REQUIRE(x_stride >= d_in && dy_stride >= d_out && (dx == nullptr || dx_stride >= d_in), NF_EINVAL,
              "row stride smaller than row width");
   MlpArgs a = {};
-  a.x = (const uint16_t*)x; a.x_stride = x_stride; a.dy = (const uint16_t*)dy; a.dy_stride = dy_stride;
-  a.dx = (uint16_t*)dx; a.dx_stride = dx_stride;
   a.w_in = (const uint16_t*)w_in; a.b_in = (const uint16_t*)b_in; a.w_hid = (const uint16_t*)w_hid;
   a.b_hid = (const uint16_t*)b_hid; a.w_out = (const uint16_t*)w_out; a.b_out = (const uint16_t*)b_out;
   a.dw_in = dw_in; a.db_in = db_in; a.dw_hid = dw_hid; a.db_hid = db_hid; a.dw_out = dw_out; a.db_out = db_out;
   a.rows = rows; a.d_in = d_in; a.d_hidden = d_hidden; a.d_out = d_out; a.depth = depth; a.act = act;
-  a.x_vec = vec_load_ok(x, x_stride, d_in);
-  a.dy_vec = vec_load_ok(dy, dy_stride, d_out);
-  a.dx_vec = dx ? vec_store_ok(dx, dx_stride, d_in) : 0;
+  a.in_act = NF_ACT_NONE;
   a.x_conv = x_dtype == dtype ? 0 : (x_dtype == NF_F16 ? 1 : 2);
+  set_rows(a, (const uint16_t*)x, x_stride, nullptr, 0, (const uint16_t*)dy, dy_stride, (uint16_t*)dx, dx_stride);
   hipStream_t s = (hipStream_t)stream;
-  bool handled = false;
-  const int rc = launch_mlp_bwd2(a, dtype, s, &handled);
-  if (rc != 0 || handled) return rc;
-  NF_REQUIRE(a.x_conv == 0, NF_EUNSUPPORTED, "x_dtype != dtype needs depth == 2 and d_hidden > 32 in the backward");
-  return dtype == NF_BF16 ? dispatch_bwd<BF16>(a, s) : dispatch_bwd<F16>(a, s);
+  const std::vector<int> first = plan_launches(depth + 1, bwd_max_linear(d_hidden, act));
+  const int n = (int)first.size() - 1;
+  if (n == 1) return bwd_one(a, dtype, s);
+  const size_t buf = boundary_bytes(rows, d_hidden);
+  const size_t need = buf * (size_t)(n - 1 + 2);
+  NF_REQUIRE(workspace != nullptr && workspace_bytes >= (int64_t)need, NF_EINVAL,
+             "backward of depth %d runs as %d launches and needs a workspace of %zu bytes (nf_mlp_workspace_bytes)", depth, n,
+             need);
+  NF_REQUIRE((uintptr_t)workspace % 16 == 0, NF_EINVAL, "workspace must be 16-byte aligned");
+  auto bound = [&](int k) { return (uint16_t*)((char*)workspace + (size_t)k * buf); };       // output of launch k, k < n-1
+  auto grad = [&](int k) { return (uint16_t*)((char*)workspace + (size_t)(n - 1 + (k & 1)) * buf); };  // d/d(input of launch k)
+  // replay the forward up to the last boundary
+  for (int k = 0; k + 1 < n; ++k) {
+    MlpArgs g = launch_args(a, first[k], first[k + 1]);
+    g.dw_in = g.dw_hid = g.dw_out = nullptr;
+    set_rows(g, k == 0 ? a.x : bound(k - 1), k == 0 ? a.x_stride : d_hidden, bound(k), d_hidden, nullptr, 0, nullptr, 0);
+    if (int rc = fwd_one(g, dtype, s)) return rc;
+  }
+  for (int k = n - 1; k >= 0; --k) {
+    MlpArgs g = launch_args(a, first[k], first[k + 1]);
+    set_rows(g, k == 0 ? a.x : bound(k - 1), k == 0 ? a.x_stride : d_hidden, nullptr, 0, k == n - 1 ? a.dy : grad(k + 1),
+             k == n - 1 ? a.dy_stride : d_hidden, k == 0 ? a.dx : grad(k), k == 0 ? a.dx_stride : d_hidden);
+    if (int rc = bwd_one(g, dtype, s)) return rc;
+  }
+  return 0;
 }
+

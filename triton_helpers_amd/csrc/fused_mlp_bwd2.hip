@@ -145,7 +145,8 @@ __device__ __forceinline__ void layer_nt(f32x4_t (&acc)[NT][4], const Frag (&in)
 }
 
 // NT: 16-row tiles per chunk (2 or 4).  Four give the scheduler two independent 32-row groups to interleave.
-// XC: how x / dx are stored (MlpArgs::x_conv), fixed at compile time so that the usual case pays nothing for it.
+// XC: how x / dx are stored (MlpArgs::x_conv), fixed at compile time so that the usual case pays nothing for it;
+// XC == 3: stored like the weights, and the network's activation is applied to x as it is loaded (MlpArgs::in_act).
 template <typename T, int KIN, int HP, int OUTP, bool RELU, bool FAST, int NT, int XC>
 __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArgs a) {
   constexpr int KC_IN = KIN / 32, KC_H = HP / 32, MT_H = HP / 16, MT_I = KIN / 16, MT_O = OUTP / 16;
@@ -209,12 +210,21 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
   for (int64_t chunk = first_chunk; chunk < n_chunks; chunk += wave_stride) {
     const int64_t row0 = chunk * ROWS;
     Frag in[NT][2], h1[NT][2], h2[NT][2], g1[NT][2], g2[NT][2], dz[NT][2];
+    Frag xraw[(XC == 3 && !RELU) ? NT : 1][2];  // x as stored, for act'(x) at the end (ReLU reads it off act(x))
     f32x4_t acc[NT][4];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
       for (int kc = 0; kc < KC_IN; ++kc) {
-        in[nt][kc] = XC == 0 ? nx[nt][kc] : convert_frag(nx[nt][kc], XC);
+        if constexpr (XC == 3 && RELU) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) in[nt][kc].w[q] = relu_pk(nx[nt][kc].w[q]);
+        } else if constexpr (XC == 3) {
+          xraw[nt][kc] = nx[nt][kc];
+          in[nt][kc] = act_frag<T>(nx[nt][kc], a.act);
+        } else {
+          in[nt][kc] = XC == 0 ? nx[nt][kc] : convert_frag(nx[nt][kc], XC);
+        }
         nx[nt][kc] = load_chain<FAST>(a.x, a.x_stride, (chunk + wave_stride) * ROWS + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
       }
 #pragma unroll
@@ -359,6 +369,11 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
       for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int mt = 0; mt < MT_I; ++mt) {
+          // chain-order fragments hold x exactly where the packed dx tiles sit
+          if constexpr (XC == 3 && RELU)
+            acc[nt][mt] = input_gate<T>(acc[nt][mt], in[nt][mt >> 1].w[2 * (mt & 1)], in[nt][mt >> 1].w[2 * (mt & 1) + 1], NF_ACT_RELU);
+          else if constexpr (XC == 3)
+            acc[nt][mt] = input_gate<T>(acc[nt][mt], xraw[nt][mt >> 1].w[2 * (mt & 1)], xraw[nt][mt >> 1].w[2 * (mt & 1) + 1], a.act);
           if (XC == 1) store_dx<F16, FAST>(a, row0 + 16 * nt, mt, lane, acc[nt][mt]);
           else if (XC == 2) store_dx<BF16, FAST>(a, row0 + 16 * nt, mt, lane, acc[nt][mt]);
           else store_dx<T, FAST>(a, row0 + 16 * nt, mt, lane, acc[nt][mt]);
@@ -442,7 +457,8 @@ constexpr int bwdn_lds_layers(int kin, int outp, int nh) {
   return (kin == 32 && outp == 16) ? 0 : 1;
 }
 
-template <typename T, int KIN, int HP, int OUTP, int NH, bool FAST>
+// IA: ReLU is applied to x as it is loaded (MlpArgs::in_act) and dx is the gradient in front of that ReLU.
+template <typename T, int KIN, int HP, int OUTP, int NH, bool FAST, bool IA>
 __global__ __launch_bounds__(256) void mlp_bwdn_k(MlpArgs a) {
   constexpr int KC_IN = KIN / 32, KC_H = HP / 32, MT_H = HP / 16, MT_I = KIN / 16, MT_O = OUTP / 16;
   constexpr int KC_O = (OUTP + 31) / 32;
@@ -530,6 +546,10 @@ __global__ __launch_bounds__(256) void mlp_bwdn_k(MlpArgs a) {
 #pragma unroll
       for (int kc = 0; kc < KC_IN; ++kc) {
         in[nt][kc] = nx[nt][kc];
+        if (IA) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) in[nt][kc].w[q] = relu_pk(in[nt][kc].w[q]);
+        }
         nx[nt][kc] = load_chain<FAST>(a.x, a.x_stride, (chunk + wave_stride) * ROWS + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
       }
 #pragma unroll
@@ -635,7 +655,11 @@ __global__ __launch_bounds__(256) void mlp_bwdn_k(MlpArgs a) {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int mt = 0; mt < MT_I; ++mt) store_dx<T, FAST>(a, row0 + 16 * nt, mt, lane, acc[nt][mt]);
+        for (int mt = 0; mt < MT_I; ++mt) {
+          if (IA)  // x > 0 where relu(x), held in chain order exactly where the packed dx tile sits, is not zero
+            acc[nt][mt] = input_gate<T>(acc[nt][mt], in[nt][mt >> 1].w[2 * (mt & 1)], in[nt][mt >> 1].w[2 * (mt & 1) + 1], NF_ACT_RELU);
+          store_dx<T, FAST>(a, row0 + 16 * nt, mt, lane, acc[nt][mt]);
+        }
     }
   }
 
@@ -746,7 +770,15 @@ static int launchn(const MlpArgs& a0, hipStream_t s) {
   if (blocks > cap) blocks = cap;
   const bool fast = a.x_vec && a.dy_vec && a.d_in % 4 == 0 && a.d_out % 4 == 0 &&
                     (a.dx == nullptr || ((uintptr_t)a.dx % 8 == 0 && a.dx_stride % 4 == 0));
-  const void* kern = fast ? (const void*)mlp_bwdn_k<T, KIN, HP, OUTP, NH, true> : (const void*)mlp_bwdn_k<T, KIN, HP, OUTP, NH, false>;
+  const void* kern;
+  if constexpr (KIN == HP) {  // a layer in front has the hidden width
+    kern = a.in_act != NF_ACT_NONE
+               ? (fast ? (const void*)mlp_bwdn_k<T, KIN, HP, OUTP, NH, true, true> : (const void*)mlp_bwdn_k<T, KIN, HP, OUTP, NH, false, true>)
+               : (fast ? (const void*)mlp_bwdn_k<T, KIN, HP, OUTP, NH, true, false> : (const void*)mlp_bwdn_k<T, KIN, HP, OUTP, NH, false, false>);
+  } else {
+    NF_REQUIRE(a.in_act == NF_ACT_NONE, NF_EUNSUPPORTED, "input activation with d_in=%d", a.d_in);
+    kern = fast ? (const void*)mlp_bwdn_k<T, KIN, HP, OUTP, NH, true, false> : (const void*)mlp_bwdn_k<T, KIN, HP, OUTP, NH, false, false>;
+  }
   if (LDS > 64 * 1024) {
     const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
@@ -792,7 +824,17 @@ static int launch2(const MlpArgs& a0, hipStream_t s) {
   // x in the other 16-bit type: built for the aligned ReLU case only (the end-to-end encoder -> MLP step)
   constexpr int XC_OTHER = T::code == NF_BF16 ? 1 : 2;
   const void* kern;
-  if (a.x_conv != 0) {
+  if (a.in_act != NF_ACT_NONE) {
+    NF_REQUIRE(KIN == HP && a.x_conv == 0 && a.in_act == a.act, NF_EUNSUPPORTED, "input activation with d_in=%d", a.d_in);
+    if constexpr (KIN == HP) {
+      if (a.act == NF_ACT_RELU)
+        kern = fast ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, true, NT, 3> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, false, NT, 3>;
+      else
+        kern = fast ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false, true, 2, 3> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false, false, 2, 3>;
+    } else {
+      return fail(NF_EUNSUPPORTED, "input activation with d_in=%d", a.d_in);
+    }
+  } else if (a.x_conv != 0) {
     NF_REQUIRE(fast && a.act == NF_ACT_RELU && a.x_conv == XC_OTHER, NF_EUNSUPPORTED,
                "x_dtype != dtype: the backward covers ReLU with 8-byte aligned rows only");
     kern = (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, true, NT, XC_OTHER>;

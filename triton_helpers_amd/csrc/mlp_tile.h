@@ -173,6 +173,28 @@ __device__ __forceinline__ void gate_pack(const f32x4_t z, int act, uint32_t h01
     g23 = pack2<T>(act_grad(z[2], act), act_grad(z[3], act));
   }
 }
+// act() of the eight packed values of a fragment (a sub-network whose input is a pre-activation).
+template <typename T>
+__device__ __forceinline__ Frag act_frag(Frag f, int act) {
+  with_act(act, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) f.w[q] = pack2<T>(act_fwd(unpack_lo<T>(f.w[q]), ACT), act_fwd(unpack_hi<T>(f.w[q]), ACT));
+  });
+  return f;
+}
+// v * act'(x) for the four values of a tile, x packed in (x01, x23).  ReLU selects rather than multiplies.
+template <typename T>
+__device__ __forceinline__ f32x4_t input_gate(f32x4_t v, uint32_t x01, uint32_t x23, int act) {
+  const float x[4] = {unpack_lo<T>(x01), unpack_hi<T>(x01), unpack_lo<T>(x23), unpack_hi<T>(x23)};
+  with_act(act, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) v[r] = ACT == NF_ACT_RELU ? (x[r] > 0.0f ? v[r] : 0.0f) : v[r] * act_grad(x[r], ACT);
+  });
+  return v;
+}
+
 // dz = dh * act'(z) from the parked gate image, packed to 16 bit.
 template <typename T, bool RELU>
 __device__ __forceinline__ void gate_apply(const f32x4_t dh, uint32_t g01, uint32_t g23, uint32_t& p01, uint32_t& p23) {
@@ -282,6 +304,24 @@ __device__ __forceinline__ void store_rows_tile(uint16_t* base, int64_t stride, 
     for (int i = 0; i < 4; ++i)
       if (c0 + i < width) p[i] = T::from_f32(v[i]);
   }
+}
+
+// The four stored values store_rows_tile() would overwrite, packed; zero beyond `rows` / `width`.
+__device__ __forceinline__ uint2 load_rows_tile(const uint16_t* base, int64_t stride, int64_t row0, int64_t rows, int width,
+                                               int mt, int lane, bool vec_ok) {
+  const int64_t r = row0 + (lane & 15);
+  const int c0 = 16 * mt + 4 * (lane >> 4);
+  uint2 o = make_uint2(0u, 0u);
+  if (r >= rows || c0 >= width) return o;
+  const uint16_t* p = base + r * stride + c0;
+  if (vec_ok && c0 + 4 <= width) return *reinterpret_cast<const uint2*>(p);
+  uint16_t e[4] = {0, 0, 0, 0};
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (c0 + i < width) e[i] = p[i];
+  o.x = (uint32_t)e[0] | ((uint32_t)e[1] << 16);
+  o.y = (uint32_t)e[2] | ((uint32_t)e[3] << 16);
+  return o;
 }
 
 // ---- transposes and row sums for products that contract over the rows of a chunk -----------

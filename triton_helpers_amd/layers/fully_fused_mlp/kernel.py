@@ -118,6 +118,14 @@ def _c(t: Optional[Tensor]) -> Optional[Tensor]:
     return None if t is None else (t if t.is_contiguous() else t.contiguous())
 
 
+def _workspace(lib, rows2d: Tensor, d_hidden: int, depth: int, activation: str, backward: bool):
+    """Scratch for networks that run as several launches (none for the usual depths)."""
+    n = lib.nf_mlp_workspace_bytes(rows2d.shape[0], d_hidden, depth, _lib.NF_ACT[activation], int(backward))
+    if n == 0:
+        return None, 0
+    return torch.empty(n, dtype=torch.uint8, device=rows2d.device), n
+
+
 class _fully_fused_mlp(Function):
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.float16)
@@ -170,11 +178,12 @@ class _fully_fused_mlp(Function):
         o = x.new_empty((B, L, D_out), dtype=w_in.dtype)
         o2 = o.view(-1, D_out)
         lib = _lib.load()
+        ws, ws_bytes = _workspace(lib, x2, D_hidden, depth, activation, backward=False)
         rc = lib.nf_mlp_fwd(
             x2.data_ptr(), x2.stride(0), o2.data_ptr(), o2.stride(0),
             w_in.data_ptr(), _lib.ptr(b_in), _lib.ptr(w_hid), _lib.ptr(b_hid), w_out.data_ptr(), _lib.ptr(b_out),
             x2.shape[0], D_in, D_hidden, D_out, depth, _lib.NF_ACT[activation], _lib.dtype_code(w_in.dtype),
-            _lib.dtype_code(x.dtype), _lib.current_stream(x.device),
+            _lib.dtype_code(x.dtype), _lib.ptr(ws), ws_bytes, _lib.current_stream(x.device),
         )
         _lib.check(rc, "nf_mlp_fwd")
         return o.float() if wide else o
@@ -199,6 +208,7 @@ class _fully_fused_mlp(Function):
         grads = _lib.GradBuffers(w_in, b_in, w_out, b_out, w_hid, b_hid)
         p_dw_in, p_db_in, p_dw_out, p_db_out, p_dw_hid, p_db_hid = grads.pointers()
         lib = _lib.load()
+        ws, ws_bytes = _workspace(lib, do2, D_hidden, ctx.depth, ctx.activation, backward=True)
         while True:
             x2 = _rows2d(x, D_in)
             dx = x.new_empty(x.shape) if need_dx else None
@@ -208,7 +218,7 @@ class _fully_fused_mlp(Function):
                 w_in.data_ptr(), _lib.ptr(b_in), _lib.ptr(w_hid), _lib.ptr(b_hid), w_out.data_ptr(), _lib.ptr(b_out),
                 p_dw_in, p_db_in, p_dw_hid, p_db_hid, p_dw_out, p_db_out,
                 x2.shape[0], D_in, D_hidden, D_out, ctx.depth, _lib.NF_ACT[ctx.activation], _lib.dtype_code(w_in.dtype),
-                _lib.dtype_code(x.dtype), _lib.current_stream(x.device),
+                _lib.dtype_code(x.dtype), _lib.ptr(ws), ws_bytes, _lib.current_stream(x.device),
             )
             if rc == _lib.NF_EUNSUPPORTED and x.dtype != w_in.dtype:
                 x = x.to(w_in.dtype)  # a shape / alignment the converting backward does not cover: cast first
