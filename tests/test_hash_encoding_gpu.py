@@ -44,6 +44,8 @@ CASES = [
     (4099, 3, 2, 2**19, 16, 16, 7006, 1.0),
     (777, 3, 2, 5000, 8, 4, 300, 1.0),  # T not a power of two: exact 64-bit remainder
     (513, 3, 4, 2**12, 4, 8, 64, 1.0),
+    (1000, 3, 8, 2**14, 8, 16, 512, 1.0),     # rows of 4 / 8 features: 8- / 16-byte gathers in the staged forward
+    (2049, 3, 4, 2**16, 16, 16, 2048, 2.0),
     (300, 1, 2, 64, 4, 8, 512, 1.0),
     (300, 3, 1, 2**12, 8, 16, 256, 0.5),
 ]
@@ -230,6 +232,31 @@ def test_backward_binned_two_dimensions(N, T, L, lo, hi, do_dtype):
     hk._FLAGS = 2
     try:
         ref = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, 2, None, T, lo, hi, L)
+    finally:
+        hk._FLAGS = 0
+    scale = max(1.0, float(want.abs().max()))
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-3, atol=1e-4 * scale)
+    torch.testing.assert_close(got, ref, rtol=1e-3, atol=1e-4 * scale)
+
+
+@pytest.mark.parametrize("do_dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("N,D,F,T,L,lo,hi", [(40000, 3, 4, 2**14, 16, 16, 512), (35001, 3, 8, 2**16, 8, 16, 1024),
+                                            (40000, 2, 4, 5000, 4, 8, 256), (33000, 3, 6, 2**12, 4, 8, 64)])
+def test_backward_binned_wide_rows(N, D, F, T, L, lo, hi, do_dtype):
+    """Tables with 4, 6 or 8 features per row: the binned backward takes the features two at a time (one fill and
+    one accumulation per pair).  Against the oracle and the scattered-atomic kernel."""
+    hk = _hk()
+    torch.manual_seed(5)
+    x = torch.rand(N, D)
+    x[0] = 0.0
+    x[1] = 1.0
+    E = O.level_row_offsets(L, T, D, lo, hi)[-1]
+    do = torch.randn(N, L * F).to(do_dtype)
+    want = O.encode_backward(x, do, E, F, None, T, L, lo, hi)
+    got = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, F, None, T, lo, hi, L)
+    hk._FLAGS = 2
+    try:
+        ref = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, F, None, T, lo, hi, L)
     finally:
         hk._FLAGS = 0
     scale = max(1.0, float(want.abs().max()))

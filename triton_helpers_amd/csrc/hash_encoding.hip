@@ -152,7 +152,9 @@ __global__ __launch_bounds__(256) void hash_indices_k(const void* coords, int cd
 // as full 16-byte pieces of contiguous output rows; the backward stages the
 // incoming gradient rows the same way before scattering.
 // ---------------------------------------------------------------------------
-template <typename TT, int PPT>
+// FW: 32-bit words (feature pairs) per table row; a corner's FW words share a cache line, so the pairs after the
+// first cost no further line fetch.
+template <typename TT, int PPT, int FW>
 __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_tiled_k(const void* coords, int cdt, int64_t csn, int64_t csd,
                                                                  const uint32_t* table, uint16_t* out,
                                                                  int64_t out_stride, int64_t N, DevGeom g,
@@ -182,8 +184,8 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_tiled_k(const void* coo
     const float fres = (float)g.res[l];
     const bool hashed = l >= g.first_hash;
     const uint32_t mask = g.rows[l] - 1;
-    const uint32_t* tab = table + g.row_offset[l];
-    uint32_t v[PPT][8];
+    const uint32_t* tab = table + g.row_offset[l] * FW;
+    uint32_t v[PPT][8][FW];
     float w[PPT][8];
 #pragma unroll
     for (int i = 0; i < PPT; ++i) {
@@ -198,25 +200,44 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_tiled_k(const void* coo
       }
       const Corner8 r = rows_d3(c, hashed, res, mask, pi);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) v[i][j] = tab[r.row[j]];
+      for (int j = 0; j < 8; ++j) {
+        if (FW == 1) {
+          v[i][j][0] = tab[r.row[j]];
+        } else if (FW == 2) {
+          const uint2 q = *reinterpret_cast<const uint2*>(tab + (size_t)r.row[j] * 2);
+          v[i][j][0] = q.x;
+          v[i][j][FW > 1 ? 1 : 0] = q.y;
+        } else if (FW == 4) {
+          const uint4 q = *reinterpret_cast<const uint4*>(tab + (size_t)r.row[j] * 4);
+          v[i][j][0] = q.x;
+          v[i][j][FW > 1 ? 1 : 0] = q.y;
+          v[i][j][FW > 2 ? 2 : 0] = q.z;
+          v[i][j][FW > 3 ? 3 : 0] = q.w;
+        } else {
+#pragma unroll
+          for (int f = 0; f < FW; ++f) v[i][j][f] = tab[(size_t)r.row[j] * FW + f];
+        }
+      }
       weights_d3(fr, w[i]);
     }
 #pragma unroll
-    for (int i = 0; i < PPT; ++i) {
-      float a0 = 0.0f, a1 = 0.0f;
+    for (int i = 0; i < PPT; ++i)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        a0 = a0 + w[i][j] * TT::to_f32((uint16_t)(v[i][j] & 0xffffu));
-        a1 = a1 + w[i][j] * TT::to_f32((uint16_t)(v[i][j] >> 16));
+      for (int f = 0; f < FW; ++f) {
+        float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          a0 = a0 + w[i][j] * TT::to_f32((uint16_t)(v[i][j][f] & 0xffffu));
+          a1 = a1 + w[i][j] * TT::to_f32((uint16_t)(v[i][j][f] >> 16));
+        }
+        stage[(l * FW + f) * LD + t + TILE_THREADS * i] = (uint32_t)TT::from_f32(a0) | ((uint32_t)TT::from_f32(a1) << 16);
       }
-      stage[l * LD + t + TILE_THREADS * i] = (uint32_t)TT::from_f32(a0) | ((uint32_t)TT::from_f32(a1) << 16);
-    }
   }
   __syncthreads();
 
-  // Each point's L*4 bytes leave as L/4 pieces of 16 bytes; consecutive lanes take
+  // Each point's L*FW*4 bytes leave as pieces of 16 bytes; consecutive lanes take
   // consecutive pieces, so a wave writes 1 KiB of contiguous output per instruction.
-  const int pieces = L >> 2;
+  const int pieces = (L * FW) >> 2;
   const int total = P * pieces;
   for (int c = t; c < total; c += TILE_THREADS) {
     const int p = c / pieces, q = c - p * pieces;
@@ -477,9 +498,9 @@ constexpr int64_t SCAN_MIN_POINTS = 32768;
 constexpr int SWEEP_PPT = 4;
 constexpr int64_t SWEEP_MIN_POINTS = (int64_t)256 * TILE_THREADS * SWEEP_PPT;
 
-static bool tiled_ok(const nf_hash_geom* g, int table_dt, const void* rows_ptr, int64_t row_stride) {
-  if (g->dims != 3 || g->feat != 2 || table_dt == NF_F32) return false;
-  if (g->levels % 4 != 0 || g->levels > 16) return false;
+static bool tiled_ok(const nf_hash_geom* g, int table_dt, const void* rows_ptr, int64_t row_stride, int feat = 2) {
+  if (g->dims != 3 || g->feat != feat || table_dt == NF_F32) return false;
+  if ((g->levels * (feat / 2)) % 4 != 0 || g->levels > 16) return false;
   for (int l = g->first_hash_level; l < g->levels; ++l) {
     if (l < 0) return false;
     const int64_t r = g->rows[l];
@@ -518,6 +539,28 @@ static int dispatch_fwd_generic(int table_dt, const void* coords, int cdt, int64
     default: launch_fwd_generic<D, BF16>(coords, cdt, csn, csd, table, out, out_stride, N, g, primes, scale, s); break;
   }
   return check_launch("hash_fwd_generic");
+}
+
+template <int FW>
+static int launch_fwd_tiled_wide(int table_dtype, const void* coords, int coords_dtype, int64_t csn, int64_t csd, const void* table,
+                                 void* out, int64_t out_stride_n, int64_t n_points, const DevGeom& g, const int64_t* primes,
+                                 float scale, hipStream_t s) {
+  constexpr int PPT = FW <= 2 ? 2 : 1;
+  constexpr int P = TILE_THREADS * PPT;
+  const size_t lds = (size_t)g.levels * FW * (P + 2) * sizeof(uint32_t);
+  dim3 grid((unsigned)((n_points + P - 1) / P));
+  const void* kern = table_dtype == NF_F16 ? (const void*)hash_fwd_tiled_k<F16, PPT, FW> : (const void*)hash_fwd_tiled_k<BF16, PPT, FW>;
+  if (lds > 64 * 1024) {
+    const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  }
+  const uint32_t* tab = (const uint32_t*)table;
+  uint16_t* o = (uint16_t*)out;
+  void* args[] = {(void*)&coords, (void*)&coords_dtype, (void*)&csn, (void*)&csd, (void*)&tab, (void*)&o,
+                  (void*)&out_stride_n, (void*)&n_points, (void*)&g, (void*)&primes, (void*)&scale};
+  const hipError_t e = hipLaunchKernel(kern, grid, dim3(TILE_THREADS), args, lds, s);
+  if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(hash_fwd_tiled): %s", hipGetErrorString(e));
+  return check_launch("hash_fwd_tiled");
 }
 
 }  // namespace nf
@@ -571,12 +614,18 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
     const size_t lds = (size_t)g.levels * (P + 2) * sizeof(uint32_t);
     dim3 grid((unsigned)((n_points + P - 1) / P));
     if (table_dtype == NF_F16)
-      hipLaunchKernelGGL((hash_fwd_tiled_k<F16, PPT>), grid, dim3(TILE_THREADS), lds, s, coords, coords_dtype, csn,
+      hipLaunchKernelGGL((hash_fwd_tiled_k<F16, PPT, 1>), grid, dim3(TILE_THREADS), lds, s, coords, coords_dtype, csn,
                          csd, (const uint32_t*)table, (uint16_t*)out, out_stride_n, n_points, g, primes, scale);
     else
-      hipLaunchKernelGGL((hash_fwd_tiled_k<BF16, PPT>), grid, dim3(TILE_THREADS), lds, s, coords, coords_dtype, csn,
+      hipLaunchKernelGGL((hash_fwd_tiled_k<BF16, PPT, 1>), grid, dim3(TILE_THREADS), lds, s, coords, coords_dtype, csn,
                          csd, (const uint32_t*)table, (uint16_t*)out, out_stride_n, n_points, g, primes, scale);
     return check_launch("hash_fwd_tiled");
+  }
+  // 16-bit rows of 4 or 8 features: the staged kernel with 8- or 16-byte gathers
+  if (!(flags & NF_HASH_FORCE_GENERIC) && (geom->feat == 4 || geom->feat == 8) && tiled_ok(geom, table_dtype, out, out_stride_n, geom->feat) &&
+      ((uintptr_t)table % (2 * geom->feat) == 0)) {
+    return geom->feat == 4 ? launch_fwd_tiled_wide<2>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s)
+                           : launch_fwd_tiled_wide<4>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
   }
   switch (g.dims) {
     case 1: return dispatch_fwd_generic<1>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);

@@ -1,4 +1,4 @@
-// Hash-encoding backward by binning (D = 3, F = 2, 16-bit upstream gradient).
+// Hash-encoding backward by binning (D = 2 or 3, an even number of features taken two at a time).
 //
 // Every (point, level, corner) contributes  w * dout[n, 2l .. 2l+1]  to one table row.  Scattering these with
 // global atomics is bound by the chip's atomic request rate; accumulating them in LDS needs the contributions to
@@ -341,7 +341,7 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
                                                                    const void* dout_v, int64_t dout_stride, int64_t N,
                                                                    DevGeom g, BinPlan bp, const int64_t* primes, float scale,
                                                                    const uint32_t* wg_counts, uint32_t* cursor, uint32_t* gmax,
-                                                                   uint32_t* records_v) {
+                                                                   uint32_t* records_v, int feat, int f0) {
   extern __shared__ __align__(16) unsigned char fill_smem[];
   const int NB = bp.binbase[bp.n_levels];
   const uint16_t* dout = reinterpret_cast<const uint16_t*>(dout_v);
@@ -371,9 +371,10 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
   const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], D > 2 ? (uint32_t)primes[D > 2 ? 2 : 0] : 0u};
   // this point's gradient row, read once (up to 16 levels live in registers); float32 rows are read level by level
   const uint32_t* grow = reinterpret_cast<const uint32_t*>(dout + (valid ? n : 0) * dout_stride);
-  const uint2* grow32 = reinterpret_cast<const uint2*>(reinterpret_cast<const float*>(dout_v) + (valid ? n : 0) * dout_stride);
+  const float* grow32 = reinterpret_cast<const float*>(dout_v) + (valid ? n : 0) * dout_stride;
   uint32_t gr[16];
-  const bool row_vec = !G32 && bp.n_levels <= 16 && (bp.n_levels & 3) == 0 && ((uintptr_t)dout & 15u) == 0 && (dout_stride & 7) == 0;
+  // this pass covers features f0, f0 + 1 of every level: the pair of level l sits at element l * feat + f0 of the row
+  const bool row_vec = !G32 && feat == 2 && bp.n_levels <= 16 && (bp.n_levels & 3) == 0 && ((uintptr_t)dout & 15u) == 0 && (dout_stride & 7) == 0;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     uint4 t = make_uint4(0u, 0u, 0u, 0u);
@@ -414,7 +415,7 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
     const uint32_t* ldelta = delta + bp.binbase[l];
     uint32_t packed = 0u;  // 16-bit: the pair; float32: the point's index in the workgroup (its pair goes to gtab)
     if (G32) {
-      const uint2 pair = valid ? grow32[l] : make_uint2(0u, 0u);
+      const uint2 pair = valid ? *reinterpret_cast<const uint2*>(grow32 + l * feat + f0) : make_uint2(0u, 0u);
       gtab[tid] = pair;
       packed = (uint32_t)tid;
       // largest |g| of the level: positive float patterns order like integers
@@ -427,7 +428,7 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
 #pragma unroll
         for (int i = 1; i < 16; ++i) packed = (l == i) ? gr[i] : packed;
       } else if (valid) {
-        packed = grow[l];
+        packed = grow[(l * feat + f0) >> 1];
       }
       // largest |g| of the level: positive 16-bit float patterns order like integers
       const uint32_t pk = packed & 0x7fff7fffu;
@@ -531,7 +532,7 @@ struct BinRec<F32> {
 template <typename GT>
 __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const typename BinRec<GT>::type* records, const uint4* tasks,
                                                                     const uint32_t* n_tasks, const uint32_t* gmax, float* dtable,
-                                                                    DevGeom g, BinPlan bp) {
+                                                                    DevGeom g, BinPlan bp, int feat, int f0) {
   typedef typename BinRec<GT>::type Rec;
   // Fixed-point sums, one plane of BIN_ROWS 64-bit cells per feature: the 64 lanes of an add go to random rows of one
   // feature, and with 8-byte cells those spread over all 64 banks (interleaved features would leave them half).
@@ -596,7 +597,7 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const typena
         if (f[k][j]) atomicAdd(acc_tile + (uint32_t)(j & 1) * BIN_ROWS + slot[k][j >> 1], (unsigned long long)(long long)f[k][j]);
   }
   lds_barrier();
-  float* dst = dtable + (g.row_offset[l] + (int64_t)row0) * 2;
+  float* dst = dtable + (g.row_offset[l] + (int64_t)row0) * feat + f0;  // features f0, f0 + 1 of the bin's rows
   const float qnan = __uint_as_float(0x7fc00000u);
   const uint32_t nvals = 2u * nrows;
   constexpr int U = 16;  // values per thread whose table reads are in flight together (a full bin in one pass)
@@ -609,14 +610,15 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const typena
       // |a| < 2^48 is exact in double and so is the division by 2^se: one rounding, to float, at the end
       x[u] = a == 0 ? 0.0f : (float)ldexp((double)a, -se);
       if (nonfinite && a != 0) x[u] = qnan;
-      old[u] = (x[u] != 0.0f && !task.w) ? dst[i] : 0.0f;
+      old[u] = (x[u] != 0.0f && !task.w) ? dst[(i >> 1) * feat + (i & 1u)] : 0.0f;
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t i = i0 + u * ACC_THREADS + tid;
       if (x[u] != 0.0f) {
-        if (task.w) unsafeAtomicAdd(dst + i, x[u]);
-        else dst[i] = old[u] + x[u];
+        float* cell = dst + (i >> 1) * feat + (i & 1u);
+        if (task.w) unsafeAtomicAdd(cell, x[u]);
+        else *cell = old[u] + x[u];
       }
     }
   }
@@ -626,7 +628,8 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const typena
 // Host side
 // ---------------------------------------------------------------------------------------
 static bool bin_plan(int64_t N, const nf_hash_geom* geom, int dout_dtype, BinPlan* bp, int64_t* records, uint32_t* max_tasks) {
-  if ((geom->dims != 3 && geom->dims != 2) || geom->feat != 2 || N <= 0) return false;
+  // features are taken two at a time (one pass of fill + accumulate per pair)
+  if ((geom->dims != 3 && geom->dims != 2) || geom->feat < 2 || geom->feat % 2 != 0 || N <= 0) return false;
   bp->n_levels = geom->levels;
   int nb_total = 0;
   for (int l = 0; l < geom->levels; ++l) {
@@ -702,6 +705,16 @@ int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const 
   hipLaunchKernelGGL(hash_bwd_bin_offsets_k, dim3(1), dim3(1024), 0, s, (const uint32_t*)ws.hist, ws.cursor, ws.n_tasks,
                      ws.tasks, NB, max_tasks);
   if (int rc = check_launch("hash_bwd_bin_offsets")) return rc;
+  const int feat = geom->feat;
+  for (int f0 = 0; f0 < feat; f0 += 2) {
+    if (f0 > 0) {
+      // the next pair of features: same bins and tasks; fresh level maxima and bin cursors
+      hipLaunchKernelGGL(hash_bwd_bin_zero_k, dim3(1), dim3(256), 0, s, ws.gmax, 32);
+      if (int rc = check_launch("hash_bwd_bin_zero")) return rc;
+      hipLaunchKernelGGL(hash_bwd_bin_offsets_k, dim3(1), dim3(1024), 0, s, (const uint32_t*)ws.hist, ws.cursor, ws.n_tasks,
+                         ws.tasks, NB, max_tasks);
+      if (int rc = check_launch("hash_bwd_bin_offsets")) return rc;
+    }
   {
     const size_t lds = (size_t)FILL_RECORDS * sizeof(uint4) + (g32 ? (size_t)FILL_POINTS * sizeof(uint2) : 0) +
                        ((size_t)2 * NB + 2 * NF_MAX_LEVELS) * 4;
@@ -711,7 +724,8 @@ int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const 
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     const uint32_t* wc = ws.wg_counts;
     void* args[] = {(void*)&coords, (void*)&cdt,   (void*)&csn,    (void*)&csd,   (void*)&dout, (void*)&dout_stride, (void*)&N, (void*)&g,
-                    (void*)&bp,     (void*)&primes, (void*)&scale, (void*)&wc,    (void*)&ws.cursor, (void*)&ws.gmax, (void*)&ws.records};
+                    (void*)&bp,     (void*)&primes, (void*)&scale, (void*)&wc,    (void*)&ws.cursor, (void*)&ws.gmax, (void*)&ws.records,
+                    (void*)&feat,   (void*)&f0};
     e = hipLaunchKernel(kern, dim3(blocks), dim3(FILL_POINTS), args, lds, s);
     if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(hash_bwd_bin_fill): %s", hipGetErrorString(e));
     if (int rc = check_launch("hash_bwd_bin_fill")) return rc;
@@ -727,11 +741,13 @@ int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const 
     const uint4* tk = ws.tasks;
     const uint32_t* nt = ws.n_tasks;
     const uint32_t* gm = ws.gmax;
-    void* args[] = {(void*)&rc_, (void*)&tk, (void*)&nt, (void*)&gm, (void*)&dtable, (void*)&g, (void*)&bp};
+    void* args[] = {(void*)&rc_, (void*)&tk, (void*)&nt, (void*)&gm, (void*)&dtable, (void*)&g, (void*)&bp, (void*)&feat, (void*)&f0};
     e = hipLaunchKernel(kern, dim3(max_tasks), dim3(ACC_THREADS), args, lds, s);
     if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(hash_bwd_bin_accum): %s", hipGetErrorString(e));
-    return check_launch("hash_bwd_bin_accum");
+    if (int rc = check_launch("hash_bwd_bin_accum")) return rc;
   }
+  }
+  return 0;
 }
 
 }  // namespace nf
