@@ -116,7 +116,7 @@ int nf_mlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_stride, const
                int64_t workspace_bytes, void* stream);
 
 /* Networks deeper than one launch holds on chip (forward: about 18 layers at d_hidden = 64; backward: 4 hidden-to-
- * hidden layers with ReLU, 2 with other activations at d_hidden = 64, 8 at d_hidden <= 32) run as a chain of
+ * hidden layers with ReLU at d_hidden = 64, 2 otherwise) run as a chain of
  * launches that hand 16-bit pre-activations [rows, d_hidden] to each other through `workspace` (16-byte aligned
  * device memory of at least this many bytes; contents are scratch).  0: one launch, workspace may be NULL.  (The
  * reference loops over the layers inside one kernel, triton_helpers/layers/fully_fused_mlp/kernel.py:139-178,

@@ -79,7 +79,8 @@ def test_mlp_workspace_sizes_without_gpu():
     assert lib.nf_mlp_workspace_bytes(rows, 64, 8, relu, 1) == (1 + 2) * buf  # 9 linear layers = 5 + 4
     assert lib.nf_mlp_workspace_bytes(rows, 64, 5, silu, 1) == (1 + 2) * buf  # 6 linear layers = 3 + 3
     assert lib.nf_mlp_workspace_bytes(rows, 64, 32, relu, 0) == 2 * buf
-    assert lib.nf_mlp_workspace_bytes(rows, 32, 8, relu, 1) == 0
+    assert lib.nf_mlp_workspace_bytes(rows, 32, 2, relu, 1) == 0
+    assert lib.nf_mlp_workspace_bytes(rows, 32, 8, relu, 1) == (2 + 2) * ((rows * 32 * 2 + 255) // 256 * 256)  # 9 linear layers = 3 + 3 + 3
     assert lib.nf_mlp_workspace_bytes(0, 64, 32, relu, 1) == 0
     # a deep call without the workspace is refused before anything is launched
     rc = lib.nf_mlp_bwd(1, 32, 1, 16, None, 32, 1, None, 1, None, 1, None, 1, None, 1, None, 1, None,

@@ -669,11 +669,12 @@ static int fwd_max_linear(int d_hidden) {
   return m;
 }
 
-// Most linear layers one backward launch takes: the register-resident kernels of the 64-wide nets reach five (ReLU)
-// or three; the general kernel takes nine at width 16 / 32.
+// Most linear layers one backward launch takes at full speed: the register-resident kernels of the 64-wide nets
+// reach five (ReLU) or three; at width 16 / 32 the general kernel keeps one hidden layer's dW in registers, and its
+// variant for more (partial dW through memory) costs several times a chain of those.
 static int bwd_max_linear(int d_hidden, int act) {
   if (d_hidden > 32) return act == NF_ACT_RELU ? 5 : 3;
-  return 9;
+  return 3;
 }
 
 // Boundaries of the launches: n_linear layers in ceil(n_linear / max_per_launch) runs of near-equal length (each >= 2).
