@@ -118,7 +118,8 @@ int nf_mlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_stride, const
 /* Networks deeper than one launch holds on chip (forward: about 18 layers at d_hidden = 64; backward: 4 hidden-to-
  * hidden layers with ReLU at d_hidden = 64, 2 otherwise) run as a chain of
  * launches that hand 16-bit pre-activations [rows, d_hidden] to each other through `workspace` (16-byte aligned
- * device memory of at least this many bytes; contents are scratch).  0: one launch, workspace may be NULL.  (The
+ * device memory of at least this many bytes; contents are scratch).  0: one launch, workspace may be NULL.  Without
+ * the workspace nf_mlp_bwd falls back to a slower one-launch kernel where the network fits it (NF_EINVAL otherwise).  (The
  * reference loops over the layers inside one kernel, triton_helpers/layers/fully_fused_mlp/kernel.py:139-178,
  * 264-304, re-reading every weight per program.) */
 int64_t nf_mlp_workspace_bytes(int64_t rows, int d_hidden, int depth, int act, int backward);

@@ -160,6 +160,49 @@ def test_chained_launches_keep_signal(act, gain, d_in, d_hidden, d_out, depth, d
         assert rel(leaves[k].grad, want["d" + k]) <= tol, k
 
 
+def test_backward_without_workspace_takes_the_one_launch_kernel():
+    """A C caller that passes no workspace still gets the gradients of a narrow deep net (slower kernel); a net that
+    fits no single launch is refused with the size it needs."""
+    from triton_helpers_amd import _lib
+
+    lib = _lib.load()
+    rows, d_in, H, d_out, depth = 500, 8, 32, 4, 4
+    dtype = torch.bfloat16
+    p = {k: _dev(v) for k, v in _params(d_in, H, d_out, depth, True, dtype, seed=7, gain=6**0.5).items()}
+    torch.manual_seed(2)
+    x = torch.randn(rows, d_in).to(dtype).to(DEV)
+    dy = torch.randn(rows, d_out).to(dtype).to(DEV)
+    relu = _lib.NF_ACT["relu"]
+    code = _lib.dtype_code(dtype)
+    stream = _lib.current_stream(x.device)
+
+    def run(ws):
+        dx = torch.empty_like(x)
+        g = {k: torch.zeros(v.shape, dtype=torch.float32, device=DEV) for k, v in p.items()}
+        rc = lib.nf_mlp_bwd(
+            x.data_ptr(), d_in, dy.data_ptr(), d_out, dx.data_ptr(), d_in,
+            p["w_in"].data_ptr(), p["b_in"].data_ptr(), p["w_hid"].data_ptr(), p["b_hid"].data_ptr(), p["w_out"].data_ptr(), p["b_out"].data_ptr(),
+            g["w_in"].data_ptr(), g["b_in"].data_ptr(), g["w_hid"].data_ptr(), g["b_hid"].data_ptr(), g["w_out"].data_ptr(), g["b_out"].data_ptr(),
+            rows, d_in, H, d_out, depth, relu, code, code, _lib.ptr(ws), 0 if ws is None else ws.numel(), stream)
+        _lib.check(rc, "nf_mlp_bwd")
+        torch.cuda.synchronize()
+        return dx, g
+
+    n = lib.nf_mlp_workspace_bytes(rows, H, depth, relu, 1)
+    assert n > 0
+    dx_a, g_a = run(torch.empty(n, dtype=torch.uint8, device=DEV))
+    dx_b, g_b = run(None)
+    for k in g_a:
+        scale = float(g_a[k].abs().max())
+        assert float((g_a[k] - g_b[k]).abs().max()) <= 2e-2 * scale, k
+    bad = ((dx_a.float() - dx_b.float()).abs() > 2e-2 * float(dx_a.float().abs().max())).float().mean().item()
+    assert bad <= 2e-3
+    # width 64, depth 8: no single launch holds it
+    rc = lib.nf_mlp_bwd(1, 32, 1, 16, None, 32, 1, None, 1, None, 1, None, 1, None, 1, None, 1, None,
+                        rows, 32, 64, 16, 8, relu, code, code, None, 0, stream)
+    assert rc == -1 and b"workspace" in lib.nf_last_error()
+
+
 @pytest.mark.parametrize("act", ["relu", "silu", "none"])
 @pytest.mark.parametrize("shape,d_in,d_hidden,d_out,depth", [((3, 40), 1, 32, 5, 1), ((2, 2), 8, 16, 4, 3), ((1, 1000), 32, 64, 16, 2)])
 def test_float32_storage(shape, d_in, d_hidden, d_out, depth, act):

@@ -801,9 +801,13 @@ extern "C" int nf_mlp_bwd(const void* x, int64_t x_stride, const void* dy, int64
   if (n == 1) return bwd_one(a, dtype, s);
   const size_t buf = boundary_bytes(rows, d_hidden);
   const size_t need = buf * (size_t)(n - 1 + 2);
-  NF_REQUIRE(workspace != nullptr && workspace_bytes >= (int64_t)need, NF_EINVAL,
-             "backward of depth %d runs as %d launches and needs a workspace of %zu bytes (nf_mlp_workspace_bytes)", depth, n,
-             need);
+  if (workspace == nullptr || workspace_bytes < (int64_t)need) {
+    // no scratch: the one-launch general kernel (partial dW through memory) where the network fits it
+    const int rc = bwd_one(a, dtype, s);
+    if (rc != NF_EUNSUPPORTED) return rc;
+    return fail(NF_EINVAL, "backward of depth %d runs as %d launches and needs a workspace of %zu bytes (nf_mlp_workspace_bytes)",
+                depth, n, need);
+  }
   NF_REQUIRE((uintptr_t)workspace % 16 == 0, NF_EINVAL, "workspace must be 16-byte aligned");
   auto bound = [&](int k) { return (uint16_t*)((char*)workspace + (size_t)k * buf); };       // output of launch k, k < n-1
   auto grad = [&](int k) { return (uint16_t*)((char*)workspace + (size_t)(n - 1 + (k & 1)) * buf); };  // d/d(input of launch k)
