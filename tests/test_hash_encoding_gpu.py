@@ -265,6 +265,25 @@ def test_backward_binned_wide_rows(N, D, F, T, L, lo, hi, do_dtype):
 
 
 @pytest.mark.parametrize("do_dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("T,L,lo,hi", [(2**22, 16, 16, 7006), (2**24, 4, 256, 2048)])
+def test_backward_binned_large_tables(T, L, lo, hi, do_dtype):
+    """Tables with more bins than the count and fill kernels hold counters for: the levels go through the pipeline
+    in groups (three groups at 2^22 rows per level, one level per group at 2^24).  Against the oracle."""
+    hk = _hk()
+    N = 40000
+    torch.manual_seed(6)
+    x = torch.rand(N, 3)
+    x[0] = 0.0
+    x[1] = 1.0
+    E = O.level_row_offsets(L, T, 3, lo, hi)[-1]
+    do = torch.randn(N, L * 2).to(do_dtype)
+    want = O.encode_backward(x, do, E, 2, None, T, L, lo, hi)
+    got = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, 2, None, T, lo, hi, L)
+    scale = max(1.0, float(want.abs().max()))
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-3, atol=1e-4 * scale)
+
+
+@pytest.mark.parametrize("do_dtype", [torch.float16, torch.float32])
 def test_backward_binned_clustered_points(do_dtype):
     """Clustered input: a few cells receive everything, so their bins are cut into several accumulation tasks
     (atomic flush), and x = 8191 sits on a bin border of the dense levels / has 13 trailing ones on hashed levels, so

@@ -29,6 +29,8 @@
 // it touches.
 //
 // Arithmetic (cell, corner rows, weights) is the forward's, see hash_encoding.hip.
+#include <vector>
+
 #include "hash_common.h"
 
 namespace nf {
@@ -44,7 +46,7 @@ constexpr int ACC_THREADS = 1024;
 constexpr int ACC_INFLIGHT = 8;               // records in flight per thread
 constexpr uint32_t SLICE_RECORDS = 98304;     // a bin with at most this many records is one accumulation task
 constexpr uint32_t SPLIT_RECORDS = 32768;     // a bigger bin is cut into tasks of about this many
-constexpr int MAX_BINS_PER_LEVEL = 1024;
+constexpr int MAX_BINS_PER_LEVEL = 2048;        // 2^24 rows
 constexpr int MAX_BINS_TOTAL = 2560;          // LDS of the count and fill kernels
 constexpr int AGG_MAX_BINS = 16;              // levels with at most this many bins rank through wave ballots
 
@@ -627,26 +629,51 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const typena
 // ---------------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------------
-static bool bin_plan(int64_t N, const nf_hash_geom* geom, int dout_dtype, BinPlan* bp, int64_t* records, uint32_t* max_tasks) {
-  // features are taken two at a time (one pass of fill + accumulate per pair)
-  if ((geom->dims != 3 && geom->dims != 2) || geom->feat < 2 || geom->feat % 2 != 0 || N <= 0) return false;
-  bp->n_levels = geom->levels;
+// Plan for levels la .. lb-1 (the kernels see them as levels 0 .. lb-la-1 of a shifted geometry).
+static bool bin_plan(int64_t N, const nf_hash_geom* geom, int la, int lb, BinPlan* bp, int64_t* records, uint32_t* max_tasks) {
+  bp->n_levels = lb - la;
   int nb_total = 0;
-  for (int l = 0; l < geom->levels; ++l) {
+  for (int l = la; l < lb; ++l) {
     const int64_t r = geom->rows[l];
     const int64_t nb = (r + BIN_ROWS - 1) / BIN_ROWS;
     if (nb > MAX_BINS_PER_LEVEL) return false;
-    bp->nbins[l] = (int)nb;
-    bp->binbase[l] = nb_total;
+    bp->nbins[l - la] = (int)nb;
+    bp->binbase[l - la] = nb_total;
     nb_total += (int)nb;
   }
-  bp->binbase[geom->levels] = nb_total;
+  bp->binbase[lb - la] = nb_total;
   if (nb_total > MAX_BINS_TOTAL) return false;
   // room for every pair to be split in two; normally half of it is used
-  const int64_t R = N * geom->levels * (geom->dims == 3 ? 8 : 4);
+  const int64_t R = N * (lb - la) * (geom->dims == 3 ? 8 : 4);
   if (R >= ((int64_t)1 << 32) - 4 * ACC_THREADS * ACC_INFLIGHT) return false;  // 32-bit record positions
   *records = R;
   *max_tasks = (uint32_t)(nb_total + R / SPLIT_RECORDS + 1);
+  return true;
+}
+
+// The count and fill kernels keep per-bin counters of all their levels in LDS (MAX_BINS_TOTAL): tables with more bins
+// go through the pipeline in groups of consecutive levels.  first[k] .. first[k+1]-1 are the levels of group k.
+static bool bin_groups(int64_t N, const nf_hash_geom* geom, std::vector<int>* first) {
+  // features are taken two at a time (one pass of fill + accumulate per pair)
+  if ((geom->dims != 3 && geom->dims != 2) || geom->feat < 2 || geom->feat % 2 != 0 || N <= 0) return false;
+  first->assign(1, 0);
+  int nb_total = 0;
+  for (int l = 0; l < geom->levels; ++l) {
+    const int64_t nb = (geom->rows[l] + BIN_ROWS - 1) / BIN_ROWS;
+    if (nb > MAX_BINS_PER_LEVEL) return false;
+    if (nb_total + nb > MAX_BINS_TOTAL) {
+      first->push_back(l);
+      nb_total = 0;
+    }
+    nb_total += (int)nb;
+  }
+  first->push_back(geom->levels);
+  for (size_t k = 0; k + 1 < first->size(); ++k) {
+    BinPlan bp;
+    int64_t R;
+    uint32_t mt;
+    if (!bin_plan(N, geom, (*first)[k], (*first)[k + 1], &bp, &R, &mt)) return false;
+  }
   return true;
 }
 
@@ -670,22 +697,57 @@ static int64_t bin_ws(void* workspace, const BinPlan& bp, int64_t N, int64_t R, 
 }
 
 int64_t bwd_bin_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype) {
-  BinPlan bp;
-  int64_t R;
-  uint32_t max_tasks;
-  if (!bin_plan(n_points, geom, dout_dtype, &bp, &R, &max_tasks)) return 0;
-  BinWs ws;
-  return bin_ws(nullptr, bp, n_points, R, dout_dtype == NF_F32 ? 4 : 3, max_tasks, &ws);
+  std::vector<int> first;
+  if (!bin_groups(n_points, geom, &first)) return 0;
+  int64_t bytes = 0;
+  for (size_t k = 0; k + 1 < first.size(); ++k) {
+    BinPlan bp;
+    int64_t R;
+    uint32_t max_tasks;
+    bin_plan(n_points, geom, first[k], first[k + 1], &bp, &R, &max_tasks);
+    BinWs ws;
+    const int64_t b = bin_ws(nullptr, bp, n_points, R, dout_dtype == NF_F32 ? 4 : 3, max_tasks, &ws);
+    if (b > bytes) bytes = b;
+  }
+  return bytes;
 }
+
+static int launch_bwd_bin_group(const void* coords, int cdt, int64_t csn, int64_t csd, const void* dout, int ddt, int64_t dout_stride,
+                                float* dtable, int64_t N, const nf_hash_geom* geom, const DevGeom& g, const BinPlan& bp, int64_t R,
+                                uint32_t max_tasks, const int64_t* primes, float scale, void* workspace, hipStream_t s);
 
 int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const void* dout, int ddt, int64_t dout_stride,
                    float* dtable, int64_t N, const nf_hash_geom* geom, const DevGeom& g, const int64_t* primes, float scale,
                    void* workspace, hipStream_t s) {
-  BinPlan bp;
-  int64_t R;
-  uint32_t max_tasks;
-  NF_REQUIRE(bin_plan(N, geom, ddt, &bp, &R, &max_tasks), NF_EUNSUPPORTED, "binned backward does not cover this geometry");
+  std::vector<int> first;
+  NF_REQUIRE(bin_groups(N, geom, &first), NF_EUNSUPPORTED, "binned backward does not cover this geometry");
   NF_REQUIRE(((uintptr_t)workspace & 15u) == 0, NF_EALIGN, "workspace must be 16-byte aligned");
+  for (size_t k = 0; k + 1 < first.size(); ++k) {
+    const int la = first[k], lb = first[k + 1];
+    BinPlan bp;
+    int64_t R;
+    uint32_t max_tasks;
+    bin_plan(N, geom, la, lb, &bp, &R, &max_tasks);
+    // the group's levels as levels 0 .. of a geometry of their own; their gradient columns start at la * feat
+    DevGeom gg = g;
+    gg.levels = lb - la;
+    gg.first_hash = g.first_hash - la;
+    for (int l = la; l < lb; ++l) {
+      gg.res[l - la] = g.res[l];
+      gg.rows[l - la] = g.rows[l];
+      gg.row_offset[l - la] = g.row_offset[l];
+    }
+    const char* dcol = (const char*)dout + (size_t)la * geom->feat * (ddt == NF_F32 ? 4 : 2);
+    if (int rc = launch_bwd_bin_group(coords, cdt, csn, csd, dcol, ddt, dout_stride, dtable, N, geom, gg, bp, R, max_tasks, primes,
+                                      scale, workspace, s))
+      return rc;
+  }
+  return 0;
+}
+
+static int launch_bwd_bin_group(const void* coords, int cdt, int64_t csn, int64_t csd, const void* dout, int ddt, int64_t dout_stride,
+                                float* dtable, int64_t N, const nf_hash_geom* geom, const DevGeom& g, const BinPlan& bp, int64_t R,
+                                uint32_t max_tasks, const int64_t* primes, float scale, void* workspace, hipStream_t s) {
   const bool g32 = ddt == NF_F32;
   BinWs ws;
   bin_ws(workspace, bp, N, R, g32 ? 4 : 3, max_tasks, &ws);

@@ -459,6 +459,7 @@ int64_t bwd_scan_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int
   int planes = 0;
   for (int l = 0; l < geom->levels; ++l)
     if (sp.plane0[l] >= 0) planes = sp.plane0[l] + sp.tiles[l];
+  if ((size_t)32 * sp.planes_pad * 4 > 150 * 1024) return 0;  // more tiles than the plan kernel's LDS holds (tables beyond 2^20 rows per level)
   // bit-planes, then the transposed gradient gT[level][point]
   return ((int64_t)planes + (int64_t)geom->levels * 32) * sp.words * 4;
 }
