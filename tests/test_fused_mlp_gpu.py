@@ -160,6 +160,61 @@ def test_chained_launches_keep_signal(act, gain, d_in, d_hidden, d_out, depth, d
         assert rel(leaves[k].grad, want["d" + k]) <= tol, k
 
 
+@pytest.mark.parametrize("depth", [2, 6])
+def test_step_replays_from_a_hip_graph(depth):
+    """The library only enqueues kernels on the caller's stream (no allocation, no synchronisation, no memset), so a
+    forward + backward step can be captured once and replayed.  Every replay, with new inputs copied into the captured
+    tensors and eager work in between, must give what the eager step gives."""
+    mk = _mk()
+    dtype = torch.bfloat16
+    rows, d_in, H, d_out = 3000, 32, 64, 16
+    p = {k: (None if v is None else v.to(DEV).requires_grad_(True)) for k, v in _params(d_in, H, d_out, depth, True, dtype, gain=6**0.5).items()}
+    x = torch.randn(1, rows, d_in).to(dtype).to(DEV).requires_grad_(True)
+    dy = torch.randn(1, rows, d_out).to(dtype).to(DEV)
+    leaves = [x] + [t for t in p.values() if t is not None]
+
+    def step():
+        for t in leaves:
+            t.grad = None
+        y = mk.fully_fused_mlp(x, p["w_in"], p["b_in"], p["w_out"], p["b_out"], p["w_hid"], p["b_hid"], "relu")
+        y.backward(dy)
+        return y
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        y_static = step()
+    grads_static = [t.grad for t in leaves]
+    for seed in (1, 2, 3):
+        torch.manual_seed(seed)
+        x_new = torch.randn(1, rows, d_in).to(dtype).to(DEV)
+        dy_new = torch.randn(1, rows, d_out).to(dtype).to(DEV)
+        with torch.no_grad():
+            x.copy_(x_new)
+            dy.copy_(dy_new)
+        g.replay()
+        torch.cuda.synchronize()
+        got_y = y_static.clone()
+        got = [t.clone() for t in grads_static]
+        # the same step eagerly, on fresh leaves holding the same values
+        xe = x_new.clone().requires_grad_(True)
+        pe = {k: (None if v is None else v.detach().clone().requires_grad_(True)) for k, v in p.items()}
+        ye = mk.fully_fused_mlp(xe, pe["w_in"], pe["b_in"], pe["w_out"], pe["b_out"], pe["w_hid"], pe["b_hid"], "relu")
+        ye.backward(dy_new)
+        torch.cuda.synchronize()
+        assert torch.equal(got_y, ye)
+        want = [xe.grad] + [t.grad for t in pe.values() if t is not None]
+        assert torch.equal(got[0], want[0])  # dx: no atomics, bitwise
+        for a, b in zip(got[1:], want[1:]):  # dW: float atomics, order may differ
+            torch.testing.assert_close(a.float(), b.float(), rtol=2e-2, atol=1e-2 * float(b.float().abs().max()))
+
+
 def test_backward_without_workspace_takes_the_one_launch_kernel():
     """A C caller that passes no workspace still gets the gradients of a narrow deep net (slower kernel); a net that
     fits no single launch is refused with the size it needs."""
