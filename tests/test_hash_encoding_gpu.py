@@ -148,6 +148,28 @@ def test_forward_kernels_agree_bitwise_at_sweep_sizes(L, hi, dtype, monkeypatch)
     torch.testing.assert_close(outs[0][idx.to(DEV)].cpu().float(), want, rtol=eps, atol=1e-6 if dtype == torch.float32 else eps * 1e-3)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("L,hi", [(16, 7006), (8, 512)])
+def test_forward_sweep_two_dimensions(L, hi, dtype, monkeypatch):
+    """Two-dimensional coordinates take the same level sweep over four corners (16-bit tables): same bits as the
+    per-(point, level) kernel (flag 1), ragged last workgroup and a coordinate scale included."""
+    hk = _hk()
+    g = GOLDEN["bench"]
+    N = 2**18 + 77
+    torch.manual_seed(3)
+    x = torch.rand(N, 2, device=DEV) * 2.5
+    table = _table(g["T"], L, 2, 16, hi, dtype=dtype, amp=1.0).to(DEV)
+    outs = []
+    for flags in (0, 1):
+        monkeypatch.setattr(hk, "_FLAGS", flags)
+        outs.append(hk.hash_encoding(x, table, None, None, g["T"], 16, hi, L, scale=2.5))
+    assert torch.equal(outs[0], outs[1])
+    idx = torch.randperm(N)[:2048]
+    want = O.encode_forward(x[idx.to(DEV)].cpu() / 2.5, table.float().cpu(), None, g["T"], L, 16, hi)
+    eps = {torch.float16: 2.0**-10, torch.bfloat16: 2.0**-7}[dtype]
+    torch.testing.assert_close(outs[0][idx.to(DEV)].cpu().float(), want, rtol=eps, atol=eps * 1e-3)
+
+
 def test_forward_config0_full_size():
     """BASELINE configs[0]: N=65536, L=16, F=2, T=2^19, fp32 table U(-1e-4, 1e-4), seed 0."""
     g = GOLDEN["bench"]

@@ -52,6 +52,35 @@ __device__ __forceinline__ Corner8 rows_d3(const uint32_t c[3], bool hashed, uin
   return r;
 }
 
+// The same for two dimensions (rows 0..3 of the result are used).
+__device__ __forceinline__ Corner8 rows_d2(const uint32_t c[3], bool hashed, uint32_t res, uint32_t mask, const uint32_t pi[3]) {
+  Corner8 r;
+  if (hashed) {
+    const uint32_t x0 = c[0] * pi[0], x1 = x0 + pi[0];
+    const uint32_t y0 = c[1] * pi[1], y1 = y0 + pi[1];
+    r.row[0] = (x0 ^ y0) & mask;
+    r.row[1] = (x1 ^ y0) & mask;
+    r.row[2] = (x0 ^ y1) & mask;
+    r.row[3] = (x1 ^ y1) & mask;
+  } else {
+    const uint32_t b = c[0] + c[1] * res;
+    r.row[0] = b;
+    r.row[1] = b + 1;
+    r.row[2] = b + res;
+    r.row[3] = b + res + 1;
+  }
+  r.row[4] = r.row[5] = r.row[6] = r.row[7] = 0u;
+  return r;
+}
+
+__device__ __forceinline__ void weights_d2(const float f[3], float w[8]) {
+  const float gx = 1.0f - f[0], gy = 1.0f - f[1];
+  w[0] = gx * gy;
+  w[1] = f[0] * gy;
+  w[2] = gx * f[1];
+  w[3] = f[0] * f[1];
+}
+
 __device__ __forceinline__ void weights_d3(const float f[3], float w[8]) {
   const float gx = 1.0f - f[0], gy = 1.0f - f[1], gz = 1.0f - f[2];
   w[0] = (gx * gy) * gz;

@@ -261,7 +261,7 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_tiled_k(const void* coo
 // that lags finds them warm and catches up).  With workgroups that start at different times, as in the staged
 // kernel's several rounds, every level's table competes for L2 at once.  (Perfect lock-step is not the aim: one
 // workgroup per CU, all in the same phase of the same level, lets the memory pipeline drain at every level.)
-template <typename TT, int PPT>
+template <typename TT, int PPT, int D>
 __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_sweep_k(const void* coords, int cdt, int64_t csn, int64_t csd,
                                                                  const uint32_t* table, uint16_t* out, int64_t out_stride,
                                                                  int64_t N, DevGeom g, const int64_t* primes, float scale) {
@@ -276,12 +276,13 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_sweep_k(const void* coo
     int64_t n = p0 + t + TILE_THREADS * i;
     if (n >= N) n = N - 1;
 #pragma unroll
-    for (int d = 0; d < 3; ++d) {
+    for (int d = 0; d < D; ++d) {
       float v = load_as_f32(coords, n * csn + d * csd, cdt);
       x[i][d] = scale != 1.0f ? v / scale : v;
     }
   }
-  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], (uint32_t)primes[2]};
+  constexpr int CN = 1 << D;  // corners of a cell
+  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], D > 2 ? (uint32_t)primes[D > 2 ? 2 : 0] : 0u};
   uint32_t enc[PPT][LMAX];
 #pragma unroll
   for (int l = 0; l < LMAX; ++l) {
@@ -300,22 +301,23 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_sweep_k(const void* coo
           uint32_t c[3];
           float fr[3];
 #pragma unroll
-          for (int d = 0; d < 3; ++d) {
+          for (int d = 0; d < D; ++d) {
             const float pos = x[i0 + i][d] * fres;
             const float fl = floorf(pos);
             c[d] = (uint32_t)(int)fl;
             fr[d] = pos - fl;
           }
-          const Corner8 r = rows_d3(c, hashed, res, mask, pi);
+          const Corner8 r = D == 3 ? rows_d3(c, hashed, res, mask, pi) : rows_d2(c, hashed, res, mask, pi);
 #pragma unroll
-          for (int j = 0; j < 8; ++j) v[i][j] = tab[r.row[j]];
-          weights_d3(fr, w[i]);
+          for (int j = 0; j < CN; ++j) v[i][j] = tab[r.row[j]];
+          if (D == 3) weights_d3(fr, w[i]);
+          else weights_d2(fr, w[i]);
         }
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
           float a0 = 0.0f, a1 = 0.0f;
 #pragma unroll
-          for (int j = 0; j < 8; ++j) {
+          for (int j = 0; j < CN; ++j) {
             a0 = a0 + w[i][j] * TT::to_f32((uint16_t)(v[i][j] & 0xffffu));
             a1 = a1 + w[i][j] * TT::to_f32((uint16_t)(v[i][j] >> 16));
           }
@@ -498,8 +500,8 @@ constexpr int64_t SCAN_MIN_POINTS = 32768;
 constexpr int SWEEP_PPT = 4;
 constexpr int64_t SWEEP_MIN_POINTS = (int64_t)256 * TILE_THREADS * SWEEP_PPT;
 
-static bool tiled_ok(const nf_hash_geom* g, int table_dt, const void* rows_ptr, int64_t row_stride, int feat = 2) {
-  if (g->dims != 3 || g->feat != feat || table_dt == NF_F32) return false;
+static bool tiled_ok(const nf_hash_geom* g, int table_dt, const void* rows_ptr, int64_t row_stride, int feat = 2, int dims = 3) {
+  if (g->dims != dims || g->feat != feat || table_dt == NF_F32) return false;
   if ((g->levels * (feat / 2)) % 4 != 0 || g->levels > 16) return false;
   for (int l = g->first_hash_level; l < g->levels; ++l) {
     if (l < 0) return false;
@@ -601,10 +603,24 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
     constexpr int P = TILE_THREADS * PPT;
     dim3 grid((unsigned)((n_points + P - 1) / P));
     if (table_dtype == NF_F16)
-      hipLaunchKernelGGL((hash_fwd_sweep_k<F16, PPT>), grid, dim3(TILE_THREADS), 0, s, coords, coords_dtype, csn, csd,
+      hipLaunchKernelGGL((hash_fwd_sweep_k<F16, PPT, 3>), grid, dim3(TILE_THREADS), 0, s, coords, coords_dtype, csn, csd,
                          (const uint32_t*)table, (uint16_t*)out, out_stride_n, n_points, g, primes, scale);
     else
-      hipLaunchKernelGGL((hash_fwd_sweep_k<BF16, PPT>), grid, dim3(TILE_THREADS), 0, s, coords, coords_dtype, csn, csd,
+      hipLaunchKernelGGL((hash_fwd_sweep_k<BF16, PPT, 3>), grid, dim3(TILE_THREADS), 0, s, coords, coords_dtype, csn, csd,
+                         (const uint32_t*)table, (uint16_t*)out, out_stride_n, n_points, g, primes, scale);
+    return check_launch("hash_fwd_sweep");
+  }
+  // two dimensions: the same sweep over four corners
+  if (!(flags & (NF_HASH_FORCE_GENERIC | NF_HASH_FWD_STAGED)) && n_points >= SWEEP_MIN_POINTS &&
+      tiled_ok(geom, table_dtype, out, out_stride_n, 2, 2)) {
+    constexpr int PPT = SWEEP_PPT;
+    constexpr int P = TILE_THREADS * PPT;
+    dim3 grid((unsigned)((n_points + P - 1) / P));
+    if (table_dtype == NF_F16)
+      hipLaunchKernelGGL((hash_fwd_sweep_k<F16, PPT, 2>), grid, dim3(TILE_THREADS), 0, s, coords, coords_dtype, csn, csd,
+                         (const uint32_t*)table, (uint16_t*)out, out_stride_n, n_points, g, primes, scale);
+    else
+      hipLaunchKernelGGL((hash_fwd_sweep_k<BF16, PPT, 2>), grid, dim3(TILE_THREADS), 0, s, coords, coords_dtype, csn, csd,
                          (const uint32_t*)table, (uint16_t*)out, out_stride_n, n_points, g, primes, scale);
     return check_launch("hash_fwd_sweep");
   }
