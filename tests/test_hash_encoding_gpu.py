@@ -431,6 +431,38 @@ def test_empty_and_edge_coordinates():
     torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-9)
 
 
+@pytest.mark.parametrize("N", [3, 2**18 + 3])
+def test_upper_edge_in_two_dimensions(N):
+    """x == scale in both of two dimensions: on a dense level the last corner (weight 0) is row (N_l + 1)^2, one past
+    the level, where the reference's CPU path raises an IndexError.  The kernels keep that corner inside the level:
+    the encoding is the table row of corner 0, whose weight is 1, and the whole upstream gradient lands there.
+    Both the small-batch kernels and the sweep / binned kernels are covered."""
+    hk = _hk()
+    T, L, lo, hi = 2**19, 16, 16, 7006
+    offs = O.level_row_offsets(L, T, 2, lo, hi)
+    table = _table(T, L, 2, lo, hi, dtype=torch.float16, amp=1.0).to(DEV).requires_grad_(True)
+    x = torch.rand(N, 2)
+    x[0] = 1.0
+    out = hk.hash_encoding(x.to(DEV), table, None, None, T, lo, hi, L)
+    rows = hk.hash_encoding_indices(x[:1].to(DEV), None, T, lo, hi, L).cpu()[0]  # (L, 4)
+    want_rows = O.encode_indices(x[1:3], None, T, L, lo, hi)
+    assert torch.equal(hk.hash_encoding_indices(x[1:3].to(DEV), None, T, lo, hi, L).cpu(), want_rows)
+    for l in range(L):
+        n_rows = offs[l + 1] - offs[l]
+        assert int(rows[l].max()) < n_rows and int(rows[l].min()) >= 0
+        assert torch.equal(out[0, 2 * l : 2 * l + 2], table[offs[l] + int(rows[l, 0])]), l
+    want = O.encode_forward(x[1:3], table.detach().float().cpu(), None, T, L, lo, hi)
+    torch.testing.assert_close(out[1:3].detach().cpu().float(), want, rtol=2.0**-10, atol=1e-6)
+    do = torch.zeros(N, 2 * L, dtype=torch.float16)
+    do[0] = 1.0
+    out.backward(do.to(DEV))
+    grad = table.grad.float().cpu()
+    for l in range(L):
+        level = grad[offs[l] : offs[l + 1]]
+        assert abs(float(level[int(rows[l, 0])].min()) - 1.0) < 1e-3  # (the binned backward carries 19-bit weights)
+        assert abs(float(level.sum()) - 2.0) < 2e-3, l
+
+
 def test_full_size_properties_config1():
     """BASELINE configs[1] at full size (N=2^20): size-independent checks.
 

@@ -63,11 +63,12 @@ __device__ __forceinline__ Corner8 rows_d2(const uint32_t c[3], bool hashed, uin
     r.row[2] = (x0 ^ y1) & mask;
     r.row[3] = (x1 ^ y1) & mask;
   } else {
+    // x == scale in both dimensions puts the last corner (weight 0) at row (res+1)^2, one past the level: keep it inside
     const uint32_t b = c[0] + c[1] * res;
     r.row[0] = b;
     r.row[1] = b + 1;
     r.row[2] = b + res;
-    r.row[3] = b + res + 1;
+    r.row[3] = min(b + res + 1, mask);
   }
   r.row[4] = r.row[5] = r.row[6] = r.row[7] = 0u;
   return r;

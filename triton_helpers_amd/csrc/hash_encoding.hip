@@ -49,7 +49,8 @@ __device__ __forceinline__ uint64_t corner_row(const Cell<D>& cell, int j, bool 
       idx += (uint64_t)(cell.c[d] + ((j >> d) & 1)) * stride;
       stride *= res;
     }
-    return idx;
+    // D <= 2: the last corner of x == scale (weight 0) would be row (res+1)^D, one past the level
+    return D <= 2 && idx >= rows ? (uint64_t)rows - 1 : idx;
   }
   uint64_t h = 0;
 #pragma unroll

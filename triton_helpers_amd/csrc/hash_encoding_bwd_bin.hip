@@ -172,7 +172,7 @@ __device__ __forceinline__ void cell_rows(const float (&v)[3], float fres, bool 
       row[0] = b;
       row[1] = b + 1;
       row[2] = b + res;
-      row[3] = b + res + 1;
+      row[3] = min(b + res + 1, mask);  // as in rows_d2: the zero-weight corner of x == scale stays inside the level
     }
     if (w != nullptr) {
       const float gx = 1.0f - fr[0], gy = 1.0f - fr[1];
