@@ -144,6 +144,9 @@ __device__ __forceinline__ void layer_nt(f32x4_t (&acc)[NT][4], const Frag (&in)
     }
 }
 
+// Four parked copies of every gradient tile and bias row must fit LDS for the one-step sum of the waves.
+constexpr bool bwd2_parallel_sum(int tiles, int nbias) { return 4 * (tiles * 1024 + nbias * 256) <= 160 * 1024; }
+
 // NT: 16-row tiles per chunk (2 or 4).  Four give the scheduler two independent 32-row groups to interleave.
 // XC: how x / dx are stored (MlpArgs::x_conv), fixed at compile time so that the usual case pays nothing for it;
 // XC == 3: stored like the weights, and the network's activation is applied to x as it is loaded (MlpArgs::in_act).
@@ -152,8 +155,25 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
   constexpr int KC_IN = KIN / 32, KC_H = HP / 32, MT_H = HP / 16, MT_I = KIN / 16, MT_O = OUTP / 16;
   constexpr int KC_O = (OUTP + 31) / 32;
   extern __shared__ __align__(16) unsigned char smem[];
-  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int tid = threadIdx.x;
+  constexpr int nthreads = 256;  // the launch's workgroup size: constant trip counts let the staging loads be issued together
   const int lane = tid & 63, wave = tid >> 6;
+
+  // the first chunk's rows are requested before the weights are staged
+  constexpr int ROWS = 16 * NT;  // rows per chunk: NT / 2 independent groups of 32 rows
+  const int64_t n_chunks = (a.rows + ROWS - 1) / ROWS;
+  const int64_t wave_stride = (int64_t)gridDim.x * 4;
+  const int64_t first_chunk = (int64_t)blockIdx.x * 4 + wave;
+  Frag nx[NT][KC_IN], ndy[NT][KC_O];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+    for (int kc = 0; kc < KC_IN; ++kc)
+      nx[nt][kc] = load_chain<FAST>(a.x, a.x_stride, first_chunk * ROWS + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
+#pragma unroll
+    for (int kc = 0; kc < KC_O; ++kc)
+      ndy[nt][kc] = load_chain<FAST>(a.dy, a.dy_stride, first_chunk * ROWS + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
+  }
 
   uint16_t* f_in = reinterpret_cast<uint16_t*>(smem);          // W_in    [MT_H][KC_IN]
   uint16_t* f_hid = f_in + MT_H * KC_IN * FRAG_ELEMS;          // W_hid   [MT_H][KC_H]
@@ -163,11 +183,11 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
   float* bias_in = reinterpret_cast<float*>(t_out + MT_H * KC_O * FRAG_ELEMS);
   float* bias_hid = bias_in + HP;
 
-  stage_weight_frags<true, false>(f_in, a.w_in, a.d_hidden, a.d_in, MT_H, KC_IN, tid, nthreads);
-  stage_weight_frags<true, false>(f_hid, a.w_hid, a.d_hidden, a.d_hidden, MT_H, KC_H, tid, nthreads);
-  stage_weight_frags<true, true>(t_in, a.w_in, a.d_hidden, a.d_in, MT_I, KC_H, tid, nthreads);
-  stage_weight_frags<true, true>(t_hid, a.w_hid, a.d_hidden, a.d_hidden, MT_H, KC_H, tid, nthreads);
-  stage_weight_frags<true, true>(t_out, a.w_out, a.d_out, a.d_hidden, MT_H, KC_O, tid, nthreads);
+  stage_weight_frags<true, false, 256>(f_in, a.w_in, a.d_hidden, a.d_in, MT_H, KC_IN, tid, nthreads);
+  stage_weight_frags<true, false, 256>(f_hid, a.w_hid, a.d_hidden, a.d_hidden, MT_H, KC_H, tid, nthreads);
+  stage_weight_frags<true, true, 256>(t_in, a.w_in, a.d_hidden, a.d_in, MT_I, KC_H, tid, nthreads);
+  stage_weight_frags<true, true, 256>(t_hid, a.w_hid, a.d_hidden, a.d_hidden, MT_H, KC_H, tid, nthreads);
+  stage_weight_frags<true, true, 256>(t_out, a.w_out, a.d_out, a.d_hidden, MT_H, KC_O, tid, nthreads);
   stage_bias<T>(bias_in, a.b_in, a.d_hidden, HP, tid, nthreads);
   stage_bias<T>(bias_hid, a.b_hid, a.d_hidden, HP, tid, nthreads);
   __syncthreads();
@@ -192,20 +212,6 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
   }
   const Frag sel[2] = {sel_frag<T>(0, lane), sel_frag<T>(1, lane)};
 
-  constexpr int ROWS = 16 * NT;  // rows per chunk: NT / 2 independent groups of 32 rows
-  const int64_t n_chunks = (a.rows + ROWS - 1) / ROWS;
-  const int64_t wave_stride = (int64_t)gridDim.x * 4;
-  const int64_t first_chunk = (int64_t)blockIdx.x * 4 + wave;
-  Frag nx[NT][KC_IN], ndy[NT][KC_O];
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-#pragma unroll
-    for (int kc = 0; kc < KC_IN; ++kc)
-      nx[nt][kc] = load_chain<FAST>(a.x, a.x_stride, first_chunk * ROWS + 16 * nt, a.rows, a.d_in, kc, lane, a.x_vec);
-#pragma unroll
-    for (int kc = 0; kc < KC_O; ++kc)
-      ndy[nt][kc] = load_chain<FAST>(a.dy, a.dy_stride, first_chunk * ROWS + 16 * nt, a.rows, a.d_out, kc, lane, a.dy_vec);
-  }
 
   for (int64_t chunk = first_chunk; chunk < n_chunks; chunk += wave_stride) {
     const int64_t row0 = chunk * ROWS;
@@ -381,6 +387,69 @@ __global__ __launch_bounds__(256, RELU ? NF_BWD2_OCC : 1) void mlp_bwd2_k(MlpArg
     }
   }
 
+  constexpr int TILES = MT_H * (MT_I + MT_H) + MT_O * MT_H, NBIAS = 2 * MT_H + MT_O;
+  constexpr bool PARALLEL_SUM = bwd2_parallel_sum(TILES, NBIAS);
+  if constexpr (PARALLEL_SUM) {
+    // ---- sum the gradients of the four waves through LDS (the weight fragments are dead by now): every wave parks its
+    // accumulators, then wave w adds up and flushes every fourth tile, so the atomics leave from all four waves ----
+    __syncthreads();
+    f32x4_t* red = reinterpret_cast<f32x4_t*>(smem);                               // [4][TILES][64]
+    float* redb = reinterpret_cast<float*>(smem) + (size_t)4 * TILES * 256;          // [4][NBIAS][64]
+    {
+      f32x4_t* mine = red + (size_t)wave * TILES * 64 + lane;
+      float* mineb = redb + (size_t)wave * NBIAS * 64 + lane;
+      int t = 0, u = 0;
+  #pragma unroll
+      for (int i = 0; i < MT_H; ++i) {
+  #pragma unroll
+        for (int j = 0; j < MT_I; ++j) mine[64 * (t++)] = dw_in[i][j];
+  #pragma unroll
+        for (int j = 0; j < MT_H; ++j) mine[64 * (t++)] = dw_hid[i][j];
+        mineb[64 * (u++)] = db_in[i];
+        mineb[64 * (u++)] = db_hid[i];
+      }
+  #pragma unroll
+      for (int i = 0; i < MT_O; ++i) {
+  #pragma unroll
+        for (int j = 0; j < MT_H; ++j) mine[64 * (t++)] = dw_out[i][j];
+        mineb[64 * (u++)] = db_out[i];
+      }
+    }
+    __syncthreads();
+    auto tile_sum = [&](int t) {
+      const f32x4_t* p = red + (size_t)t * 64 + lane;
+      return (p[0] + p[(size_t)TILES * 64]) + (p[(size_t)2 * TILES * 64] + p[(size_t)3 * TILES * 64]);
+    };
+    auto bias_sum = [&](int u) {
+      const float* p = redb + (size_t)u * 64 + lane;
+      return (p[0] + p[(size_t)NBIAS * 64]) + (p[(size_t)2 * NBIAS * 64] + p[(size_t)3 * NBIAS * 64]);
+    };
+    {
+      int t = 0, u = 0;
+  #pragma unroll
+      for (int i = 0; i < MT_H; ++i) {
+  #pragma unroll
+        for (int j = 0; j < MT_I; ++j, ++t)
+          if ((t & 3) == wave) flush_dw_tile(a.dw_in, a.d_hidden, a.d_in, i, j, lane, tile_sum(t));
+  #pragma unroll
+        for (int j = 0; j < MT_H; ++j, ++t)
+          if ((t & 3) == wave) flush_dw_tile(a.dw_hid, a.d_hidden, a.d_hidden, i, j, lane, tile_sum(t));
+        if ((u & 3) == wave) flush_db(a.db_in, a.d_hidden, i, lane, bias_sum(u));
+        ++u;
+        if ((u & 3) == wave) flush_db(a.db_hid, a.d_hidden, i, lane, bias_sum(u));
+        ++u;
+      }
+  #pragma unroll
+      for (int i = 0; i < MT_O; ++i) {
+  #pragma unroll
+        for (int j = 0; j < MT_H; ++j, ++t)
+          if ((t & 3) == wave) flush_dw_tile(a.dw_out, a.d_out, a.d_hidden, i, j, lane, tile_sum(t));
+        if ((u & 3) == wave) flush_db(a.db_out, a.d_out, i, lane, bias_sum(u));
+        ++u;
+      }
+    }
+    return;
+  }
   // ---- reduce the gradients over the four waves through LDS (the weight fragments are dead by now), then
   // one pass of atomics per workgroup ----
   __syncthreads();
@@ -805,9 +874,10 @@ static int launch2(const MlpArgs& a0, hipStream_t s) {
   constexpr int MT_H = HP / 16, MT_I = KIN / 16, MT_O = OUTP / 16;
   constexpr size_t W_BYTES = ((size_t)MT_H * (KIN / 32) + (size_t)MT_I * (HP / 32) + 2 * (size_t)MT_H * (HP / 32) + (size_t)MT_H * KC_O) * 1024 +
                              (size_t)2 * HP * 4;
-  constexpr size_t RED = (size_t)(MT_H * (MT_I + MT_H) + MT_O * MT_H) * 1024 + (size_t)(2 * MT_H + MT_O) * 256;
+  constexpr int TILES = MT_H * (MT_I + MT_H) + MT_O * MT_H, NBIAS = 2 * MT_H + MT_O;
+  constexpr size_t RED = (bwd2_parallel_sum(TILES, NBIAS) ? 4 : 1) * ((size_t)TILES * 1024 + (size_t)NBIAS * 256);
   constexpr size_t LDS = W_BYTES > RED ? W_BYTES : RED;
-  static_assert(LDS <= 64 * 1024, "LDS budget");
+  static_assert(LDS <= 160 * 1024, "LDS budget");
   a.waves = 4;
   // chain-order loads move 8 bytes at a time
   a.x_vec = ((uintptr_t)a.x % 8 == 0) && (a.x_stride % 4 == 0);
@@ -842,6 +912,10 @@ static int launch2(const MlpArgs& a0, hipStream_t s) {
     kern = fast ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, true, NT, 0> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, true, false, NT, 0>;
   } else {
     kern = fast ? (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false, true, 2, 0> : (const void*)mlp_bwd2_k<T, KIN, HP, OUTP, false, false, 2, 0>;
+  }
+  if (LDS > 64 * 1024) {
+    const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
+    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
   }
   void* args[] = {(void*)&a};
   const hipError_t e = hipLaunchKernel(kern, dim3((unsigned)blocks), dim3(256), args, LDS, s);

@@ -211,13 +211,15 @@ __device__ __forceinline__ void gate_apply(const f32x4_t dh, uint32_t g01, uint3
 // dst: fragment array [MT][KC][64 lanes][8 elements]; element (mt, kc, lane(m,g), j) =
 //   transposed ? W[kmap(kc,g,j)][16*mt+m] : W[16*mt+m][kmap(kc,g,j)]
 // where W is [w_rows][w_cols] row-major; out-of-range entries are zero.
-template <bool CHAIN, bool TRANSPOSED>
+// NTHREADS > 0: the workgroup size is that compile-time constant, the loop is unrolled and all loads of a matrix
+// are in flight together.
+template <bool CHAIN, bool TRANSPOSED, int NTHREADS = 0>
 __device__ __forceinline__ void stage_weight_frags(uint16_t* dst, const uint16_t* w, int w_rows, int w_cols, int MT,
                                                    int KC, int tid, int nthreads) {
   // one unit = the 8 elements of one lane of one fragment; the 8 loads of a unit are independent
   const int units = MT * KC * 64;
   const bool vec_ok = !TRANSPOSED && (w_cols % 4 == 0) && ((uintptr_t)w % 8 == 0);
-  for (int u = tid; u < units; u += nthreads) {
+  auto stage_unit = [&](int u) {
     const int lane = u & 63;
     const int frag = u >> 6;
     const int kc = frag % KC, mt = frag / KC;
@@ -238,7 +240,7 @@ __device__ __forceinline__ void stage_weight_frags(uint16_t* dst, const uint16_t
         for (int j = 0; j < 4; ++j)
           if (k1 + j < w_cols) reinterpret_cast<uint16_t*>(&hi)[j] = w[(size_t)m * w_cols + k1 + j];
       *reinterpret_cast<uint4*>(dst + (size_t)u * 8) = make_uint4(lo.x, lo.y, hi.x, hi.y);
-      continue;
+      return;
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -253,6 +255,12 @@ __device__ __forceinline__ void stage_weight_frags(uint16_t* dst, const uint16_t
     o.z = (uint32_t)v[4] | ((uint32_t)v[5] << 16);
     o.w = (uint32_t)v[6] | ((uint32_t)v[7] << 16);
     *reinterpret_cast<uint4*>(dst + (size_t)u * 8) = o;
+  };
+  if constexpr (NTHREADS > 0) {
+#pragma unroll
+    for (int u = tid; u < units; u += NTHREADS) stage_unit(u);
+  } else {
+    for (int u = tid; u < units; u += nthreads) stage_unit(u);
   }
 }
 
