@@ -333,6 +333,19 @@ def main():
         "step_roofline_frac": step_bytes / (h["ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "autograd_ms_per_step": h["ms_autograd"],
     }
+    # What a plain stream reaches on this GPU, next to the 8 TB/s of the data sheet: a 256 MiB out-of-place add
+    # (reads 256 MiB, writes 256 MiB) timed with events, median of 20.
+    ca = torch.zeros(64 * 2**20, dtype=torch.float32, device="cuda")
+    cb = torch.empty_like(ca)
+    copy_ms = statistics.median(event_times(lambda: torch.add(ca, 1.0, out=cb), 20)[5:])
+    copy_gbs = 2 * ca.numel() * 4 / (copy_ms * 1e-3) / 1e9
+    del ca, cb
+    out["achievable"] = {
+        "stream_GBs": copy_gbs, "how": "256 MiB read + 256 MiB write elementwise add, event-timed",
+        "fwd_frac_of_stream": achieved / copy_gbs,
+        "bwd_frac_of_stream": bwd_achieved / copy_gbs,
+        "step_frac_of_stream": step_bytes / (h["ms"] * 1e-3) / 1e9 / copy_gbs,
+    }
     if not args.no_extras:
         s, w = max(5, args.steps // 2), max(3, args.warmup // 2)
         out["workloads"] = {
