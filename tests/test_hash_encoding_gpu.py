@@ -463,6 +463,30 @@ def test_upper_edge_in_two_dimensions(N):
         assert abs(float(level.sum()) - 2.0) < 2e-3, l
 
 
+def test_upper_edge_in_one_dimension():
+    """The same edge with one coordinate: x == scale puts the second corner (weight 0) at row N_l + 1, one past a
+    dense level; it is kept at the level's last row, the encoding is the row of corner 0 and the gradient lands there."""
+    hk = _hk()
+    T, L, lo, hi = 64, 4, 8, 512
+    offs = O.level_row_offsets(L, T, 1, lo, hi)
+    table = _table(T, L, 1, lo, hi, dtype=torch.float32, amp=1.0).to(DEV).requires_grad_(True)
+    x = torch.tensor([[1.0], [0.25], [0.0]])
+    out = hk.hash_encoding(x.to(DEV), table, None, None, T, lo, hi, L)
+    rows = hk.hash_encoding_indices(x.to(DEV), None, T, lo, hi, L).cpu()
+    assert torch.equal(rows[1:], O.encode_indices(x[1:], None, T, L, lo, hi))
+    want = O.encode_forward(x[1:], table.detach().cpu(), None, T, L, lo, hi)
+    torch.testing.assert_close(out[1:].detach().cpu(), want, rtol=1e-5, atol=1e-9)
+    do = torch.zeros(3, 2 * L)
+    do[0] = 1.0
+    out.backward(do.to(DEV))
+    grad = table.grad.cpu()
+    for l in range(L):
+        n_rows = offs[l + 1] - offs[l]
+        assert 0 <= int(rows[0, l].min()) and int(rows[0, l].max()) < n_rows
+        assert torch.equal(out[0, 2 * l : 2 * l + 2], table[offs[l] + int(rows[0, l, 0])])
+        assert float(grad[offs[l] : offs[l + 1]].sum()) == 2.0
+
+
 def test_full_size_properties_config1():
     """BASELINE configs[1] at full size (N=2^20): size-independent checks.
 
