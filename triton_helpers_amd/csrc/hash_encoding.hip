@@ -262,7 +262,7 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_tiled_k(const void* coo
 // that lags finds them warm and catches up).  With workgroups that start at different times, as in the staged
 // kernel's several rounds, every level's table competes for L2 at once.  (Perfect lock-step is not the aim: one
 // workgroup per CU, all in the same phase of the same level, lets the memory pipeline drain at every level.)
-template <typename TT, int PPT, int D>
+template <typename TT, int PPT, int D, bool LDS0 = false>
 __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_sweep_k(const void* coords, int cdt, int64_t csn, int64_t csd,
                                                                  const uint32_t* table, uint16_t* out, int64_t out_stride,
                                                                  int64_t N, DevGeom g, const int64_t* primes, float scale) {
@@ -281,6 +281,13 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_sweep_k(const void* coo
       float v = load_as_f32(coords, n * csn + d * csd, cdt);
       x[i][d] = scale != 1.0f ? v / scale : v;
     }
+  }
+  // LDS0: the rows of level 0 (dense, a few thousand) are copied to LDS once per workgroup and gathered from there
+  extern __shared__ uint32_t level0_rows[];
+  if constexpr (LDS0) {
+    const uint32_t* src = table + g.row_offset[0];
+    for (uint32_t i = t; i < g.rows[0]; i += TILE_THREADS) level0_rows[i] = src[i];
+    __syncthreads();
   }
   constexpr int CN = 1 << D;  // corners of a cell
   const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], D > 2 ? (uint32_t)primes[D > 2 ? 2 : 0] : 0u};
@@ -310,7 +317,7 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_sweep_k(const void* coo
           }
           const Corner8 r = D == 3 ? rows_d3(c, hashed, res, mask, pi) : rows_d2(c, hashed, res, mask, pi);
 #pragma unroll
-          for (int j = 0; j < CN; ++j) v[i][j] = tab[r.row[j]];
+          for (int j = 0; j < CN; ++j) v[i][j] = (LDS0 && l == 0) ? level0_rows[r.row[j]] : tab[r.row[j]];
           if (D == 3) weights_d3(fr, w[i]);
           else weights_d2(fr, w[i]);
         }
@@ -603,12 +610,17 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
     constexpr int PPT = SWEEP_PPT;
     constexpr int P = TILE_THREADS * PPT;
     dim3 grid((unsigned)((n_points + P - 1) / P));
-    if (table_dtype == NF_F16)
-      hipLaunchKernelGGL((hash_fwd_sweep_k<F16, PPT, 3>), grid, dim3(TILE_THREADS), 0, s, coords, coords_dtype, csn, csd,
-                         (const uint32_t*)table, (uint16_t*)out, out_stride_n, n_points, g, primes, scale);
-    else
-      hipLaunchKernelGGL((hash_fwd_sweep_k<BF16, PPT, 3>), grid, dim3(TILE_THREADS), 0, s, coords, coords_dtype, csn, csd,
-                         (const uint32_t*)table, (uint16_t*)out, out_stride_n, n_points, g, primes, scale);
+    // level 0 in LDS where it is dense and small (19.6 KB at resolution 16): worth about 1 % (its rows mostly hit L1 anyway)
+    const bool lds0 = geom->first_hash_level > 0 && geom->rows[0] * 4 <= 32 * 1024;
+    const size_t lds = lds0 ? (size_t)geom->rows[0] * 4 : 0;
+    const void* kern = table_dtype == NF_F16 ? (lds0 ? (const void*)hash_fwd_sweep_k<F16, PPT, 3, true> : (const void*)hash_fwd_sweep_k<F16, PPT, 3>)
+                                             : (lds0 ? (const void*)hash_fwd_sweep_k<BF16, PPT, 3, true> : (const void*)hash_fwd_sweep_k<BF16, PPT, 3>);
+    const uint32_t* tab = (const uint32_t*)table;
+    uint16_t* o = (uint16_t*)out;
+    void* args[] = {(void*)&coords, (void*)&coords_dtype, (void*)&csn, (void*)&csd, (void*)&tab, (void*)&o, (void*)&out_stride_n,
+                    (void*)&n_points, (void*)&g, (void*)&primes, (void*)&scale};
+    const hipError_t e = hipLaunchKernel(kern, grid, dim3(TILE_THREADS), args, lds, s);
+    if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(hash_fwd_sweep): %s", hipGetErrorString(e));
     return check_launch("hash_fwd_sweep");
   }
   // two dimensions: the same sweep over four corners
