@@ -196,7 +196,12 @@ def bench_mlp(steps, warmup, d_out=16, rows=2**20):
         x.grad = w_in.grad = w_hid.grad = w_out.grad = None
         mk.fully_fused_mlp(x, w_in, None, w_out, None, w_hid, None, "relu").backward(dy)
 
-    ms = wall_time(step, steps, warmup)
+    # By default the autograd engine runs the backward on a device thread of its own: two hand-overs between host
+    # threads per step, which on some runs of this process cost more than the kernels (160 us against 110 us per
+    # step).  torch.autograd.set_multithreading_enabled(False) runs it on the calling thread; both are reported.
+    ms_engine_thread = wall_time(step, steps, warmup)
+    with torch.autograd.set_multithreading_enabled(False):
+        ms = wall_time(step, steps, warmup)
     flop_row = 3 * 2 * (32 * 64 + 64 * 64 + 64 * d_out)
     tflops = rows * flop_row / (ms * 1e-3) / 1e12
     out = {
@@ -205,6 +210,8 @@ def bench_mlp(steps, warmup, d_out=16, rows=2**20):
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None},
         "hbm_GBs": rows * 256 / (ms * 1e-3) / 1e9,
+        "autograd": "backward on the calling thread (torch.autograd.set_multithreading_enabled(False))",
+        "ms_per_step_engine_thread": ms_engine_thread,
     }
     # the same autograd step replayed from a HIP graph: what the kernels take once the host is out of the way
     gms = graph_time(step, steps, warmup, lambda: [x.grad, w_in.grad, w_hid.grad, w_out.grad])
