@@ -199,7 +199,8 @@ def bench_mlp(steps, warmup, d_out=16, rows=2**20):
     # By default the autograd engine runs the backward on a device thread of its own: two hand-overs between host
     # threads per step, which on some runs of this process cost more than the kernels (160 us against 110 us per
     # step).  torch.autograd.set_multithreading_enabled(False) runs it on the calling thread; both are reported.
-    ms_engine_thread = wall_time(step, steps, warmup)
+    with torch.autograd.set_multithreading_enabled(True):
+        ms_engine_thread = wall_time(step, steps, warmup)
     with torch.autograd.set_multithreading_enabled(False):
         ms = wall_time(step, steps, warmup)
     flop_row = 3 * 2 * (32 * 64 + 64 * 64 + 64 * d_out)
@@ -355,11 +356,12 @@ def main():
     }
     if not args.no_extras:
         s, w = max(5, args.steps // 2), max(3, args.warmup // 2)
-        out["workloads"] = {
-            "configs[2]": bench_mlp(s, w, 16),
-            "configs[3]": bench_rev(max(3, s // 2), 2),
-            "configs[4]": bench_e2e(max(3, s // 2), 2),
-        }
+        with torch.autograd.set_multithreading_enabled(False):  # backward on the calling thread, see bench_mlp
+            out["workloads"] = {
+                "configs[2]": bench_mlp(s, w, 16),
+                "configs[3]": bench_rev(max(3, s // 2), 2),
+                "configs[4]": bench_e2e(max(3, s // 2), 2),
+            }
     if args.calibrate_copy:
         a = torch.zeros(64 * 2**20, dtype=torch.float32, device="cuda")
         b = torch.empty_like(a)
