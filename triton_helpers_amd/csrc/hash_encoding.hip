@@ -616,11 +616,19 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
     const void* kern = table_dtype == NF_F16 ? (lds0 ? (const void*)hash_fwd_sweep_k<F16, PPT, 3, true> : (const void*)hash_fwd_sweep_k<F16, PPT, 3>)
                                              : (lds0 ? (const void*)hash_fwd_sweep_k<BF16, PPT, 3, true> : (const void*)hash_fwd_sweep_k<BF16, PPT, 3>);
     const uint32_t* tab = (const uint32_t*)table;
-    uint16_t* o = (uint16_t*)out;
-    void* args[] = {(void*)&coords, (void*)&coords_dtype, (void*)&csn, (void*)&csd, (void*)&tab, (void*)&o, (void*)&out_stride_n,
-                    (void*)&n_points, (void*)&g, (void*)&primes, (void*)&scale};
-    const hipError_t e = hipLaunchKernel(kern, grid, dim3(TILE_THREADS), args, lds, s);
-    if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(hash_fwd_sweep): %s", hipGetErrorString(e));
+    // Launches of at most 2^20 points: the workgroups of one launch are (nearly) all resident and walk the levels
+    // together; in one launch of 2^22 points later rounds of workgroups meet earlier ones at other levels and the
+    // tables compete for L2 (1545 us against 1324 us in four launches; 677 against 661 us at 2^21).
+    constexpr int64_t CHUNK = (int64_t)1 << 20;
+    for (int64_t n0 = 0; n0 < n_points; n0 += CHUNK) {
+      const int64_t n = n_points - n0 < CHUNK ? n_points - n0 : CHUNK;
+      const void* c = (const char*)coords + n0 * csn * dtype_size(coords_dtype);
+      uint16_t* o = (uint16_t*)out + n0 * out_stride_n;
+      void* args[] = {(void*)&c, (void*)&coords_dtype, (void*)&csn, (void*)&csd, (void*)&tab, (void*)&o, (void*)&out_stride_n,
+                      (void*)&n, (void*)&g, (void*)&primes, (void*)&scale};
+      const hipError_t e = hipLaunchKernel(kern, dim3((unsigned)((n + P - 1) / P)), dim3(TILE_THREADS), args, lds, s);
+      if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(hash_fwd_sweep): %s", hipGetErrorString(e));
+    }
     return check_launch("hash_fwd_sweep");
   }
   // two dimensions: the same sweep over four corners
