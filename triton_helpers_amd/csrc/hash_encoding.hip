@@ -598,9 +598,15 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
       sweep32_ok(geom, table, out, out_stride_n)) {
     constexpr int PPT = 2;
     constexpr int P = TILE_THREADS * PPT;
-    dim3 grid((unsigned)((n_points + P - 1) / P));
-    hipLaunchKernelGGL((hash_fwd_sweep32_k<PPT>), grid, dim3(TILE_THREADS), 0, s, coords, coords_dtype, csn, csd,
-                       (const float2*)table, (float*)out, out_stride_n, n_points, g, primes, scale);
+    // launches of 1024 workgroups (2^19 points), for the reason given at the 16-bit sweep below
+    // (2^20 points: 663 -> 613 us, 2^22 points: 3514 -> 2687 us)
+    constexpr int64_t CHUNK = (int64_t)1024 * P;
+    for (int64_t n0 = 0; n0 < n_points; n0 += CHUNK) {
+      const int64_t n = n_points - n0 < CHUNK ? n_points - n0 : CHUNK;
+      const void* c = (const char*)coords + n0 * csn * dtype_size(coords_dtype);
+      hipLaunchKernelGGL((hash_fwd_sweep32_k<PPT>), dim3((unsigned)((n + P - 1) / P)), dim3(TILE_THREADS), 0, s, c, coords_dtype, csn,
+                         csd, (const float2*)table, (float*)out + n0 * out_stride_n, out_stride_n, n, g, primes, scale);
+    }
     return check_launch("hash_fwd_sweep32");
   }
   // The level sweep wants at least one workgroup per compute unit; below that the staged kernel's smaller tiles
@@ -609,7 +615,6 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
       tiled_ok(geom, table_dtype, out, out_stride_n)) {
     constexpr int PPT = SWEEP_PPT;
     constexpr int P = TILE_THREADS * PPT;
-    dim3 grid((unsigned)((n_points + P - 1) / P));
     // level 0 in LDS where it is dense and small (19.6 KB at resolution 16): worth about 1 % (its rows mostly hit L1 anyway)
     const bool lds0 = geom->first_hash_level > 0 && geom->rows[0] * 4 <= 32 * 1024;
     const size_t lds = lds0 ? (size_t)geom->rows[0] * 4 : 0;
