@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define NF_ABI_VERSION 3
+#define NF_ABI_VERSION 4
 
 /* element types */
 enum { NF_F32 = 0, NF_F16 = 1, NF_BF16 = 2 };
@@ -106,6 +106,17 @@ int nf_hash_encode_indices(const void* coords, int coords_dtype, int64_t coords_
                            int64_t* out_rows, float* out_w, int64_t n_points, const nf_hash_geom* geom,
                            const int64_t* primes, float scale, void* stream);
 
+/* Host-side range check, the counterpart of the reference's debug-build asserts (tl.device_assert under
+ * TRITON_DEBUG, triton_helpers/layers/hash_encoding/kernel.py:109-122, 151, 227-228).  Runs on the CPU, launches
+ * nothing: coords is a HOST array [n_points, D] of float32 (row-contiguous), primes a HOST array of >= D values.
+ * The kernels' own index functions are evaluated for every (point, level, corner); variant 0 is the 64-bit form of
+ * the per-(point, level) kernels, variant 1 the 32-bit wrap-around form of the fast D = 2 / 3 kernels.
+ * *n_bad_rows = corner rows >= rows[level] (cells are clamped to [0, N_l], so this is 0 for any input);
+ * *n_bad_coords = coordinates outside [0, scale] or NaN (what the reference asserts);
+ * rows_out (may be NULL): HOST array [n_points, L, 2^D] receiving the level-local rows. */
+int nf_hash_check_host(const float* coords, int64_t n_points, const nf_hash_geom* geom, const int64_t* primes,
+                       float scale, int variant, int64_t* rows_out, int64_t* n_bad_rows, int64_t* n_bad_coords);
+
 /* Fully fused MLP.  x [rows, d_in] (row stride x_stride) in x_dtype, y [rows, d_out] (row stride y_stride) in `dtype`;
  * w_in [d_hidden, d_in], w_hid [(depth-1)*d_hidden, d_hidden], w_out [d_out, d_hidden], all
  * row-contiguous in `dtype`; biases b_in [d_hidden], b_hid [depth-1, d_hidden], b_out [d_out]
@@ -145,7 +156,8 @@ int nf_revmlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_stride, co
                   void* stream);
 
 /* Backward from the OUTPUT y: the inputs are recomputed block by block inside the kernel.
- * dx [rows, 2*half] in `dtype`; x_rec (may be NULL) receives the reconstructed input;
+ * dx [rows, 2*half] in `dtype`; x_rec [rows, 2*half] in `dtype` (required: the kernel carries the stream between
+ * couplings in it) receives the reconstructed input;
  * dw1, dw2, db1, db2 are float32 accumulators, NOT cleared by the call (db1, db2 may be NULL). */
 int nf_revmlp_bwd(const void* y, int64_t y_stride, const void* dy, int64_t dy_stride, void* dx, int64_t dx_stride,
                   void* x_rec, int64_t x_rec_stride, const void* w1, const void* b1, const void* w2, const void* b2,

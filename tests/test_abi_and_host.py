@@ -157,3 +157,47 @@ def test_bench_rejects_more_than_one_gpu():
 
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+def test_hash_module_seeded_table_is_the_reference_recipe():
+    """Same seed, same table: one ``randn`` draw per level, concatenated (reference hash_encoding/module.py:20-21);
+    a single draw over the stacked table gives other values."""
+    from triton_helpers_amd.layers.hash_encoding import HashEncoding
+    from triton_helpers_amd.layers.hash_encoding.helpers import compute_embedding_counts
+
+    for kw in (dict(), dict(max_entries_per_level=2**10, num_levels=4, d_in=2, d_embed=4, min_res=2, max_res=64)):
+        torch.manual_seed(123)
+        layer = HashEncoding(**kw)
+        T, L, D, F = layer.max_entries_per_level, layer.num_levels, kw.get("d_in", 3), kw.get("d_embed", 2)
+        counts = compute_embedding_counts(L, T, D, layer.min_res, layer.max_res)
+        torch.manual_seed(123)
+        want = torch.cat([torch.randn(int(t), F) for t in counts], dim=0)
+        assert torch.equal(layer.embeddings.detach(), want)
+        torch.manual_seed(123)
+        assert not torch.equal(torch.randn(sum(counts), F), want)
+        assert set(layer.state_dict().keys()) == {"embeddings", "pi"}
+        assert layer.pi.tolist() == [1, 2654435761, 805459861]
+
+
+def test_row_views_of_broadcast_and_strided_tensors():
+    """An expanded upstream gradient (``out.sum(0).backward(g)`` hands the backward ``g.expand(N, W)``, row stride 0)
+    or a strided inner dimension must reach the C ABI as rows that do not overlap."""
+    from triton_helpers_amd.layers.fully_fused_mlp.kernel import _rows2d as mlp_rows
+    from triton_helpers_amd.layers.hash_encoding.kernel import _as_rows
+    from triton_helpers_amd.layers.reversible_mlp.kernel import _rows2d as rev_rows
+
+    for fn in (_as_rows, mlp_rows, rev_rows):
+        g = torch.arange(32.0)
+        e = g.expand(5, 32)
+        r = fn(e, 32)
+        assert r.shape == (5, 32) and r.stride() == (32, 1) and torch.equal(r, e)
+        e3 = g.expand(2, 3, 32)
+        r = fn(e3, 32)
+        assert r.shape == (6, 32) and r.stride(1) == 1 and r.stride(0) >= 32 and torch.equal(r, e3.reshape(6, 32))
+        t = torch.arange(5 * 64.0).view(5, 64)
+        v = fn(t[:, :32], 32)  # wider row stride: stays a view
+        assert v.data_ptr() == t.data_ptr() and v.stride() == (64, 1)
+        s = fn(t[:, ::2], 32)  # strided inner dimension: copied
+        assert s.stride() == (32, 1) and torch.equal(s, t[:, ::2])
+        one = fn(g.expand(1, 32), 32)  # a single row has nothing to overlap with
+        assert one.shape == (1, 32)

@@ -14,7 +14,7 @@ import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "libnf_cdna4.so"
 
-NF_ABI_VERSION = 3
+NF_ABI_VERSION = 4
 NF_F32, NF_F16, NF_BF16 = 0, 1, 2
 NF_ACT = {"none": 0, "relu": 1, "silu": 2, "relu2": 3, "gelu": 4}
 NF_MAX_LEVELS = 32
@@ -34,6 +34,7 @@ EXPORTS = (
     "nf_hash_encode_bwd",
     "nf_hash_encode_bwd_workspace_bytes",
     "nf_hash_encode_indices",
+    "nf_hash_check_host",
     "nf_mlp_fwd",
     "nf_mlp_bwd",
     "nf_mlp_workspace_bytes",
@@ -85,6 +86,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.nf_hash_encode_bwd_workspace_bytes.argtypes = [I64, POINTER(HashGeom), I, I]
     lib.nf_hash_encode_indices.restype = c_int
     lib.nf_hash_encode_indices.argtypes = [P, I, I64, I64, P, P, I64, POINTER(HashGeom), P, c_float, P]
+    lib.nf_hash_check_host.restype = c_int
+    lib.nf_hash_check_host.argtypes = [P, I64, POINTER(HashGeom), P, c_float, I, P, P, P]
     lib.nf_mlp_fwd.restype = c_int
     lib.nf_mlp_fwd.argtypes = [P, I64, P, I64, P, P, P, P, P, P, I64, I, I, I, I, I, I, I, P, I64, P]
     lib.nf_mlp_workspace_bytes.restype = I64

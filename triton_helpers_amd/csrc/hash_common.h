@@ -20,7 +20,15 @@ struct Corner8 {
   uint32_t row[8];
 };
 
-__device__ __forceinline__ Corner8 rows_d3(const uint32_t c[3], bool hashed, uint32_t res, uint32_t mask,
+// Cell of a scaled coordinate: floor(pos) kept inside [0, res].  Coordinates in [0, scale] are unaffected (their
+// floor is already there); anything else -- slightly negative from normalisation noise, beyond scale, inf, NaN --
+// lands on an edge cell instead of indexing outside the level (fmaxf(NaN, 0) is 0).  The reference only asserts the
+// range in its debug build (triton_helpers/layers/hash_encoding/kernel.py:227-228).
+__host__ __device__ __forceinline__ uint32_t cell_index(float fl, float fres) {
+  return (uint32_t)(int)fminf(fmaxf(fl, 0.0f), fres);
+}
+
+__host__ __device__ __forceinline__ Corner8 rows_d3(const uint32_t c[3], bool hashed, uint32_t res, uint32_t mask,
                                            const uint32_t pi[3]) {
   Corner8 r;
   if (hashed) {
@@ -53,7 +61,7 @@ __device__ __forceinline__ Corner8 rows_d3(const uint32_t c[3], bool hashed, uin
 }
 
 // The same for two dimensions (rows 0..3 of the result are used).
-__device__ __forceinline__ Corner8 rows_d2(const uint32_t c[3], bool hashed, uint32_t res, uint32_t mask, const uint32_t pi[3]) {
+__host__ __device__ __forceinline__ Corner8 rows_d2(const uint32_t c[3], bool hashed, uint32_t res, uint32_t mask, const uint32_t pi[3]) {
   Corner8 r;
   if (hashed) {
     const uint32_t x0 = c[0] * pi[0], x1 = x0 + pi[0];
@@ -68,13 +76,13 @@ __device__ __forceinline__ Corner8 rows_d2(const uint32_t c[3], bool hashed, uin
     r.row[0] = b;
     r.row[1] = b + 1;
     r.row[2] = b + res;
-    r.row[3] = min(b + res + 1, mask);
+    r.row[3] = b + res + 1 < mask ? b + res + 1 : mask;
   }
   r.row[4] = r.row[5] = r.row[6] = r.row[7] = 0u;
   return r;
 }
 
-__device__ __forceinline__ void weights_d2(const float f[3], float w[8]) {
+__host__ __device__ __forceinline__ void weights_d2(const float f[3], float w[8]) {
   const float gx = 1.0f - f[0], gy = 1.0f - f[1];
   w[0] = gx * gy;
   w[1] = f[0] * gy;
@@ -82,7 +90,7 @@ __device__ __forceinline__ void weights_d2(const float f[3], float w[8]) {
   w[3] = f[0] * f[1];
 }
 
-__device__ __forceinline__ void weights_d3(const float f[3], float w[8]) {
+__host__ __device__ __forceinline__ void weights_d3(const float f[3], float w[8]) {
   const float gx = 1.0f - f[0], gy = 1.0f - f[1], gz = 1.0f - f[2];
   w[0] = (gx * gy) * gz;
   w[1] = (f[0] * gy) * gz;
@@ -94,6 +102,55 @@ __device__ __forceinline__ void weights_d3(const float f[3], float w[8]) {
   w[7] = (f[0] * f[1]) * f[2];
 }
 
+// ---- generic form: any D <= NF_MAX_DIMS, any level size (exact 64-bit remainder) ----
+template <int D>
+struct Cell {
+  uint32_t c[D];
+  float frac[D];
+};
+
+// x: the point's coordinates already divided by scale
+template <int D>
+__host__ __device__ __forceinline__ Cell<D> locate_cell(const float* x, int res) {
+  Cell<D> r;
+  const float fres = (float)res;
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    const float pos = x[d] * fres;
+    const float fl = floorf(pos);
+    r.c[d] = cell_index(fl, fres);
+    r.frac[d] = pos - fl;
+  }
+  return r;
+}
+
+template <int D>
+__host__ __device__ __forceinline__ uint64_t corner_row(const Cell<D>& cell, int j, bool hashed, uint32_t res, uint32_t rows,
+                                                        const uint64_t* pi) {
+  if (!hashed) {
+    uint64_t idx = 0, stride = 1;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      idx += (uint64_t)(cell.c[d] + ((j >> d) & 1)) * stride;
+      stride *= res;
+    }
+    // D <= 2: the last corner of x == scale (weight 0) would be row (res+1)^D, one past the level
+    return D <= 2 && idx >= rows ? (uint64_t)rows - 1 : idx;
+  }
+  uint64_t h = 0;
+#pragma unroll
+  for (int d = 0; d < D; ++d) h ^= (uint64_t)(cell.c[d] + ((j >> d) & 1)) * pi[d];
+  // power-of-two sizes take the mask; anything else the exact 64-bit remainder
+  return (rows & (rows - 1)) == 0 ? (h & (uint64_t)(rows - 1)) : (h % (uint64_t)rows);
+}
+
+template <int D>
+__host__ __device__ __forceinline__ float corner_weight(const Cell<D>& cell, int j) {
+  float w = ((j & 1) ? cell.frac[0] : 1.0f - cell.frac[0]);
+#pragma unroll
+  for (int d = 1; d < D; ++d) w = w * (((j >> d) & 1) ? cell.frac[d] : 1.0f - cell.frac[d]);
+  return w;
+}
 
 inline int make_dev_geom(const nf_hash_geom* geom, DevGeom* d) {
   NF_REQUIRE(geom != nullptr, NF_EINVAL, "geom is NULL");

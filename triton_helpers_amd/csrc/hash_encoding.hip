@@ -17,54 +17,15 @@ namespace nf {
 // Generic path: one thread per (point, level); any D <= 4, any F, any dtype mix.
 // ---------------------------------------------------------------------------
 template <int D>
-struct Cell {
-  uint32_t c[D];
-  float frac[D];
-};
-
-template <int D>
 __device__ __forceinline__ Cell<D> locate(const void* coords, int cdt, int64_t sn, int64_t sd, int64_t n, float scale,
                                           int res) {
-  Cell<D> r;
-  const float fres = (float)res;
+  float x[D];
 #pragma unroll
   for (int d = 0; d < D; ++d) {
-    float x = load_as_f32(coords, n * sn + d * sd, cdt);
-    if (scale != 1.0f) x = x / scale;
-    float pos = x * fres;
-    float fl = floorf(pos);
-    r.c[d] = (uint32_t)(int)fl;
-    r.frac[d] = pos - fl;
+    x[d] = load_as_f32(coords, n * sn + d * sd, cdt);
+    if (scale != 1.0f) x[d] = x[d] / scale;
   }
-  return r;
-}
-
-template <int D>
-__device__ __forceinline__ uint64_t corner_row(const Cell<D>& cell, int j, bool hashed, uint32_t res, uint32_t rows,
-                                               const uint64_t* pi) {
-  if (!hashed) {
-    uint64_t idx = 0, stride = 1;
-#pragma unroll
-    for (int d = 0; d < D; ++d) {
-      idx += (uint64_t)(cell.c[d] + ((j >> d) & 1)) * stride;
-      stride *= res;
-    }
-    // D <= 2: the last corner of x == scale (weight 0) would be row (res+1)^D, one past the level
-    return D <= 2 && idx >= rows ? (uint64_t)rows - 1 : idx;
-  }
-  uint64_t h = 0;
-#pragma unroll
-  for (int d = 0; d < D; ++d) h ^= (uint64_t)(cell.c[d] + ((j >> d) & 1)) * pi[d];
-  // power-of-two sizes take the mask; anything else the exact 64-bit remainder
-  return (rows & (rows - 1)) == 0 ? (h & (uint64_t)(rows - 1)) : (h % (uint64_t)rows);
-}
-
-template <int D>
-__device__ __forceinline__ float corner_weight(const Cell<D>& cell, int j) {
-  float w = ((j & 1) ? cell.frac[0] : 1.0f - cell.frac[0]);
-#pragma unroll
-  for (int d = 1; d < D; ++d) w = w * (((j >> d) & 1) ? cell.frac[d] : 1.0f - cell.frac[d]);
-  return w;
+  return locate_cell<D>(x, res);
 }
 
 template <int D>
@@ -196,7 +157,7 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_tiled_k(const void* coo
       for (int d = 0; d < 3; ++d) {
         const float pos = x[i][d] * fres;
         const float fl = floorf(pos);
-        c[d] = (uint32_t)(int)fl;
+        c[d] = cell_index(fl, fres);
         fr[d] = pos - fl;
       }
       const Corner8 r = rows_d3(c, hashed, res, mask, pi);
@@ -312,7 +273,7 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_sweep_k(const void* coo
           for (int d = 0; d < D; ++d) {
             const float pos = x[i0 + i][d] * fres;
             const float fl = floorf(pos);
-            c[d] = (uint32_t)(int)fl;
+            c[d] = cell_index(fl, fres);
             fr[d] = pos - fl;
           }
           const Corner8 r = D == 3 ? rows_d3(c, hashed, res, mask, pi) : rows_d2(c, hashed, res, mask, pi);
@@ -390,7 +351,7 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_sweep32_k(const void* c
         for (int d = 0; d < 3; ++d) {
           const float pos = x[i][d] * fres;
           const float fl = floorf(pos);
-          c[d] = (uint32_t)(int)fl;
+          c[d] = cell_index(fl, fres);
           fr[d] = pos - fl;
         }
         const Corner8 r = rows_d3(c, hashed, res, mask, pi);
@@ -484,7 +445,7 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_bwd_tiled_k(const void* coo
       for (int d = 0; d < 3; ++d) {
         const float pos = x[i][d] * fres;
         const float fl = floorf(pos);
-        c[d] = (uint32_t)(int)fl;
+        c[d] = cell_index(fl, fres);
         fr[d] = pos - fl;
       }
       const Corner8 r = rows_d3(c, hashed, res, mask, pi);

@@ -93,7 +93,7 @@ __device__ __forceinline__ Located3 locate(const float (&v)[3], float fres) {
   for (int d = 0; d < 3; ++d) {
     const float pos = v[d] * fres;
     const float fl = floorf(pos);
-    r.c[d] = (uint32_t)(int)fl;
+    r.c[d] = cell_index(fl, fres);
     r.fr[d] = pos - fl;
   }
   return r;
@@ -122,7 +122,7 @@ __device__ __forceinline__ void cell_rows(const float (&v)[3], float fres, bool 
     for (int d = 0; d < D; ++d) {
       const float pos = v[d] * fres;
       const float fl = floorf(pos);
-      c[d] = (uint32_t)(int)fl;
+      c[d] = cell_index(fl, fres);
       fr[d] = pos - fl;
     }
 #pragma unroll
@@ -158,7 +158,7 @@ __device__ __forceinline__ void cell_rows(const float (&v)[3], float fres, bool 
     for (int d = 0; d < 2; ++d) {
       const float pos = v[d] * fres;
       const float fl = floorf(pos);
-      c[d] = (uint32_t)(int)fl;
+      c[d] = cell_index(fl, fres);
       fr[d] = pos - fl;
     }
     if (hashed) {

@@ -63,7 +63,7 @@ __device__ __forceinline__ Located locate3(const void* coords, int cdt, int64_t 
     if (scale != 1.0f) v = v / scale;
     const float pos = v * fres;
     const float fl = floorf(pos);
-    r.c[d] = (uint32_t)(int)fl;
+    r.c[d] = cell_index(fl, fres);
     r.fr[d] = pos - fl;
   }
   return r;
@@ -238,7 +238,7 @@ __device__ __forceinline__ void scatter_point(float2* tile, uint32_t tile_id, co
     const float v = scale != 1.0f ? p.x[d] / scale : p.x[d];
     const float pos = v * fres;
     const float fl = floorf(pos);
-    q.c[d] = (uint32_t)(int)fl;
+    q.c[d] = cell_index(fl, fres);
     q.fr[d] = pos - fl;
   }
   if (hashed && xfree) {

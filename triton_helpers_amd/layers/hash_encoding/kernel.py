@@ -142,7 +142,8 @@ def _launch_backward(coords2d: Tensor, do2d: Tensor, de: Tensor, pi: Tensor, T: 
 def _as_rows(t: Tensor, width: int) -> Tensor:
     """2-D view ``(N, width)`` with unit inner stride (copies only when the layout forces it)."""
     t2 = t.reshape(-1, width)
-    if t2.stride(1) != 1:
+    # rows that overlap (an expanded / broadcast tensor has row stride 0) or a strided inner dimension: copy
+    if t2.stride(1) != 1 or (t2.shape[0] > 1 and t2.stride(0) < width):
         t2 = t2.contiguous()
     return t2
 

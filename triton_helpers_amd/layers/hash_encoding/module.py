@@ -1,7 +1,8 @@
 """``nn.Module`` wrapper of the hash encoding (reference hash_encoding/module.py:8-39).
 
 State-dict keys (``embeddings``, ``pi``), constructor arguments and the N(0,1)
-initialisation are those of the reference, so checkpoints interchange.
+initialisation (one ``torch.randn`` draw per level, in level order, reference module.py:21)
+are those of the reference, so checkpoints interchange and a seed gives the same table.
 """
 from __future__ import annotations
 
@@ -11,7 +12,7 @@ import torch
 import torch.nn as nn
 from torch import Tensor
 
-from .helpers import total_rows
+from .helpers import compute_embedding_counts
 from .kernel import PI_1, PI_2, PI_3, hash_encoding
 
 
@@ -26,9 +27,10 @@ class HashEncoding(nn.Module):
         max_res: int = 512,
     ):
         super().__init__()
-        rows = total_rows(max_entries_per_level, num_levels, d_in, min_res, max_res)
-        # one draw over the stacked table == concatenating per-level draws from the same generator
-        self.embeddings = nn.Parameter(torch.randn(rows, d_embed))
+        counts = compute_embedding_counts(num_levels, max_entries_per_level, d_in, min_res, max_res)
+        # one draw per level: the generator's block-wise normal sampling makes this differ from a single draw over
+        # the stacked table, and the seeded table has to be the reference's
+        self.embeddings = nn.Parameter(torch.cat([torch.randn(t, d_embed) for t in counts], dim=0))
         self.register_buffer("pi", torch.tensor([PI_1, PI_2, PI_3], dtype=torch.int64))
         self.max_entries_per_level = max_entries_per_level
         self.num_levels = num_levels

@@ -24,7 +24,8 @@ _ACTIVATIONS = ("gelu", "relu", "relu2", "silu", "none")
 
 def _rows2d(t: Tensor, width: int) -> Tensor:
     t2 = t.reshape(-1, width)
-    if t2.stride(1) != 1:
+    # rows that overlap (an expanded / broadcast tensor has row stride 0) or a strided inner dimension: copy
+    if t2.stride(1) != 1 or (t2.shape[0] > 1 and t2.stride(0) < width):
         t2 = t2.contiguous()
     return t2
 
