@@ -27,7 +27,15 @@ Pinning status (what independent evidence fixes each function):
   through ``encode_forward`` and the per-level column-sum invariant.
 * ``mlp.*`` -- pinned against ``torch.nn.Linear`` chains with autograd, the
   reference's own baseline (``tests/test_layers/test_fully_fused_mlp.py:21-35``).
+  The 16-bit mode (``round_to=``, ``ste_round``) is pinned separately in
+  ``tests/test_oracle_mlp.py``: against ``nn.Linear`` chains whose tensors are
+  bfloat16 / float16 under CPU autograd, against a hand-written float64
+  back-propagation through the rounded activations, on integer inputs where
+  nothing rounds (the mode must be invisible), and on a known answer.
 * ``reversible.*`` -- PARITY UNPINNED BY THE REFERENCE (the reference holds no
   reversible MLP).  Pinned only by mathematics: ``inverse(forward(x)) == x`` and
-  gradients equal to autograd through the plain composition.
+  gradients equal to autograd through the plain composition.  Its 16-bit mode
+  (``round_to=``, ``stream_round_every=``) is pinned against a composition with
+  the rounding points written out, against couplings of 16-bit ``nn.Linear``
+  modules, on integer inputs where nothing rounds, and on a known answer.
 """

@@ -103,15 +103,19 @@ __device__ __forceinline__ void flush_dw_tile(float* dw, int out_dim, int in_dim
     if (r0 + r < out_dim) unsafeAtomicAdd(dw + (size_t)(r0 + r) * in_dim + c, v[r]);
 }
 
+// Compute units of the current device.  The count is cached per device ordinal (written once with the same value by
+// whichever thread asks first); besides the thread-local error text this is the only state the library keeps.
 inline int device_cus() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0;
+  static int cus[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cus[dev] == 0) {
     hipDeviceProp_t p;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) cus = p.multiProcessorCount;
-    if (cus <= 0) cus = 256;
+    int n = 0;
+    if (hipGetDeviceProperties(&p, dev) == hipSuccess) n = p.multiProcessorCount;
+    cus[dev] = n > 0 ? n : 256;
   }
-  return cus;
+  return cus[dev];
 }
 
 constexpr size_t LDS_LIMIT = 160 * 1024;

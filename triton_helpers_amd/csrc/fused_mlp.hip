@@ -809,6 +809,17 @@ extern "C" int nf_mlp_bwd(const void* x, int64_t x_stride, const void* dy, int64
                 depth, n, need);
   }
   NF_REQUIRE((uintptr_t)workspace % 16 == 0, NF_EINVAL, "workspace must be 16-byte aligned");
+  if (a.x_conv != 0) {
+    // Only the first launch sees x, and it runs last: by then the launches behind it have added into the caller's
+    // accumulators.  Whatever would make it refuse the conversion is therefore checked before anything is launched,
+    // so that a caller who casts x and calls again does not count the later layers' gradients twice.
+    const MlpArgs g0 = launch_args(a, first[0], first[1]);
+    const bool aligned = ((uintptr_t)x % 8 == 0) && (x_stride % 4 == 0) && (d_in % 4 == 0) &&
+                         (dx == nullptr || ((uintptr_t)dx % 8 == 0 && dx_stride % 4 == 0));
+    NF_REQUIRE(g0.depth == 2 && d_hidden > 32 && act == NF_ACT_RELU && aligned, NF_EUNSUPPORTED,
+               "x_dtype != dtype: the backward converts x on the fly only in a first launch of three linear layers, d_hidden > 32, "
+               "ReLU and 8-byte aligned rows (nothing was launched; cast x and call again)");
+  }
   auto bound = [&](int k) { return (uint16_t*)((char*)workspace + (size_t)k * buf); };       // output of launch k, k < n-1
   auto grad = [&](int k) { return (uint16_t*)((char*)workspace + (size_t)(n - 1 + (k & 1)) * buf); };  // d/d(input of launch k)
   // replay the forward up to the last boundary
