@@ -3,8 +3,8 @@
 The reference holds no reversible MLP, so parity with the reference is UNPINNED for this layer; the
 oracle is pinned by mathematics (tests/test_oracle_mlp.py).  Tolerance: rtol 2e-2 / atol 1e-2 on y,
 dx and (relative to their scale) dw/db, against the oracle on the 16-bit-rounded inputs with the
-stream rounded to the storage dtype after every coupling; beyond 4 couplings the absolute tolerance
-grows with blocks / 4.  ReLU is left out of the gradient check on purpose: the backward rebuilds the
+stream rounded to the storage dtype after every coupling, plus half a storage ulp of the stream's largest
+magnitude per coupling (see ``_close``).  ReLU is left out of the gradient check on purpose: the backward rebuilds the
 inputs from 16-bit outputs, so pre-activations within rounding of zero switch their gate and move
 single gradients by whole weights; the smooth activations (GELU is the BASELINE one) have no such jump.
 """
@@ -30,13 +30,21 @@ def _params(blocks, H, bias, dtype, seed=0):
     return u(blocks * 2 * H, H), (u(blocks * 2, H) if bias else None), u(blocks * 2 * H, H), (u(blocks * 2, H) if bias else None)
 
 
+EPS = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11}
+
+
 def _close(got, want, what, scale_rel=False, blocks=4):
+    """rtol 2e-2 / atol 1e-2, plus what the storage format itself costs: the backward hands the stream (x, dx) from
+    one coupling to the next in the 16-bit storage dtype, so every element of the stream is rounded once per
+    coupling, by at most half an ulp of the stream's magnitude (2^-9 of it in bfloat16, 2^-12 in float16).  An element
+    whose terms cancel to ~0 keeps that absolute error, hence the term ``blocks * eps / 2 * max|want|``.  Weight
+    gradients (``scale_rel``) are sums over all rows and are compared relative to their largest magnitude."""
+    dtype = got.dtype
     got, want = got.detach().cpu().float(), want.float()
-    # a stream element is a sum of terms of the stream's own size, each rounded to 16 bit at the block
-    # boundaries of the backward: where the stream has grown past unit scale (identity activation) an
-    # element that cancels to ~0 keeps a rounding error proportional to that scale
-    k = max(1.0, blocks / 4) * max(1.0, float(want.pow(2).mean().sqrt()))
-    atol = max(ATOL * k, RTOL * k * float(want.abs().max())) if scale_rel else ATOL * k
+    peak = float(want.abs().max())
+    atol = ATOL + blocks * 0.5 * EPS.get(dtype, 2.0**-8) * peak
+    if scale_rel:
+        atol = max(atol, RTOL * peak)
     torch.testing.assert_close(got, want, rtol=RTOL, atol=atol, msg=lambda m: f"{what}: {m}")
 
 
@@ -62,7 +70,7 @@ def test_forward_backward(rows, H, blocks, bias, act, dtype):
     xd = x.to(DEV).requires_grad_(True)
     y = rk.reversible_mlp(xd, *leaves, act)
     assert y.shape == x.shape and y.dtype == dtype
-    _close(y, want_y, "y", blocks=blocks)
+    _close(y, want_y, "y", blocks=(blocks + 3) // 4)  # the forward rounds the stream once per four couplings
     y.backward(dy.to(DEV))
     _close(xd.grad, want["dx"], "dx", blocks=blocks)
     for name, leaf in zip(("dw1", "db1", "dw2", "db2"), leaves):
@@ -116,7 +124,7 @@ def test_relu_forward(rows, H, blocks, dtype):
     x = torch.randn(rows, 2 * H).to(dtype)
     want_y = R.rev_forward(x, w1, b1, w2, b2, "relu", round_to=dtype, stream_round_every=4).to(dtype)
     y = rk.reversible_mlp(x.to(DEV), *(t.to(DEV) for t in (w1, b1, w2, b2)), "relu")
-    _close(y, want_y, "y", blocks=blocks)
+    _close(y, want_y, "y", blocks=(blocks + 3) // 4)  # the forward rounds the stream once per four couplings
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -203,3 +211,35 @@ def test_module_and_errors():
     y32 = layer(x.detach())
     assert y32.dtype == torch.float32
     torch.testing.assert_close(y32, y.detach().float(), rtol=2e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize(
+    "case,rows,H,blocks,act,bias,dtype",
+    [
+        (22, 1000, 16, 5, "gelu", False, torch.bfloat16),
+        (47, 40000, 48, 8, "gelu", False, torch.bfloat16),
+        (93, 1024, 64, 4, "none", True, torch.bfloat16),
+        (111, 4097, 32, 4, "none", False, torch.bfloat16),
+    ],
+)
+def test_cases_that_once_missed_the_tolerance(case, rows, H, blocks, act, bias, dtype):
+    """Four randomly drawn shapes on which a single element of dx came out 10-15 % beyond an absolute tolerance that
+    was scaled with the RMS of dx: the element was one whose terms cancel, and its error was the 16-bit rounding of
+    the stream at the coupling boundaries, which scales with the stream's magnitude, not with the element's.  They
+    are kept as regression cases for the bound stated in ``_close``."""
+    rk = _rk()
+    torch.manual_seed(case)
+    w1, b1, w2, b2 = _params(blocks, H, bias, dtype, seed=case)
+    x = torch.randn(rows, 2 * H).to(dtype)
+    dy = torch.randn(rows, 2 * H).to(dtype)
+    want_y = R.rev_forward(x, w1, b1, w2, b2, act, round_to=dtype, stream_round_every=4).to(dtype)
+    want = R.rev_backward(x, dy, w1, b1, w2, b2, act, round_to=dtype)
+    leaves = [None if t is None else t.to(DEV).requires_grad_(True) for t in (w1, b1, w2, b2)]
+    xd = x.to(DEV).requires_grad_(True)
+    y = rk.reversible_mlp(xd, *leaves, act)
+    _close(y, want_y, "y", blocks=(blocks + 3) // 4)  # the forward rounds the stream once per four couplings
+    y.backward(dy.to(DEV))
+    _close(xd.grad, want["dx"], "dx", blocks=blocks)
+    for name, leaf in zip(("dw1", "db1", "dw2", "db2"), leaves):
+        if leaf is not None:
+            _close(leaf.grad, want[name], name, scale_rel=True, blocks=blocks)
