@@ -6,23 +6,31 @@
 The headline workload is BASELINE.json ``configs[1]``: multiresolution hash encoding,
 forward + backward, N = 2^20 points, L = 16, F = 2, T = 2^19, fp16 tables, fp16 upstream
 gradient, float32 table gradient.  One step = forward launch + clearing the float32
-gradient table + backward launch(es), inputs resident in HBM.  ``value`` is Mpoints/s.
+gradient table + backward launch(es), inputs resident in HBM.  ``value`` is Mpoints/s over
+exactly K steps of wall time; ``event_ms`` gives the median and the 20 % / 80 % quantiles of the
+same K steps timed one by one with events (the reference's ``do_bench`` statistics,
+triton_helpers/benchmark.py:151-153, 179-184: warm-up 20, 100 repetitions, median, quantiles).
 
 Extra objects in the same line:
   roofline      the dominant kernel of the step (the forward gather kernel: the backward is a
                 chain of five shorter kernels), algorithmic bytes per launch / launch time measured
-                here with events against the 8 TB/s HBM peak; ``traffic`` is that kernel's HBM
-                traffic from the FETCH_SIZE / WRITE_SIZE counters of a profiler run;
+                here with events against the 8 TB/s HBM peak; ``traffic`` (HBM bytes per launch) and
+                the L2 request count come from the counters in the committed profile summary;
   cpu_baseline  the CPU oracle (a port of the reference's PyTorch path) timed on this host
-                on a 65536-point sample of the same workload;
+                on a 65536-point sample of the same workload; ``cpu_baselines`` holds the same for
+                the other configurations (configs[0] is the reference's own CPU-runnable case);
   workloads     the other BASELINE configs (fused MLP, reversible MLP, end-to-end step) with
                 their own throughput and MFMA roofline fraction.
+
+``--only 2`` (= ``configs[2]``; also 1, 3, 4) runs that workload alone, W warm-up + K steps, and prints its object: the
+command to put behind ``rocprofv3 ... --`` for per-kernel counters.
 """
 from __future__ import annotations
 
 import argparse
 import json
 import os
+import re
 import statistics
 import sys
 import time
@@ -35,6 +43,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16
+# L2: 16 channels per XCD, 128 bytes per clock each, 8 XCDs, 2.4 GHz
+L2_PEAK_GBS = 16 * 128 * 8 * 2.4
 
 # geometry of BASELINE configs[1] ("base 16, growth 1.5, L=16" == min_res 16, max_res 7006)
 T, L, F, D, MIN_RES, MAX_RES = 2**19, 16, 2, 3, 16, 7006
@@ -42,13 +52,33 @@ N_POINTS = 2**20
 # algorithmic bytes per point: fwd = 4D + L*2^D*F*2 + L*F*2 ; bwd = 4D + L*F*2 + L*2^D*F*4
 FWD_BYTES_PER_POINT = 4 * D + L * 8 * F * 2 + L * F * 2  # 588
 BWD_BYTES_PER_POINT = 4 * D + L * F * 2 + L * 8 * F * 4  # 1100
-# HBM bytes per forward launch at N = 2^20 measured with rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a 256 MiB copy
-# kernel gives for that counter) + WRITE_SIZE (x1.0): 842 MB + 67 MB
-FWD_TRAFFIC_BYTES = 9.10e8
+PROFILE_SUMMARY = os.path.join(ROOT, "profiles", "hash_encoding_fwd_bwd_2p20.md")
+E2E_LOSS_SCALE = 2.0**20
+CPU_SAMPLE = 65536
+
+
+def profile_figures():
+    """Counter-derived figures of the forward kernel, kept in the committed profile summary as a line
+    ``<!-- bench-figures: key=value ... -->`` next to the tables they come from (None when absent)."""
+    try:
+        text = open(PROFILE_SUMMARY).read()
+    except OSError:
+        return {}
+    m = re.search(r"<!--\s*bench-figures:(.*?)-->", text, flags=re.S)
+    if not m:
+        return {}
+    return {k: float(v) for k, v in re.findall(r"(\w+)=([0-9.eE+-]+)", m.group(1))}
+
+
+def quantiles(ms):
+    s = sorted(ms)
+    pick = lambda q: s[min(len(s) - 1, int(q * (len(s) - 1) + 0.5))]  # noqa: E731
+    return {"median": statistics.median(s), "p20": pick(0.2), "p80": pick(0.8), "n": len(s)}
 
 
 def event_times(fn, reps):
-    """Per-call GPU duration (ms) of ``fn`` measured with events on the current stream."""
+    """Per-call GPU duration (ms) of ``fn`` measured with events on the current stream (the stream the library
+    launches on)."""
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
     for a, b in evs:
         a.record()
@@ -100,6 +130,7 @@ def graph_time(fn, steps, warmup, check):
         return None
 
 
+# ------------------------------------------------------------------------------------------------ GPU workloads
 def bench_hash(steps, warmup):
     from triton_helpers_amd.layers.hash_encoding import kernel as hk
     from triton_helpers_amd.layers.hash_encoding.helpers import total_rows
@@ -129,10 +160,11 @@ def bench_hash(steps, warmup):
         bwd()
 
     ms = wall_time(step, steps, warmup)
-    reps = max(10, min(steps, 50))
-    t_fwd = statistics.mean(event_times(fwd, reps))
-    t_zero = statistics.mean(event_times(zero, reps))
-    t_bwd = statistics.mean(event_times(bwd, reps))
+    step_ev = quantiles(event_times(step, steps))
+    reps = max(10, min(steps, 100))
+    fwd_ev = quantiles(event_times(fwd, reps))
+    t_zero = statistics.median(event_times(zero, reps))
+    bwd_ev = quantiles(event_times(bwd, reps))
 
     # the same step through autograd (table grad rounded to fp16 by the engine), for information
     e = table.clone().requires_grad_(True)
@@ -142,44 +174,10 @@ def bench_hash(steps, warmup):
         hk.hash_encoding(x, e, None, pi, T, MIN_RES, MAX_RES, L).backward(do)
 
     ms_autograd = wall_time(step_autograd, max(5, steps // 5), 3)
-    return dict(ms=ms, t_fwd=t_fwd, t_zero=t_zero, t_bwd=t_bwd, ms_autograd=ms_autograd, E=E)
+    return dict(ms=ms, step_ev=step_ev, fwd_ev=fwd_ev, t_zero=t_zero, bwd_ev=bwd_ev, ms_autograd=ms_autograd, E=E)
 
 
-def cpu_baseline_hash():
-    """CPU oracle (port of the reference's PyTorch path) on a 65536-point sample of the workload."""
-    from oracle import hash_encoding as O
-
-    n = 65536
-    threads = min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(threads)
-    torch.manual_seed(0)
-    E = O.level_row_offsets(L, T, D, MIN_RES, MAX_RES)[-1]
-    x = torch.rand(n, D)
-    table = ((torch.rand(E, F) * 2 - 1) * 1e-4).half()
-    do = torch.randn(n, L * F).half()
-
-    def run():
-        O.encode_forward(x, table, None, T, L, MIN_RES, MAX_RES)
-        O.encode_backward(x, do, E, F, None, T, L, MIN_RES, MAX_RES)
-
-    run()
-    times = []
-    t_start = time.perf_counter()
-    while len(times) < 3 or (time.perf_counter() - t_start < 10 and len(times) < 20):
-        t0 = time.perf_counter()
-        run()
-        times.append(time.perf_counter() - t0)
-    med = statistics.median(times)
-    return {
-        "value": n / med / 1e6,
-        "unit": "Mpoints/s",
-        "cores": torch.get_num_threads(),
-        "kind": "port",
-        "sample": f"fwd+bwd of {n} points, same geometry (L=16,F=2,T=2^19), fp16 table, fp32 grad; median of {len(times)} runs",
-    }
-
-
-def bench_mlp(steps, warmup, d_out=16, rows=2**20):
+def bench_mlp(steps, warmup, d_out=16, rows=2**20, graph=True):
     from triton_helpers_amd.layers.fully_fused_mlp import kernel as mk
 
     dev = torch.device("cuda", 0)
@@ -196,29 +194,35 @@ def bench_mlp(steps, warmup, d_out=16, rows=2**20):
         x.grad = w_in.grad = w_hid.grad = w_out.grad = None
         mk.fully_fused_mlp(x, w_in, None, w_out, None, w_hid, None, "relu").backward(dy)
 
-    # By default the autograd engine runs the backward on a device thread of its own: two hand-overs between host
-    # threads per step, which on some runs of this process cost more than the kernels (160 us against 110 us per
-    # step).  torch.autograd.set_multithreading_enabled(False) runs it on the calling thread; both are reported.
+    # The headline is the step as torch runs it by default: the autograd engine executes the backward on a device
+    # thread of its own, two hand-overs between host threads per step.  With
+    # torch.autograd.set_multithreading_enabled(False) the backward runs on the calling thread; that figure and the
+    # replay of the captured step from a HIP graph are reported beside it.
     with torch.autograd.set_multithreading_enabled(True):
-        ms_engine_thread = wall_time(step, steps, warmup)
-    with torch.autograd.set_multithreading_enabled(False):
         ms = wall_time(step, steps, warmup)
+        ev = quantiles(event_times(step, steps))
+    with torch.autograd.set_multithreading_enabled(False):
+        ms_calling_thread = wall_time(step, steps, warmup)
     flop_row = 3 * 2 * (32 * 64 + 64 * 64 + 64 * d_out)
-    tflops = rows * flop_row / (ms * 1e-3) / 1e12
+
+    def tf(t_ms):
+        return rows * flop_row / (t_ms * 1e-3) / 1e12
+
     out = {
-        "workload": f"fused MLP 32->64->64->{d_out} ReLU bf16 fwd+bwd, {rows} rows (through autograd)",
-        "value": rows / ms / 1e3, "unit": "Mrows/s", "ms_per_step": ms,
-        "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None},
+        "workload": f"configs[2]: fused MLP 32->64->64->{d_out} ReLU bf16 fwd+bwd, {rows} rows (through autograd, default engine)",
+        "value": rows / ms / 1e3, "unit": "Mrows/s", "ms_per_step": ms, "event_ms": ev,
+        "roofline": {"bound": "mfma", "achieved": tf(ms), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tf(ms) / MFMA_BF16_PEAK_TFLOPS, "traffic": None},
         "hbm_GBs": rows * 256 / (ms * 1e-3) / 1e9,
-        "autograd": "backward on the calling thread (torch.autograd.set_multithreading_enabled(False))",
-        "ms_per_step_engine_thread": ms_engine_thread,
+        "backward_on_calling_thread": {"ms_per_step": ms_calling_thread, "achieved": tf(ms_calling_thread), "unit": "TFLOP/s",
+                                       "frac": tf(ms_calling_thread) / MFMA_BF16_PEAK_TFLOPS,
+                                       "how": "torch.autograd.set_multithreading_enabled(False)"},
     }
-    # the same autograd step replayed from a HIP graph: what the kernels take once the host is out of the way
-    gms = graph_time(step, steps, warmup, lambda: [x.grad, w_in.grad, w_hid.grad, w_out.grad])
-    if gms is not None:
-        gt = rows * flop_row / (gms * 1e-3) / 1e12
-        out["hip_graph"] = {"ms_per_step": gms, "achieved": gt, "unit": "TFLOP/s", "frac": gt / MFMA_BF16_PEAK_TFLOPS}
+    if graph:
+        with torch.autograd.set_multithreading_enabled(False):
+            gms = graph_time(step, steps, warmup, lambda: [x.grad, w_in.grad, w_hid.grad, w_out.grad])
+        if gms is not None:
+            out["hip_graph"] = {"ms_per_step": gms, "achieved": tf(gms), "unit": "TFLOP/s", "frac": tf(gms) / MFMA_BF16_PEAK_TFLOPS}
     return out
 
 
@@ -238,18 +242,19 @@ def bench_rev(steps, warmup, rows=2**20):
         rk.reversible_mlp(x, w1, None, w2, None, "gelu").backward(dy)
 
     ms = wall_time(step, steps, warmup)
+    ev = quantiles(event_times(step, steps))
     flop_row = 3 * 2 * blocks * 4 * H * H
     tflops = rows * flop_row / (ms * 1e-3) / 1e12
     return {
-        "workload": f"reversible MLP width 128, 4 couplings, GELU bf16 fwd+bwd, {rows} rows (through autograd)",
-        "value": rows / ms / 1e3, "unit": "Mrows/s", "ms_per_step": ms,
+        "workload": f"configs[3]: reversible MLP width 128, 4 couplings, GELU bf16 fwd+bwd, {rows} rows (through autograd)",
+        "value": rows / ms / 1e3, "unit": "Mrows/s", "ms_per_step": ms, "event_ms": ev,
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None},
     }
 
 
 def bench_e2e(steps, warmup, n=2**21):
-    """BASELINE configs[4]: encode -> MLP 32->64->64->4 -> MSE, forward + backward through autograd."""
+    """BASELINE configs[4]: encode -> MLP 32->64->64->4 -> MSE (mean), forward + backward through autograd."""
     from triton_helpers_amd.layers.fully_fused_mlp import kernel as mk
     from triton_helpers_amd.layers.hash_encoding import kernel as hk
     from triton_helpers_amd.layers.hash_encoding.helpers import total_rows
@@ -271,22 +276,128 @@ def bench_e2e(steps, warmup, n=2**21):
         enc = hk.hash_encoding(x, table, None, None, T, MIN_RES, MAX_RES, L)
         # the fp16 encoding goes straight into the bf16 MLP, which converts it while loading (and writes dx as fp16)
         y = mk.fully_fused_mlp(enc.unsqueeze(0), w_in, None, w_out, None, w_hid, None, "relu")
-        # summed (not averaged) squared error: keeps the fp16 gradient that reaches the encoder out of underflow
-        loss = torch.nn.functional.mse_loss(y.float().squeeze(0), target, reduction="sum")
-        loss.backward()
+        loss = torch.nn.functional.mse_loss(y.float().squeeze(0), target)
+        # Mean over n * 4 elements: the gradient that reaches the fp16 encoding is ~1e-9 and would underflow, as in
+        # any fp16 training step; a constant loss scale (what torch.amp.GradScaler applies dynamically) keeps it in
+        # range.  The gradients come out multiplied by it (an optimiser step would divide them).
+        (loss * E2E_LOSS_SCALE).backward()
 
     ms = wall_time(step, steps, warmup)
-    return {"workload": f"end-to-end step: {n} points -> hash encoding -> MLP 32->64->64->4 -> summed squared error, fwd+bwd",
-            "value": n / ms / 1e3, "unit": "Mpoints/s", "ms_per_step": ms}
+    ev = quantiles(event_times(step, steps))
+    return {"workload": f"configs[4]: end-to-end step: {n} points -> hash encoding -> MLP 32->64->64->4 -> MSE (mean), "
+                        f"loss scale 2^20, fwd+bwd",
+            "value": n / ms / 1e3, "unit": "Mpoints/s", "ms_per_step": ms, "event_ms": ev}
 
 
+# ------------------------------------------------------------------------------------------------ CPU baselines
+def _cpu_threads():
+    """Threads for the CPU baselines: the host's cores, at most 16 -- a GPU box of this pool gives one GPU's job a share
+    of 16 cores (its OMP_NUM_THREADS is preset to 16), whatever os.cpu_count() shows."""
+    n = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(n)
+    return n
+
+
+def _time_cpu(run, budget_s=6.0, max_reps=20):
+    run()  # warm-up
+    times, t_start = [], time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < max_reps):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    return statistics.median(times), len(times)
+
+
+def _cpu_entry(n, med, reps, unit, sample):
+    return {"value": n / med / 1e6, "unit": unit, "cores": torch.get_num_threads(), "host_cpu_count": os.cpu_count(),
+            "kind": "port", "sample": f"{sample}; median of {reps} runs"}
+
+
+def cpu_baseline_hash(backward=True, fp32=False):
+    """CPU oracle (port of the reference's PyTorch path, triton_helpers/layers/hash_encoding/kernel.py:482-502) on a
+    65536-point sample of the workload; ``fp32`` + forward only is BASELINE configs[0] at its full size."""
+    from oracle import hash_encoding as O
+
+    n = CPU_SAMPLE
+    _cpu_threads()
+    torch.manual_seed(0)
+    E = O.level_row_offsets(L, T, D, MIN_RES, MAX_RES)[-1]
+    x = torch.rand(n, D)
+    table = (torch.rand(E, F) * 2 - 1) * 1e-4
+    table = table if fp32 else table.half()
+    do = torch.randn(n, L * F).half()
+
+    def run():
+        O.encode_forward(x, table, None, T, L, MIN_RES, MAX_RES)
+        if backward:
+            O.encode_backward(x, do, E, F, None, T, L, MIN_RES, MAX_RES)
+
+    med, reps = _time_cpu(run)
+    what = "fwd+bwd" if backward else "forward"
+    tab = "fp32 table" if fp32 else "fp16 table, fp32 grad"
+    return _cpu_entry(n, med, reps, "Mpoints/s", f"{what} of {n} points, same geometry (L=16,F=2,T=2^19), {tab}")
+
+
+def cpu_baseline_mlp(d_out=16):
+    """float32 F.linear chain with autograd (the reference tests' baseline, tests/test_layers/test_fully_fused_mlp.py:21-35)."""
+    from oracle import mlp as M
+
+    n = CPU_SAMPLE
+    _cpu_threads()
+    torch.manual_seed(0)
+    w_in, w_hid, w_out = torch.randn(64, 32) / 6, torch.randn(64, 64) / 8, torch.randn(d_out, 64) / 8
+    x, dy = torch.randn(n, 32), torch.randn(n, d_out)
+    med, reps = _time_cpu(lambda: M.mlp_backward(x, dy, w_in, None, w_out, None, w_hid, None, "relu"))
+    return _cpu_entry(n, med, reps, "Mrows/s", f"fwd+bwd of {n} rows, 32->64->64->{d_out} ReLU, float32")
+
+
+def cpu_baseline_rev():
+    from oracle import reversible as R
+
+    n = CPU_SAMPLE
+    _cpu_threads()
+    torch.manual_seed(0)
+    w1, w2 = torch.randn(4 * 2 * 64, 64) / 8, torch.randn(4 * 2 * 64, 64) / 8
+    x, dy = torch.randn(n, 128), torch.randn(n, 128)
+    med, reps = _time_cpu(lambda: R.rev_backward(x, dy, w1, None, w2, None, "gelu"))
+    return _cpu_entry(n, med, reps, "Mrows/s", f"fwd+bwd of {n} rows, width 128, 4 couplings, GELU, float32, stored activations")
+
+
+def cpu_baseline_e2e():
+    from oracle import hash_encoding as O
+    from oracle import mlp as M
+
+    n = CPU_SAMPLE
+    _cpu_threads()
+    torch.manual_seed(0)
+    E = O.level_row_offsets(L, T, D, MIN_RES, MAX_RES)[-1]
+    x = torch.rand(n, D)
+    table = ((torch.rand(E, F) * 2 - 1) * 1e-4).half()
+    target = torch.rand(n, 4)
+    w_in, w_hid, w_out = torch.randn(64, 32) / 6, torch.randn(64, 64) / 8, torch.randn(4, 64) / 8
+
+    def run():
+        enc = O.encode_forward(x, table, None, T, L, MIN_RES, MAX_RES).float().requires_grad_(True)
+        leaves = [t.clone().requires_grad_(True) for t in (w_in, w_out, w_hid)]
+        y = M.mlp_forward(enc, leaves[0], None, leaves[1], None, leaves[2], None, "relu")
+        torch.nn.functional.mse_loss(y, target).backward()
+        O.encode_backward(x, enc.grad, E, F, None, T, L, MIN_RES, MAX_RES)
+
+    med, reps = _time_cpu(run)
+    return _cpu_entry(n, med, reps, "Mpoints/s", f"fwd+bwd of {n} points: encode -> MLP 32->64->64->4 -> MSE, float32")
+
+
+# ------------------------------------------------------------------------------------------------ main
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--only", choices=["configs[1]", "configs[2]", "configs[3]", "configs[4]", "1", "2", "3", "4"], default=None,
+                    help="run this workload alone (for per-kernel profiling) and print its object; a bare digit is "
+                         "short for configs[digit]")
     ap.add_argument("--no-extras", action="store_true", help="skip the MLP / end-to-end workloads")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one out-of-place add over 256 MiB (a copy kernel of known traffic, for scaling "
                          "the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
@@ -294,6 +405,8 @@ def main():
                     help="NF_HASH_* flag bits passed to the hash-encoding entry points (profiling the alternative "
                          "kernels, e.g. 8 = LDS-staged forward); the default 0 is what the bench line is quoted on")
     args = ap.parse_args()
+    if args.only and len(args.only) == 1:
+        args.only = f"configs[{args.only}]"
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (points are independent, so the work "
               "would shard over points with one gradient all-reduce). Run with --gpus 1.", file=sys.stderr)
@@ -306,13 +419,34 @@ def main():
         from triton_helpers_amd.layers.hash_encoding import kernel as hk
         hk._FLAGS = args.hash_kernel_flags
 
+    if args.only and args.only != "configs[1]":
+        fn = {"configs[2]": lambda: bench_mlp(args.steps, args.warmup, 16, graph=False),
+              "configs[3]": lambda: bench_rev(args.steps, args.warmup),
+              "configs[4]": lambda: bench_e2e(args.steps, args.warmup)}[args.only]
+        print(json.dumps(fn()))
+        return
+
     h = bench_hash(args.steps, args.warmup)
     # The forward is one kernel (hash_fwd_sweep_k); the backward is zero + count + offsets + fill + accumulate, each
     # shorter than the forward kernel.
-    dom, dom_ms, dom_bytes = ("hash_fwd_tiled_k" if args.hash_kernel_flags & 8 else "hash_fwd_sweep_k"), h["t_fwd"], FWD_BYTES_PER_POINT * N_POINTS
+    dom = "hash_fwd_tiled_k" if args.hash_kernel_flags & 8 else "hash_fwd_sweep_k"
+    dom_ms, dom_bytes = h["fwd_ev"]["median"], FWD_BYTES_PER_POINT * N_POINTS
+    t_bwd = h["bwd_ev"]["median"]
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
-    bwd_achieved = BWD_BYTES_PER_POINT * N_POINTS / (h["t_bwd"] * 1e-3) / 1e9
+    bwd_achieved = BWD_BYTES_PER_POINT * N_POINTS / (t_bwd * 1e-3) / 1e9
     step_bytes = (FWD_BYTES_PER_POINT + BWD_BYTES_PER_POINT) * N_POINTS + h["E"] * F * 4
+    figs = profile_figures() if not args.hash_kernel_flags else {}
+    roofline = {
+        "bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": achieved / HBM_PEAK_GBS, "traffic": figs.get("fwd_traffic_bytes"),
+        "launch_ms": dom_ms, "launch_ms_p20_p80": [h["fwd_ev"]["p20"], h["fwd_ev"]["p80"]],
+        "algorithmic_bytes_per_launch": dom_bytes,
+    }
+    if "fwd_l2_read_requests" in figs:
+        # the gathers are served by L2 (90 % hits): requests that leave the CUs x 128-byte lines over the launch time
+        l2 = figs["fwd_l2_read_requests"] * 128 / (dom_ms * 1e-3) / 1e9
+        roofline["l2"] = {"read_requests": figs["fwd_l2_read_requests"], "achieved": l2, "peak": L2_PEAK_GBS, "unit": "GB/s",
+                          "frac": l2 / L2_PEAK_GBS, "peak_how": "16 channels x 128 B/clk x 8 XCDs x 2.4 GHz"}
     out = {
         "metric": "Mpoints/s fwd+bwd: hash-enc+fused MLP @2^20 pts; % HBM / MFMA peak",
         "value": N_POINTS / h["ms"] / 1e3,
@@ -331,16 +465,17 @@ def main():
                         "fp16 tables and upstream grad, float32 table gradient (zero-fill included in the step)",
             "points": N_POINTS, "levels": L, "features": F, "table_rows_per_level": T,
         },
-        "roofline": {
-            "bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": FWD_TRAFFIC_BYTES,
-            "launch_ms": dom_ms, "algorithmic_bytes_per_launch": dom_bytes,
-        },
-        "phases_ms": {"hash_fwd": h["t_fwd"], "grad_zero_fill": h["t_zero"], "hash_bwd": h["t_bwd"]},
+        "event_ms": h["step_ev"],
+        "roofline": roofline,
+        "phases_ms": {"hash_fwd": dom_ms, "grad_zero_fill": h["t_zero"], "hash_bwd": t_bwd,
+                      "hash_bwd_p20_p80": [h["bwd_ev"]["p20"], h["bwd_ev"]["p80"]]},
         "bwd_roofline_frac": bwd_achieved / HBM_PEAK_GBS,
         "step_roofline_frac": step_bytes / (h["ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "autograd_ms_per_step": h["ms_autograd"],
     }
+    if args.only == "configs[1]":
+        print(json.dumps(out))
+        return
     # What a plain stream reaches on this GPU, next to the 8 TB/s of the data sheet: a 256 MiB out-of-place add
     # (reads 256 MiB, writes 256 MiB) timed with events, median of 20.
     ca = torch.zeros(64 * 2**20, dtype=torch.float32, device="cuda")
@@ -356,12 +491,11 @@ def main():
     }
     if not args.no_extras:
         s, w = max(5, args.steps // 2), max(3, args.warmup // 2)
-        with torch.autograd.set_multithreading_enabled(False):  # backward on the calling thread, see bench_mlp
-            out["workloads"] = {
-                "configs[2]": bench_mlp(s, w, 16),
-                "configs[3]": bench_rev(max(3, s // 2), 2),
-                "configs[4]": bench_e2e(max(3, s // 2), 2),
-            }
+        out["workloads"] = {
+            "configs[2]": bench_mlp(s, w, 16),
+            "configs[3]": bench_rev(max(3, s // 2), 3),
+            "configs[4]": bench_e2e(max(3, s // 2), 3),
+        }
     if args.calibrate_copy:
         a = torch.zeros(64 * 2**20, dtype=torch.float32, device="cuda")
         b = torch.empty_like(a)
@@ -370,6 +504,12 @@ def main():
         torch.cuda.synchronize()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_hash()
+        out["cpu_baselines"] = {
+            "configs[0]": cpu_baseline_hash(backward=False, fp32=True),
+            "configs[2]": cpu_baseline_mlp(16),
+            "configs[3]": cpu_baseline_rev(),
+            "configs[4]": cpu_baseline_e2e(),
+        }
     print(json.dumps(out))
 
 

@@ -124,5 +124,10 @@ constexpr size_t LDS_LIMIT = 160 * 1024;
 // Specialised backward for exactly one hidden layer (fused_mlp_bwd2.hip), bias gradients included.
 // *handled = false: shape not covered, nothing was launched.
 int launch_mlp_bwd2(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
+// The same for two or three hidden-to-hidden layers of width 64 with ReLU (fused_mlp_bwdn.hip).
+int launch_mlp_bwdn(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
+// The benchmark shape of launch_mlp_bwd2 (d_in <= 32, d_hidden = 64, d_out <= 16, ReLU, aligned rows, extents below
+// 2^31 bytes) on eight waves per workgroup (fused_mlp_bwd2_w8.hip).  *handled = false: not that shape.
+int launch_mlp_bwd2_w8(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
 
 }  // namespace nf

@@ -364,6 +364,39 @@ __device__ __forceinline__ Frag sel_frag(int half, int lane) {
   return e;
 }
 
+// Transpose through LDS with gfx950's transposing reads.  A wave parks the row-per-lane fragments of a 32-row chunk as a
+// row-major panel panel[row][feature] (TR_STRIDE dwords per row: 64 features + 2, so the 16 rows a store instruction
+// touches fall on 16 different bank pairs and the rows r, r+4, r+8, r+12 of one read on disjoint 8-bank windows), then
+// reads, for a tile of 16 features, lane (i, g) <- feature 16*tile + i of the rows g + 4k (k = 0..3) and 16 + g + 4k: the
+// operand of a product that contracts over the chunk's 32 rows.  Both operands of such a product come from here, so
+// they share the row order.  ds_read_b64_tr_b16: within 16 lanes, lane p supplies the address of 4 consecutive 16-bit
+// values M[p][0..3]; lane i receives M[4k + i / 4][i % 4], k = 0..3.  LDS operations of one wave complete in order, so
+// a wave that parks and reads its own panel needs no barrier.
+constexpr int TR_STRIDE = 34;
+constexpr int TR_PANEL_DWORDS = 32 * TR_STRIDE;
+// fragment f = K-chunk kc (chain order) of row tile nt (rows 16*nt .. 16*nt+15)
+template <bool BOTH_HALVES = true>
+__device__ __forceinline__ void park_frag_rows(uint32_t* panel, const Frag& f, int nt, int kc, int lane) {
+  uint32_t* p = panel + (16 * nt + (lane & 15)) * TR_STRIDE + 16 * kc + 2 * (lane >> 4);
+  *reinterpret_cast<uint2*>(p) = make_uint2(f.w[0], f.w[1]);                       // features 32*kc + 4g .. +3
+  if (BOTH_HALVES) *reinterpret_cast<uint2*>(p + 8) = make_uint2(f.w[2], f.w[3]);  // features 32*kc + 16 + 4g .. +3
+}
+typedef short tr_v4i16 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ Frag tr_operand(const uint32_t* panel, int tile, int lane) {
+  const int i = lane & 15, g = lane >> 4;
+  const uint32_t* p = panel + (g + 4 * (i >> 2)) * TR_STRIDE + 8 * tile + 2 * (i & 3);
+  typedef tr_v4i16 __attribute__((address_space(3))) * lds_ptr;
+  const tr_v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)p);
+  const tr_v4i16 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 16 * TR_STRIDE));
+  Frag f;
+  const uint2 a = __builtin_bit_cast(uint2, lo), b = __builtin_bit_cast(uint2, hi);
+  f.w[0] = a.x;
+  f.w[1] = a.y;
+  f.w[2] = b.x;
+  f.w[3] = b.y;
+  return f;
+}
+
 // acc + lo + hi of a packed 16-bit pair (one v_dot2 instruction)
 template <typename T>
 __device__ __forceinline__ float dot2_ones(uint32_t p, float acc);
