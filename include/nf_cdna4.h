@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define NF_ABI_VERSION 4
+#define NF_ABI_VERSION 5
 
 /* element types */
 enum { NF_F32 = 0, NF_F16 = 1, NF_BF16 = 2 };
@@ -99,6 +99,19 @@ int nf_hash_encode_bwd(const void* coords, int coords_dtype, int64_t coords_stri
  * (No counterpart in the reference: its backward allocates nothing besides the gradient table,
  * triton_helpers/layers/hash_encoding/kernel.py:636.) */
 int64_t nf_hash_encode_bwd_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype, int flags);
+
+/* nf_hash_encode_bwd without the workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The
+ * scratch of the sort-and-accumulate kernels is a device array inside the library, NF_HASH_BWD_STATIC_BYTES per GPU,
+ * held until the process ends; the call allocates and frees nothing.  Batches whose scratch does not fit take the
+ * smaller bit-plane variant where that applies (3-D points, 16-bit gradients: up to about 1.1 M points at L = 16) and
+ * are refused with NF_EINVAL beyond that.  All calls on one GPU share the array: calls that overlap in time on one
+ * GPU race on it.  Same arguments and results as nf_hash_encode_bwd otherwise. */
+#define NF_HASH_BWD_STATIC_BYTES (128 * 1024 * 1024)
+int nf_hash_encode_bwd_static(const void* coords, int coords_dtype, int64_t coords_stride_n, int64_t coords_stride_d,
+                              const void* dout, int dout_dtype, int64_t dout_stride_n, float* dtable, int64_t n_points,
+                              const nf_hash_geom* geom, const int64_t* primes, float scale, int flags, void* stream);
+int64_t nf_hash_encode_bwd_static_bytes(void);
 
 /* Level-local table rows of all 2^D corners: out_rows [n_points, L, 2^D] int64, and
  * (optional, may be NULL) the interpolation weights out_w [n_points, L, 2^D] float32. */

@@ -14,7 +14,7 @@ import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "libnf_cdna4.so"
 
-NF_ABI_VERSION = 4
+NF_ABI_VERSION = 5
 NF_F32, NF_F16, NF_BF16 = 0, 1, 2
 NF_ACT = {"none": 0, "relu": 1, "silu": 2, "relu2": 3, "gelu": 4}
 NF_MAX_LEVELS = 32
@@ -33,6 +33,8 @@ EXPORTS = (
     "nf_hash_encode_fwd",
     "nf_hash_encode_bwd",
     "nf_hash_encode_bwd_workspace_bytes",
+    "nf_hash_encode_bwd_static",
+    "nf_hash_encode_bwd_static_bytes",
     "nf_hash_encode_indices",
     "nf_hash_check_host",
     "nf_mlp_fwd",
@@ -84,6 +86,10 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.nf_hash_encode_bwd.argtypes = [P, I, I64, I64, P, I, I64, P, I64, POINTER(HashGeom), P, c_float, P, I64, I, P]
     lib.nf_hash_encode_bwd_workspace_bytes.restype = c_int64
     lib.nf_hash_encode_bwd_workspace_bytes.argtypes = [I64, POINTER(HashGeom), I, I]
+    lib.nf_hash_encode_bwd_static.restype = c_int
+    lib.nf_hash_encode_bwd_static.argtypes = [P, I, I64, I64, P, I, I64, P, I64, POINTER(HashGeom), P, c_float, I, P]
+    lib.nf_hash_encode_bwd_static_bytes.restype = c_int64
+    lib.nf_hash_encode_bwd_static_bytes.argtypes = []
     lib.nf_hash_encode_indices.restype = c_int
     lib.nf_hash_encode_indices.argtypes = [P, I, I64, I64, P, P, I64, POINTER(HashGeom), P, c_float, P]
     lib.nf_hash_check_host.restype = c_int

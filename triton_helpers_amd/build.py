@@ -33,7 +33,7 @@ COMMON_FLAGS = [
     f"-I{CSRC}",
 ]
 # Files whose float arithmetic must not be contracted into FMAs (bit-exact cell / weight math).
-NO_CONTRACT = {"hash_encoding.hip", "hash_encoding_bwd_scan.hip", "hash_encoding_bwd_bin.hip"}
+NO_CONTRACT = {"hash_encoding.hip", "hash_encoding_bwd_scan.hip", "hash_encoding_bwd_bin.hip", "hash_encoding_bwd_static.hip", "hash_check_host.hip"}
 # Files whose MFMA results feed vector ALU work directly: keep them in architectural VGPRs instead of
 # bouncing every result through an accumulation register.
 MFMA_VGPR_FORM = {"fused_mlp.hip", "fused_mlp_bwd2.hip", "fused_mlp_bwdn.hip", "fused_mlp_bwd2_w8.hip", "reversible_mlp.hip"}

@@ -29,8 +29,6 @@
 // it touches.
 //
 // Arithmetic (cell, corner rows, weights) is the forward's, see hash_encoding.hip.
-#include <vector>
-
 #include "hash_common.h"
 
 namespace nf {
@@ -653,26 +651,34 @@ static bool bin_plan(int64_t N, const nf_hash_geom* geom, int la, int lb, BinPla
 
 // The count and fill kernels keep per-bin counters of all their levels in LDS (MAX_BINS_TOTAL): tables with more bins
 // go through the pipeline in groups of consecutive levels.  first[k] .. first[k+1]-1 are the levels of group k.
-static bool bin_groups(int64_t N, const nf_hash_geom* geom, std::vector<int>* first) {
+// (A fixed array, no heap: the entry points allocate nothing, on the host either.)
+struct LevelGroups {
+  int n;                             // groups
+  int first[NF_MAX_LEVELS + 2];      // first[k] .. first[k + 1] - 1
+  size_t size() const { return (size_t)n + 1; }
+  int operator[](size_t k) const { return first[k]; }
+};
+static bool bin_groups(int64_t N, const nf_hash_geom* geom, LevelGroups* groups) {
   // features are taken two at a time (one pass of fill + accumulate per pair)
   if ((geom->dims != 3 && geom->dims != 2) || geom->feat < 2 || geom->feat % 2 != 0 || N <= 0) return false;
-  first->assign(1, 0);
+  groups->n = 0;
+  groups->first[0] = 0;
   int nb_total = 0;
   for (int l = 0; l < geom->levels; ++l) {
     const int64_t nb = (geom->rows[l] + BIN_ROWS - 1) / BIN_ROWS;
     if (nb > MAX_BINS_PER_LEVEL) return false;
     if (nb_total + nb > MAX_BINS_TOTAL) {
-      first->push_back(l);
+      groups->first[++groups->n] = l;
       nb_total = 0;
     }
     nb_total += (int)nb;
   }
-  first->push_back(geom->levels);
-  for (size_t k = 0; k + 1 < first->size(); ++k) {
+  groups->first[++groups->n] = geom->levels;
+  for (int k = 0; k < groups->n; ++k) {
     BinPlan bp;
     int64_t R;
     uint32_t mt;
-    if (!bin_plan(N, geom, (*first)[k], (*first)[k + 1], &bp, &R, &mt)) return false;
+    if (!bin_plan(N, geom, groups->first[k], groups->first[k + 1], &bp, &R, &mt)) return false;
   }
   return true;
 }
@@ -697,7 +703,7 @@ static int64_t bin_ws(void* workspace, const BinPlan& bp, int64_t N, int64_t R, 
 }
 
 int64_t bwd_bin_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype) {
-  std::vector<int> first;
+  LevelGroups first;
   if (!bin_groups(n_points, geom, &first)) return 0;
   int64_t bytes = 0;
   for (size_t k = 0; k + 1 < first.size(); ++k) {
@@ -719,7 +725,7 @@ static int launch_bwd_bin_group(const void* coords, int cdt, int64_t csn, int64_
 int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const void* dout, int ddt, int64_t dout_stride,
                    float* dtable, int64_t N, const nf_hash_geom* geom, const DevGeom& g, const int64_t* primes, float scale,
                    void* workspace, hipStream_t s) {
-  std::vector<int> first;
+  LevelGroups first;
   NF_REQUIRE(bin_groups(N, geom, &first), NF_EUNSUPPORTED, "binned backward does not cover this geometry");
   NF_REQUIRE(((uintptr_t)workspace & 15u) == 0, NF_EALIGN, "workspace must be 16-byte aligned");
   for (size_t k = 0; k + 1 < first.size(); ++k) {
