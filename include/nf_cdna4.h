@@ -19,6 +19,7 @@
  *   nf_mlp_fwd             <- _fwd_kernel[grid](...)   triton_helpers/layers/fully_fused_mlp/kernel.py:553-562 (kernel :181-261)
  *   nf_mlp_bwd             <- _bwd_kernel_rfs[grid](...) + host sum(0)
  *                                                      triton_helpers/layers/fully_fused_mlp/kernel.py:612-633 (kernel :307-500)
+ *   nf_table_adam_step, nf_hash_encode_bwd_static, nf_hash_check_host : no counterpart (see their declarations)
  *   nf_revmlp_fwd / nf_revmlp_bwd : no counterpart in the reference (it has no
  *                             reversible MLP); same conventions as nf_mlp_*.
  */
@@ -129,6 +130,16 @@ int nf_hash_encode_indices(const void* coords, int coords_dtype, int64_t coords_
  * rows_out (may be NULL): HOST array [n_points, L, 2^D] receiving the level-local rows. */
 int nf_hash_check_host(const float* coords, int64_t n_points, const nf_hash_geom* geom, const int64_t* primes,
                        float scale, int variant, int64_t* rows_out, int64_t* n_bad_rows, int64_t* n_bad_coords);
+
+/* One Adam step (torch.optim.Adam's arithmetic: no amsgrad, L2 weight decay) over a table of n_elems values and the
+ * float32 gradient nf_hash_encode_bwd accumulated for it.  No counterpart in the reference, which ships no
+ * optimiser: the natural neighbour of its scatter-add, triton_helpers/layers/hash_encoding/kernel.py:432, 636.
+ * table [n_elems] in table_dtype; master: float32 copy of the parameters (NULL: the table itself is the parameter);
+ * grad is divided by grad_scale (the loss scale) before use and, with clear_grad != 0, zeroed for the next backward;
+ * exp_avg / exp_avg_sq: float32 moments; step counts from 1. */
+int nf_table_adam_step(void* table, int table_dtype, float* master, float* grad, float* exp_avg, float* exp_avg_sq,
+                       int64_t n_elems, int64_t step, float lr, float beta1, float beta2, float eps, float weight_decay,
+                       float grad_scale, int clear_grad, void* stream);
 
 /* Fully fused MLP.  x [rows, d_in] (row stride x_stride) in x_dtype, y [rows, d_out] (row stride y_stride) in `dtype`;
  * w_in [d_hidden, d_in], w_hid [(depth-1)*d_hidden, d_hidden], w_out [d_out, d_hidden], all

@@ -37,6 +37,7 @@ EXPORTS = (
     "nf_hash_encode_bwd_static_bytes",
     "nf_hash_encode_indices",
     "nf_hash_check_host",
+    "nf_table_adam_step",
     "nf_mlp_fwd",
     "nf_mlp_bwd",
     "nf_mlp_workspace_bytes",
@@ -94,6 +95,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.nf_hash_encode_indices.argtypes = [P, I, I64, I64, P, P, I64, POINTER(HashGeom), P, c_float, P]
     lib.nf_hash_check_host.restype = c_int
     lib.nf_hash_check_host.argtypes = [P, I64, POINTER(HashGeom), P, c_float, I, P, P, P]
+    lib.nf_table_adam_step.restype = c_int
+    lib.nf_table_adam_step.argtypes = [P, I, P, P, P, P, I64, I64, c_float, c_float, c_float, c_float, c_float, c_float, I, P]
     lib.nf_mlp_fwd.restype = c_int
     lib.nf_mlp_fwd.argtypes = [P, I64, P, I64, P, P, P, P, P, P, I64, I, I, I, I, I, I, I, P, I64, P]
     lib.nf_mlp_workspace_bytes.restype = I64
