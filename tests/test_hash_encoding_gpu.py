@@ -545,3 +545,27 @@ def test_full_size_properties_config1():
     const = torch.full((E, 2), 0.25, dtype=torch.float16, device=DEV)
     oc = hk.hash_encoding(xd, const, None, None, T, 16, 7006, 16)
     torch.testing.assert_close(oc.float(), torch.full_like(oc, 0.25, dtype=torch.float32), rtol=1e-3, atol=0)
+
+
+def test_backward_in_pieces_beyond_two_million_points():
+    """Batches above 2^21 points run through the sort-and-accumulate pipeline in pieces: the workspace stops growing and
+    the gradient equals the sum of the halves' gradients computed separately."""
+    from triton_helpers_amd import _lib
+
+    hk = _hk()
+    T, L, lo, hi = 2**14, 16, 16, 512
+    E = O.level_row_offsets(L, T, 3, lo, hi)[-1]
+    from triton_helpers_amd.layers.hash_encoding.helpers import level_geometry
+
+    geom = level_geometry(T, L, 3, 2, lo, hi)
+    lib = _lib.load()
+    assert lib.nf_hash_encode_bwd_workspace_bytes(2**22, geom, _lib.NF_F16, 0) == lib.nf_hash_encode_bwd_workspace_bytes(2**21, geom, _lib.NF_F16, 0)
+    N = 2**21 + 12345
+    g = torch.Generator().manual_seed(3)
+    x = torch.rand(N, 3, generator=g).to(DEV)
+    do = torch.randn(N, 32, generator=g).half().to(DEV)
+    whole = hk.hash_encoding_table_grad(x, do, E, 2, None, T, lo, hi, L)
+    cut = 2**20 + 77
+    parts = hk.hash_encoding_table_grad(x[:cut], do[:cut], E, 2, None, T, lo, hi, L)
+    hk.hash_encoding_table_grad(x[cut:], do[cut:], E, 2, None, T, lo, hi, L, out=parts)
+    torch.testing.assert_close(whole, parts, rtol=1e-4, atol=1e-3 * float(parts.abs().mean()))

@@ -702,7 +702,14 @@ static int64_t bin_ws(void* workspace, const BinPlan& bp, int64_t N, int64_t R, 
   return o * 4;
 }
 
+// Batches above this many points go through the pipeline in pieces of this size, one after the other on the stream:
+// the scratch stays at ~3 GiB (4 GiB with a float32 upstream gradient) whatever the batch, and record positions stay
+// inside 32 bits.  The gradient table accumulates across the pieces.  (Pieces of 2^20 points would halve the scratch
+// and cost 2.5 % of a 2^21-point training step: every piece pays the fixed part of the pipeline again.)
+constexpr int64_t BIN_CHUNK_POINTS = (int64_t)1 << 21;
+
 int64_t bwd_bin_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype) {
+  if (n_points > BIN_CHUNK_POINTS) n_points = BIN_CHUNK_POINTS;
   LevelGroups first;
   if (!bin_groups(n_points, geom, &first)) return 0;
   int64_t bytes = 0;
@@ -722,9 +729,25 @@ static int launch_bwd_bin_group(const void* coords, int cdt, int64_t csn, int64_
                                 float* dtable, int64_t N, const nf_hash_geom* geom, const DevGeom& g, const BinPlan& bp, int64_t R,
                                 uint32_t max_tasks, const int64_t* primes, float scale, void* workspace, hipStream_t s);
 
+static int launch_bwd_bin_piece(const void* coords, int cdt, int64_t csn, int64_t csd, const void* dout, int ddt, int64_t dout_stride,
+                                float* dtable, int64_t N, const nf_hash_geom* geom, const DevGeom& g, const int64_t* primes, float scale,
+                                void* workspace, hipStream_t s);
+
 int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const void* dout, int ddt, int64_t dout_stride,
                    float* dtable, int64_t N, const nf_hash_geom* geom, const DevGeom& g, const int64_t* primes, float scale,
                    void* workspace, hipStream_t s) {
+  for (int64_t n0 = 0; n0 < N; n0 += BIN_CHUNK_POINTS) {
+    const int64_t n = N - n0 < BIN_CHUNK_POINTS ? N - n0 : BIN_CHUNK_POINTS;
+    const char* c = (const char*)coords + n0 * csn * dtype_size(cdt);
+    const char* d = (const char*)dout + n0 * dout_stride * dtype_size(ddt);
+    if (int rc = launch_bwd_bin_piece(c, cdt, csn, csd, d, ddt, dout_stride, dtable, n, geom, g, primes, scale, workspace, s)) return rc;
+  }
+  return 0;
+}
+
+static int launch_bwd_bin_piece(const void* coords, int cdt, int64_t csn, int64_t csd, const void* dout, int ddt, int64_t dout_stride,
+                                float* dtable, int64_t N, const nf_hash_geom* geom, const DevGeom& g, const int64_t* primes, float scale,
+                                void* workspace, hipStream_t s) {
   LevelGroups first;
   NF_REQUIRE(bin_groups(N, geom, &first), NF_EUNSUPPORTED, "binned backward does not cover this geometry");
   NF_REQUIRE(((uintptr_t)workspace & 15u) == 0, NF_EALIGN, "workspace must be 16-byte aligned");
