@@ -5,7 +5,7 @@ Here the comparison is with the oracle as the reference's tests use it -- a floa
 rounds (tests/test_layers/test_fully_fused_mlp.py:231-289) -- at rtol 2e-2 / atol 1e-2, and what is asserted is the
 FRACTION of elements outside that tolerance: a ReLU unit whose pre-activation lies within 16-bit rounding of zero has
 its gate on one side in float32 and on the other in bfloat16, which moves that row's ``dx`` by a whole weight.  Every
-test appends what it measured to ``gpurun_out/parity_report.json`` when that folder exists.
+test appends what it measured to the file named by the environment variable ``NF_PARITY_REPORT``, when that is set.
 
 Also here: the binned hash-encoding backward against the oracle at the full 2^20 points of configs[1], level by
 level, and the composed end-to-end step of configs[4].
@@ -28,10 +28,9 @@ T, L, F, D, LO, HI = 2**19, 16, 2, 3, 16, 7006
 
 
 def _report(name, values):
-    out = os.path.join(ROOT, "gpurun_out")
-    if not os.path.isdir(out):
+    path = os.environ.get("NF_PARITY_REPORT")
+    if not path:
         return
-    path = os.path.join(out, "parity_report.json")
     data = {}
     if os.path.exists(path):
         try:

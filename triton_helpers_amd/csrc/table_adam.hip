@@ -1,7 +1,7 @@
 // One Adam step over a stacked hash table and the float32 gradient table that nf_hash_encode_bwd accumulates.
 //
-// The reference has no optimiser; this is the natural neighbour of its scatter-add (SURVEY of the hot path, "next"
-// rows): the step reads the float32 gradient once, un-scales it (loss scaling), updates the float32 moments and the
+// The reference has no optimiser; this is the natural neighbour of its scatter-add
+// (triton_helpers/layers/hash_encoding/kernel.py:432, 636): the step reads the float32 gradient once, un-scales it (loss scaling), updates the float32 moments and the
 // float32 master copy, writes the 16-bit (or float32) table the encoder gathers from, and clears the gradient for the
 // next backward -- the separate zero-fill pass over the gradient table disappears.
 //
