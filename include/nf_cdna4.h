@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define NF_ABI_VERSION 5
+#define NF_ABI_VERSION 6
 
 /* element types */
 enum { NF_F32 = 0, NF_F16 = 1, NF_BF16 = 2 };
@@ -144,7 +144,10 @@ int nf_table_adam_step(void* table, int table_dtype, float* master, float* grad,
 /* Fully fused MLP.  x [rows, d_in] (row stride x_stride) in x_dtype, y [rows, d_out] (row stride y_stride) in `dtype`;
  * w_in [d_hidden, d_in], w_hid [(depth-1)*d_hidden, d_hidden], w_out [d_out, d_hidden], all
  * row-contiguous in `dtype`; biases b_in [d_hidden], b_hid [depth-1, d_hidden], b_out [d_out]
- * may each be NULL.  depth >= 1 counts the input layer plus the hidden layers. */
+ * may each be NULL.  depth >= 1 counts the input layer plus the hidden layers.
+ * dtype NF_F16 / NF_BF16: 16-bit operands, float32 accumulation (x_dtype may be the other 16-bit type).
+ * dtype NF_F32 (x_dtype NF_F32 too): float32 storage, operands and accumulation (v_mfma_f32_16x16x4_f32) -- the
+ * reference's float32 case, fully_fused_mlp/kernel.py:17-47 (TF32 products there: same range, shorter mantissa). */
 int nf_mlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_stride, const void* w_in, const void* b_in,
                const void* w_hid, const void* b_hid, const void* w_out, const void* b_out, int64_t rows, int d_in,
                int d_hidden, int d_out, int depth, int act, int dtype, int x_dtype, void* workspace,
@@ -156,8 +159,10 @@ int nf_mlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_stride, const
  * device memory of at least this many bytes; contents are scratch).  0: one launch, workspace may be NULL.  Without
  * the workspace nf_mlp_bwd falls back to a slower one-launch kernel where the network fits it (NF_EINVAL otherwise).  (The
  * reference loops over the layers inside one kernel, triton_helpers/layers/fully_fused_mlp/kernel.py:139-178,
- * 264-304, re-reading every weight per program.) */
-int64_t nf_mlp_workspace_bytes(int64_t rows, int d_hidden, int depth, int act, int backward);
+ * 264-304, re-reading every weight per program.)
+ * dtype NF_F32: the forward needs none; the backward keeps every hidden layer's float32 pre-activation and always
+ * needs depth * rows * d_hidden * 4 bytes plus 8.5 MB of partial weight gradients. */
+int64_t nf_mlp_workspace_bytes(int64_t rows, int d_hidden, int depth, int act, int backward, int dtype);
 
 /* x_dtype may be the other 16-bit type than `dtype` (an fp16 encoder output feeding bf16 weights): the rows are
  * converted while they are loaded, as a cast kernel in front would, and the backward writes dx in x_dtype.

@@ -72,16 +72,27 @@ def test_mlp_workspace_sizes_without_gpu():
     rows = 1000
     buf = (rows * 64 * 2 + 255) // 256 * 256
     for depth in (1, 2, 4):
-        assert lib.nf_mlp_workspace_bytes(rows, 64, depth, relu, 0) == 0
-        assert lib.nf_mlp_workspace_bytes(rows, 64, depth, relu, 1) == 0
-    assert lib.nf_mlp_workspace_bytes(rows, 64, 2, silu, 1) == 0
-    assert lib.nf_mlp_workspace_bytes(rows, 64, 8, relu, 0) == 0           # 9 layers of weights fit LDS
-    assert lib.nf_mlp_workspace_bytes(rows, 64, 8, relu, 1) == (1 + 2) * buf  # 9 linear layers = 5 + 4
-    assert lib.nf_mlp_workspace_bytes(rows, 64, 5, silu, 1) == (1 + 2) * buf  # 6 linear layers = 3 + 3
-    assert lib.nf_mlp_workspace_bytes(rows, 64, 32, relu, 0) == 2 * buf
-    assert lib.nf_mlp_workspace_bytes(rows, 32, 2, relu, 1) == 0
-    assert lib.nf_mlp_workspace_bytes(rows, 32, 8, relu, 1) == (2 + 2) * ((rows * 32 * 2 + 255) // 256 * 256)  # 9 linear layers = 3 + 3 + 3
-    assert lib.nf_mlp_workspace_bytes(0, 64, 32, relu, 1) == 0
+        assert lib.nf_mlp_workspace_bytes(rows, 64, depth, relu, 0, _lib.NF_BF16) == 0
+        assert lib.nf_mlp_workspace_bytes(rows, 64, depth, relu, 1, _lib.NF_BF16) == 0
+    assert lib.nf_mlp_workspace_bytes(rows, 64, 2, silu, 1, _lib.NF_BF16) == 0
+    assert lib.nf_mlp_workspace_bytes(rows, 64, 8, relu, 0, _lib.NF_BF16) == 0           # 9 layers of weights fit LDS
+    assert lib.nf_mlp_workspace_bytes(rows, 64, 8, relu, 1, _lib.NF_BF16) == (1 + 2) * buf  # 9 linear layers = 5 + 4
+    assert lib.nf_mlp_workspace_bytes(rows, 64, 5, silu, 1, _lib.NF_BF16) == (1 + 2) * buf  # 6 linear layers = 3 + 3
+    assert lib.nf_mlp_workspace_bytes(rows, 64, 32, relu, 0, _lib.NF_BF16) == 2 * buf
+    assert lib.nf_mlp_workspace_bytes(rows, 32, 2, relu, 1, _lib.NF_BF16) == 0
+    assert lib.nf_mlp_workspace_bytes(rows, 32, 8, relu, 1, _lib.NF_BF16) == (2 + 2) * ((rows * 32 * 2 + 255) // 256 * 256)  # 9 linear layers = 3 + 3 + 3
+    assert lib.nf_mlp_workspace_bytes(0, 64, 32, relu, 1, _lib.NF_BF16) == 0
+    # float32: nothing in the forward, every hidden layer's float32 pre-activation in the backward (+ partial dW / db)
+    part = 512 * (64 * 64 + 64) * 4
+    assert lib.nf_mlp_workspace_bytes(rows, 64, 32, relu, 0, _lib.NF_F32) == 0
+    assert lib.nf_mlp_workspace_bytes(rows, 64, 2, relu, 1, _lib.NF_F32) == 2 * rows * 64 * 4 + part
+    assert lib.nf_mlp_workspace_bytes(rows, 16, 3, silu, 1, _lib.NF_F32) == 3 * rows * 16 * 4 + part
+    rc = lib.nf_mlp_bwd(1, 32, 1, 16, None, 32, 1, None, 1, None, 1, None, 1, None, 1, None, 1, None,
+                        rows, 32, 64, 16, 2, relu, _lib.NF_F32, _lib.NF_F32, None, 0, None)
+    assert rc == -1 and b"workspace" in lib.nf_last_error()
+    # float32 parameters with 16-bit rows (or the reverse) are refused
+    rc = lib.nf_mlp_fwd(1, 32, 1, 16, 1, None, 1, None, 1, None, rows, 32, 64, 16, 2, relu, _lib.NF_F32, _lib.NF_F16, None, 0, None)
+    assert rc == -2 and b"x_dtype" in lib.nf_last_error()
     # a deep call without the workspace is refused before anything is launched
     rc = lib.nf_mlp_bwd(1, 32, 1, 16, None, 32, 1, None, 1, None, 1, None, 1, None, 1, None, 1, None,
                         rows, 32, 64, 16, 8, relu, _lib.NF_BF16, _lib.NF_BF16, None, 0, None)

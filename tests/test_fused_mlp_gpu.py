@@ -243,7 +243,7 @@ def test_backward_without_workspace_takes_the_one_launch_kernel():
         torch.cuda.synchronize()
         return dx, g
 
-    n = lib.nf_mlp_workspace_bytes(rows, H, depth, relu, 1)
+    n = lib.nf_mlp_workspace_bytes(rows, H, depth, relu, 1, code)
     assert n > 0
     dx_a, g_a = run(torch.empty(n, dtype=torch.uint8, device=DEV))
     dx_b, g_b = run(None)
@@ -261,11 +261,20 @@ def test_backward_without_workspace_takes_the_one_launch_kernel():
 @pytest.mark.parametrize("act", ["relu", "silu", "none"])
 @pytest.mark.parametrize("shape,d_in,d_hidden,d_out,depth", [((3, 40), 1, 32, 5, 1), ((2, 2), 8, 16, 4, 3), ((1, 1000), 32, 64, 16, 2)])
 def test_float32_storage(shape, d_in, d_hidden, d_out, depth, act):
-    """float32 tensors: the reference multiplies them in TF32 (10-bit mantissa) and its tests allow 1e-3 forward,
-    1e-2 backward (tests/test_layers/test_fully_fused_mlp.py:42-46, 235-239); this build multiplies float16 roundings
-    of the same values with float32 accumulation and returns float32.  Checked against the float32 oracle on the
-    unrounded values at those tolerances (relative to each tensor's scale), and the results must be float32."""
+    """float32 tensors with ``set_float32_operands("float16")``: the reference multiplies them in TF32 (10-bit
+    mantissa) and its tests allow 1e-3 forward, 1e-2 backward (tests/test_layers/test_fully_fused_mlp.py:42-46,
+    235-239); this mode multiplies float16 roundings of the same values with float32 accumulation and returns
+    float32.  Checked against the float32 oracle on the unrounded values at those tolerances (relative to each
+    tensor's scale), and the results must be float32.  (The default float32 mode: test_fused_mlp_f32_gpu.py.)"""
     mk = _mk()
+    previous = mk.set_float32_operands("float16")
+    try:
+        _float32_storage_half_operands(mk, shape, d_in, d_hidden, d_out, depth, act)
+    finally:
+        mk.set_float32_operands(previous)
+
+
+def _float32_storage_half_operands(mk, shape, d_in, d_hidden, d_out, depth, act):
     torch.manual_seed(0)
     p = _params(d_in, d_hidden, d_out, depth, True, torch.float32)
     x = torch.randn(*shape, d_in)

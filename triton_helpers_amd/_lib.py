@@ -14,7 +14,7 @@ import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "libnf_cdna4.so"
 
-NF_ABI_VERSION = 5
+NF_ABI_VERSION = 6
 NF_F32, NF_F16, NF_BF16 = 0, 1, 2
 NF_ACT = {"none": 0, "relu": 1, "silu": 2, "relu2": 3, "gelu": 4}
 NF_MAX_LEVELS = 32
@@ -100,7 +100,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.nf_mlp_fwd.restype = c_int
     lib.nf_mlp_fwd.argtypes = [P, I64, P, I64, P, P, P, P, P, P, I64, I, I, I, I, I, I, I, P, I64, P]
     lib.nf_mlp_workspace_bytes.restype = I64
-    lib.nf_mlp_workspace_bytes.argtypes = [I64, I, I, I, I]
+    lib.nf_mlp_workspace_bytes.argtypes = [I64, I, I, I, I, I]
     lib.nf_mlp_bwd.restype = c_int
     lib.nf_mlp_bwd.argtypes = [P, I64, P, I64, P, I64, P, P, P, P, P, P, P, P, P, P, P, P, I64, I, I, I, I, I, I, I, P, I64, P]
     lib.nf_revmlp_fwd.restype = c_int

@@ -130,4 +130,15 @@ int launch_mlp_bwdn(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
 // 2^31 bytes) on eight waves per workgroup (fused_mlp_bwd2_w8.hip).  *handled = false: not that shape.
 int launch_mlp_bwd2_w8(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
 
+
+// float32 storage and float32 products (fused_mlp_f32.hip).  The backward needs mlp32_bwd_workspace_bytes of scratch.
+size_t mlp32_bwd_workspace_bytes(int64_t rows, int d_hidden, int depth);
+int mlp32_fwd(const float* x, int64_t x_stride, float* y, int64_t y_stride, const float* w_in, const float* b_in,
+              const float* w_hid, const float* b_hid, const float* w_out, const float* b_out, int64_t rows, int d_in,
+              int d_hidden, int d_out, int depth, int act, hipStream_t s);
+int mlp32_bwd(const float* x, int64_t x_stride, const float* dy, int64_t dy_stride, float* dx, int64_t dx_stride,
+              const float* w_in, const float* b_in, const float* w_hid, const float* b_hid, const float* w_out, float* dw_in,
+              float* db_in, float* dw_hid, float* db_hid, float* dw_out, float* db_out, int64_t rows, int d_in, int d_hidden,
+              int d_out, int depth, int act, void* workspace, int64_t workspace_bytes, hipStream_t s);
+
 }  // namespace nf

@@ -531,8 +531,7 @@ static int validate(int64_t rows, int d_in, int d_hidden, int d_out, int depth, 
              "d_hidden=%d must be 16, 32 or 64", d_hidden);
   NF_REQUIRE(depth >= 1, NF_EINVAL, "depth=%d must be >= 1", depth);
   NF_REQUIRE(act >= NF_ACT_NONE && act <= NF_ACT_GELU, NF_EINVAL, "unknown activation %d", act);
-  NF_REQUIRE(dtype == NF_F16 || dtype == NF_BF16, NF_EUNSUPPORTED,
-             "dtype code %d: the fused MLP kernels take float16 or bfloat16 storage", dtype);
+  NF_REQUIRE(dtype_ok(dtype), NF_EINVAL, "unknown dtype code %d", dtype);
   return 0;
 }
 
@@ -730,8 +729,9 @@ static void set_rows(MlpArgs& g, const uint16_t* x, int64_t x_stride, uint16_t* 
 
 using namespace nf;
 
-extern "C" int64_t nf_mlp_workspace_bytes(int64_t rows, int d_hidden, int depth, int act, int backward) {
+extern "C" int64_t nf_mlp_workspace_bytes(int64_t rows, int d_hidden, int depth, int act, int backward, int dtype) {
   if (rows <= 0 || depth < 1 || d_hidden < 1) return 0;
+  if (dtype == NF_F32) return backward ? (int64_t)mlp32_bwd_workspace_bytes(rows, d_hidden, depth) : 0;
   const int n_linear = depth + 1;
   const int n = (int)plan_launches(n_linear, backward ? bwd_max_linear(d_hidden, act) : fwd_max_linear(d_hidden)).size() - 1;
   if (n <= 1) return 0;
@@ -744,11 +744,16 @@ extern "C" int nf_mlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y_st
                           int d_in, int d_hidden, int d_out, int depth, int act, int dtype, int x_dtype, void* workspace,
                           int64_t workspace_bytes, void* stream) {
   if (int rc = validate(rows, d_in, d_hidden, d_out, depth, act, dtype)) return rc;
-  NF_REQUIRE(x_dtype == NF_F16 || x_dtype == NF_BF16, NF_EUNSUPPORTED, "x_dtype code %d: float16 or bfloat16", x_dtype);
+  NF_REQUIRE(dtype == NF_F32 ? x_dtype == NF_F32 : (x_dtype == NF_F16 || x_dtype == NF_BF16), NF_EUNSUPPORTED,
+             "x_dtype code %d with dtype code %d: float32 with float32, float16 or bfloat16 with the 16-bit types", x_dtype, dtype);
   if (rows == 0) return 0;
   NF_REQUIRE(x && y && w_in && w_out, NF_EINVAL, "NULL pointer argument");
   NF_REQUIRE(depth == 1 || w_hid, NF_EINVAL, "w_hid is NULL but depth=%d", depth);
   NF_REQUIRE(x_stride >= d_in && y_stride >= d_out, NF_EINVAL, "row stride smaller than row width");
+  if (dtype == NF_F32)
+    return mlp32_fwd((const float*)x, x_stride, (float*)y, y_stride, (const float*)w_in, (const float*)b_in, (const float*)w_hid,
+                     (const float*)b_hid, (const float*)w_out, (const float*)b_out, rows, d_in, d_hidden, d_out, depth, act,
+                     (hipStream_t)stream);
   MlpArgs a = {};
   a.w_in = (const uint16_t*)w_in; a.b_in = (const uint16_t*)b_in; a.w_hid = (const uint16_t*)w_hid;
   a.b_hid = (const uint16_t*)b_hid; a.w_out = (const uint16_t*)w_out; a.b_out = (const uint16_t*)b_out;
@@ -781,12 +786,18 @@ extern "C" int nf_mlp_bwd(const void* x, int64_t x_stride, const void* dy, int64
                           float* db_out, int64_t rows, int d_in, int d_hidden, int d_out, int depth, int act, int dtype,
                           int x_dtype, void* workspace, int64_t workspace_bytes, void* stream) {
   if (int rc = validate(rows, d_in, d_hidden, d_out, depth, act, dtype)) return rc;
-  NF_REQUIRE(x_dtype == NF_F16 || x_dtype == NF_BF16, NF_EUNSUPPORTED, "x_dtype code %d: float16 or bfloat16", x_dtype);
+  NF_REQUIRE(dtype == NF_F32 ? x_dtype == NF_F32 : (x_dtype == NF_F16 || x_dtype == NF_BF16), NF_EUNSUPPORTED,
+             "x_dtype code %d with dtype code %d: float32 with float32, float16 or bfloat16 with the 16-bit types", x_dtype, dtype);
   if (rows == 0) return 0;
   NF_REQUIRE(x && dy && w_in && w_out && dw_in && dw_out, NF_EINVAL, "NULL pointer argument");
   NF_REQUIRE(depth == 1 || (w_hid && dw_hid), NF_EINVAL, "w_hid / dw_hid is NULL but depth=%d", depth);
   NF_REQUIRE(x_stride >= d_in && dy_stride >= d_out && (dx == nullptr || dx_stride >= d_in), NF_EINVAL,
              "row stride smaller than row width");
+  if (dtype == NF_F32)
+    return mlp32_bwd((const float*)x, x_stride, (const float*)dy, dy_stride, (float*)dx, dx_stride, (const float*)w_in,
+                     (const float*)b_in, (const float*)w_hid, (const float*)b_hid, (const float*)w_out, dw_in, db_in, dw_hid,
+                     db_hid, dw_out, db_out, rows, d_in, d_hidden, d_out, depth, act, workspace, workspace_bytes,
+                     (hipStream_t)stream);
   MlpArgs a = {};
   a.w_in = (const uint16_t*)w_in; a.b_in = (const uint16_t*)b_in; a.w_hid = (const uint16_t*)w_hid;
   a.b_hid = (const uint16_t*)b_hid; a.w_out = (const uint16_t*)w_out; a.b_out = (const uint16_t*)b_out;

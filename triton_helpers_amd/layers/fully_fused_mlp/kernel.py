@@ -11,11 +11,12 @@ Supersets / differences:
   * weight gradients are accumulated in float32 inside the kernel and rounded once
     (the reference sums per-program partials in the storage dtype, kernel.py:599-633);
   * ``fp16_acc`` is accepted and ignored: accumulation is always float32 (MFMA);
-  * storage dtypes of the kernels are float16 and bfloat16 (what autocast produces).  float32 tensors
-    (the reference feeds them to ``tl.dot``, which multiplies in TF32: 10-bit mantissa, float32
-    accumulation) are run with float16 operands -- the same 10-bit mantissa, float32 accumulation;
-    operands beyond +-65504 overflow, which TF32's 8-bit exponent would not -- and the output, ``dx`` and
-    the weight gradients (straight from the float32 accumulators) come back as float32.
+  * float16 and bfloat16 storage (what autocast produces) runs on the 16-bit matrix instructions: the fast path.
+    float32 tensors (the reference feeds them to ``tl.dot``, which multiplies in TF32: float32 range, 10-bit
+    mantissa) run on the float32 matrix instruction: float32 range and mantissa, about a sixth of the 16-bit rate, and
+    a backward scratch of ``depth * rows * d_hidden * 4`` bytes.  ``set_float32_operands("float16")`` trades the
+    range for speed: float32 tensors are then multiplied with float16 operands (the same 10-bit mantissa as TF32,
+    float32 accumulation and results; operands beyond +-65504 overflow).
 """
 from __future__ import annotations
 
@@ -32,6 +33,22 @@ from ... import _lib
 FULLY_FUSED_MAX_DIM: Final = 64
 
 _ACTIVATIONS = ("relu", "relu2", "silu", "none")
+
+_FLOAT32_OPERANDS = "float32"
+
+
+def set_float32_operands(kind: str) -> str:
+    """How float32 tensors are multiplied: ``"float32"`` (default: float32 range and mantissa) or ``"float16"``
+    (float16 operands, float32 accumulation: several times faster, operands limited to +-65504).  Returns the
+    previous setting.  (The counterpart of ``allow_tf32`` for ``tl.dot`` in the reference, kernel.py:17-47.)"""
+    global _FLOAT32_OPERANDS
+    assert kind in ("float32", "float16"), f"float32 operands are 'float32' or 'float16', got {kind!r}"
+    previous, _FLOAT32_OPERANDS = _FLOAT32_OPERANDS, kind
+    return previous
+
+
+def get_float32_operands() -> str:
+    return _FLOAT32_OPERANDS
 
 
 # ---------------------------------------------------------------------------
@@ -87,7 +104,7 @@ def feedforward_bwd_dx(w: Tensor, dz: Tensor, DTYPE: torch.dtype = torch.float32
 def _check_storage(x: Tensor, w_in: Tensor, *others: Optional[Tensor]) -> None:
     """Parameters share one dtype.  With 16-bit parameters ``x`` may be in the other 16-bit dtype (an fp16 encoder
     output in front of bf16 weights): the kernels convert it while loading, exactly as a cast in front would.
-    float32 runs as a whole (``x`` and parameters) with float16 operands."""
+    float32 runs as a whole (``x`` and parameters)."""
     if w_in.dtype == torch.float32:
         assert x.dtype == torch.float32, f"float32 parameters take a float32 input, got {x.dtype}"
     else:
@@ -119,9 +136,10 @@ def _c(t: Optional[Tensor]) -> Optional[Tensor]:
     return None if t is None else (t if t.is_contiguous() else t.contiguous())
 
 
-def _workspace(lib, rows2d: Tensor, d_hidden: int, depth: int, activation: str, backward: bool):
-    """Scratch for networks that run as several launches (none for the usual depths)."""
-    n = lib.nf_mlp_workspace_bytes(rows2d.shape[0], d_hidden, depth, _lib.NF_ACT[activation], int(backward))
+def _workspace(lib, rows2d: Tensor, d_hidden: int, depth: int, activation: str, backward: bool, dtype: torch.dtype):
+    """Scratch for networks that run as several launches (none for the usual depths) and for the float32 backward."""
+    n = lib.nf_mlp_workspace_bytes(rows2d.shape[0], d_hidden, depth, _lib.NF_ACT[activation], int(backward),
+                                   _lib.dtype_code(dtype))
     if n == 0:
         return None, 0
     return torch.empty(n, dtype=torch.uint8, device=rows2d.device), n
@@ -171,7 +189,7 @@ class _fully_fused_mlp(Function):
         ctx.activation = activation
         ctx.fp16_acc = fp16_acc
         ctx.depth = depth
-        wide = w_in.dtype == torch.float32
+        ctx.wide = wide = w_in.dtype == torch.float32 and _FLOAT32_OPERANDS == "float16"
         if wide:  # float16 operands, float32 accumulation and results
             x, w_in, b_in, w_out, b_out, w_hid, b_hid = (_half(t) for t in (x, w_in, b_in, w_out, b_out, w_hid, b_hid))
         w_in, b_in, w_out, b_out, w_hid, b_hid = (_c(t) for t in (w_in, b_in, w_out, b_out, w_hid, b_hid))
@@ -179,7 +197,7 @@ class _fully_fused_mlp(Function):
         o = x.new_empty((B, L, D_out), dtype=w_in.dtype)
         o2 = o.view(-1, D_out)
         lib = _lib.load()
-        ws, ws_bytes = _workspace(lib, x2, D_hidden, depth, activation, backward=False)
+        ws, ws_bytes = _workspace(lib, x2, D_hidden, depth, activation, False, w_in.dtype)
         rc = lib.nf_mlp_fwd(
             x2.data_ptr(), x2.stride(0), o2.data_ptr(), o2.stride(0),
             w_in.data_ptr(), _lib.ptr(b_in), _lib.ptr(w_hid), _lib.ptr(b_hid), w_out.data_ptr(), _lib.ptr(b_out),
@@ -197,19 +215,19 @@ class _fully_fused_mlp(Function):
         B, L, D_in = x.shape
         D_hidden = w_in.shape[0]
         D_out = w_out.shape[0]
-        wide = w_in.dtype == torch.float32
+        wide = ctx.wide
         if wide:
             x, w_in, b_in, w_out, b_out, w_hid, b_hid = (_half(t) for t in (x, w_in, b_in, w_out, b_out, w_hid, b_hid))
         if do.dtype != w_in.dtype:
             do = do.to(w_in.dtype)
-        if x.dtype != w_in.dtype and not (ctx.depth == 2 and D_hidden > 32 and ctx.activation == "relu"):
+        if x.dtype != w_in.dtype and not (w_in.dtype != torch.float32 and ctx.depth == 2 and D_hidden > 32 and ctx.activation == "relu"):
             x = x.to(w_in.dtype)  # only the one-hidden-layer ReLU backward converts on the fly
         do2 = _rows2d(do, D_out)
         need_dx = ctx.needs_input_grad[0]
         grads = _lib.GradBuffers(w_in, b_in, w_out, b_out, w_hid, b_hid)
         p_dw_in, p_db_in, p_dw_out, p_db_out, p_dw_hid, p_db_hid = grads.pointers()
         lib = _lib.load()
-        ws, ws_bytes = _workspace(lib, do2, D_hidden, ctx.depth, ctx.activation, backward=True)
+        ws, ws_bytes = _workspace(lib, do2, D_hidden, ctx.depth, ctx.activation, True, w_in.dtype)
         while True:
             x2 = _rows2d(x, D_in)
             dx = x.new_empty(x.shape) if need_dx else None
