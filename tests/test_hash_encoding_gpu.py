@@ -287,11 +287,22 @@ def test_backward_binned_two_dimensions(N, T, L, lo, hi, do_dtype):
 
 @pytest.mark.parametrize("do_dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("N,D,F,T,L,lo,hi", [(40000, 3, 4, 2**14, 16, 16, 512), (35001, 3, 8, 2**16, 8, 16, 1024),
-                                            (40000, 2, 4, 5000, 4, 8, 256), (33000, 3, 6, 2**12, 4, 8, 64)])
+                                            (40000, 2, 4, 5000, 4, 8, 256), (33000, 3, 6, 2**12, 4, 8, 64),
+                                            # one feature, and odd numbers of them: the last feature goes alone
+                                            (40000, 3, 1, 2**14, 16, 16, 512), (33000, 3, 3, 2**12, 4, 8, 64),
+                                            (35001, 2, 5, 5000, 4, 8, 256), (33000, 3, 1, 2**19, 16, 16, 7006),
+                                            # rows of an odd number of elements are not 4-byte aligned: scattered atomics
+                                            (33000, 3, 3, 2**12, 5, 8, 64)])
 def test_backward_binned_wide_rows(N, D, F, T, L, lo, hi, do_dtype):
-    """Tables with 4, 6 or 8 features per row: the binned backward takes the features two at a time (one fill and
+    """Tables with 1 to 8 features per row: the binned backward takes the features two at a time (one fill and
     one accumulation per pair).  Against the oracle and the scattered-atomic kernel."""
     hk = _hk()
+    from triton_helpers_amd import _lib
+    from triton_helpers_amd.layers.hash_encoding.helpers import level_geometry
+
+    # every one of these geometries has a sorted-records plan (the kernel is taken when the rows are 4-byte aligned)
+    geom = level_geometry(T, L, D, F, lo, hi)
+    assert _lib.load().nf_hash_encode_bwd_workspace_bytes(N, geom, _lib.dtype_code(do_dtype), 0) > 0
     torch.manual_seed(5)
     x = torch.rand(N, D)
     x[0] = 0.0

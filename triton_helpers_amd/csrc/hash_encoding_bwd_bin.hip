@@ -1,4 +1,4 @@
-// Hash-encoding backward by binning (D = 2 or 3, an even number of features taken two at a time).
+// Hash-encoding backward by binning (D = 2 or 3; features taken two at a time, the last one alone when their number is odd).
 //
 // Every (point, level, corner) contributes  w * dout[n, 2l .. 2l+1]  to one table row.  Scattering these with
 // global atomics is bound by the chip's atomic request rate; accumulating them in LDS needs the contributions to
@@ -415,7 +415,15 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
     const uint32_t* ldelta = delta + bp.binbase[l];
     uint32_t packed = 0u;  // 16-bit: the pair; float32: the point's index in the workgroup (its pair goes to gtab)
     if (G32) {
-      const uint2 pair = valid ? *reinterpret_cast<const uint2*>(grow32 + l * feat + f0) : make_uint2(0u, 0u);
+      uint2 pair = make_uint2(0u, 0u);
+      if (valid) {
+        if (feat & 1) {  // an odd row width: the pair is not 8-byte aligned, and the last feature has no partner
+          pair.x = __float_as_uint(grow32[l * feat + f0]);
+          if (f0 + 1 < feat) pair.y = __float_as_uint(grow32[l * feat + f0 + 1]);
+        } else {
+          pair = *reinterpret_cast<const uint2*>(grow32 + l * feat + f0);
+        }
+      }
       gtab[tid] = pair;
       packed = (uint32_t)tid;
       // largest |g| of the level: positive float patterns order like integers
@@ -428,7 +436,13 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
 #pragma unroll
         for (int i = 1; i < 16; ++i) packed = (l == i) ? gr[i] : packed;
       } else if (valid) {
-        packed = grow[(l * feat + f0) >> 1];
+        if (feat & 1) {  // an odd row width: 16-bit loads, and the last feature has no partner
+          const uint16_t* g16 = reinterpret_cast<const uint16_t*>(grow);
+          packed = g16[l * feat + f0];
+          if (f0 + 1 < feat) packed |= (uint32_t)g16[l * feat + f0 + 1] << 16;
+        } else {
+          packed = grow[(l * feat + f0) >> 1];
+        }
       }
       // largest |g| of the level: positive 16-bit float patterns order like integers
       const uint32_t pk = packed & 0x7fff7fffu;
@@ -659,8 +673,8 @@ struct LevelGroups {
   int operator[](size_t k) const { return first[k]; }
 };
 static bool bin_groups(int64_t N, const nf_hash_geom* geom, LevelGroups* groups) {
-  // features are taken two at a time (one pass of fill + accumulate per pair)
-  if ((geom->dims != 3 && geom->dims != 2) || geom->feat < 2 || geom->feat % 2 != 0 || N <= 0) return false;
+  // features are taken two at a time (one pass of fill + accumulate per pair; the last feature of an odd count alone)
+  if ((geom->dims != 3 && geom->dims != 2) || geom->feat < 1 || N <= 0) return false;
   groups->n = 0;
   groups->first[0] = 0;
   int nb_total = 0;
