@@ -131,6 +131,9 @@ int launch_mlp_bwdn(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
 int launch_mlp_bwd2_w8(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
 
 
+// The forward of that shape (fused_mlp_fwd2.hip).  *handled = false: not that shape, nothing was launched.
+int launch_mlp_fwd2(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
+
 // float32 storage and float32 products (fused_mlp_f32.hip).  The backward needs mlp32_bwd_workspace_bytes of scratch.
 size_t mlp32_bwd_workspace_bytes(int64_t rows, int d_hidden, int depth);
 int mlp32_fwd(const float* x, int64_t x_stride, float* y, int64_t y_stride, const float* w_in, const float* b_in,

@@ -643,6 +643,9 @@ static int dispatch_bwd(const MlpArgs& a, hipStream_t s) {
 // last boundary, keeping each boundary's rows (rows * d_hidden * 2 bytes), then walks the launches last to first.
 
 static int fwd_one(const MlpArgs& a, int dtype, hipStream_t s) {
+  bool handled = false;
+  const int rc = launch_mlp_fwd2(a, dtype, s, &handled);
+  if (rc != 0 || handled) return rc;
   return dtype == NF_BF16 ? dispatch_fwd<BF16>(a, s) : dispatch_fwd<F16>(a, s);
 }
 
