@@ -573,43 +573,61 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const typena
   const float s_lo = nonfinite ? 0.0f : ldexpf(1.0f, se / 2), s_hi = ldexpf(1.0f, se - se / 2) * (1.0f / (float)W_MAX);
   for (uint32_t i = tid; i < 2u * nrows; i += ACC_THREADS) acc_tile[(i & 1u) * BIN_ROWS + (i >> 1)] = 0ull;
   lds_barrier();
-  // the next round's records are loaded before this round's adds
-  Rec q[ACC_INFLIGHT];
+  // The task's records behind a buffer descriptor that ends with them: reads past the end return zeros (zero weights),
+  // so the loop carries no bounds tests.
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<Rec*>(records + task.y), 0,
+                                                                      (int)((task.z - task.y) * (uint32_t)sizeof(Rec)), 0x00020000);
+  auto load_rec = [&](uint32_t at) {  // record `at` of the task
+    Rec r;
+    if constexpr (sizeof(Rec) == 12) {
+      typedef unsigned int v3u __attribute__((ext_vector_type(3)));
+      const v3u v = __builtin_amdgcn_raw_buffer_load_b96(rs, at * 12u, 0, 0);
+      r.x = v[0]; r.y = v[1]; r.z = v[2];
+    } else {
+      typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+      const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rs, at * 16u, 0, 0);
+      r.x = v[0]; r.y = v[1]; r.z = v[2]; r.w = v[3];
+    }
+    return r;
+  };
+  const uint32_t n_rec = task.z - task.y;
+  // the next round's records are loaded before this round's adds; a level with an inf or a nan in its gradient only
+  // marks the rows it touches (its own copy of the loop, so that the usual one has no test per record)
+  auto accumulate = [&](auto nonfinite_c) {
+    constexpr bool NONFINITE = decltype(nonfinite_c)::value;
+    Rec q[ACC_INFLIGHT];
 #pragma unroll
-  for (int k = 0; k < ACC_INFLIGHT; ++k) {
-    const uint32_t i = task.y + k * ACC_THREADS + tid;
-    q[k] = i < task.z ? records[i] : BinRec<GT>::zero();
-  }
-  for (uint32_t i0 = task.y; i0 < task.z; i0 += ACC_THREADS * ACC_INFLIGHT) {
-    uint32_t slot[ACC_INFLIGHT][2];
-    int32_t f[ACC_INFLIGHT][4];
+    for (int k = 0; k < ACC_INFLIGHT; ++k) q[k] = load_rec(k * ACC_THREADS + tid);
+    for (uint32_t i0 = 0; i0 < n_rec; i0 += ACC_THREADS * ACC_INFLIGHT) {
+      uint32_t slot[ACC_INFLIGHT][2];
+      int32_t f[ACC_INFLIGHT][4];
 #pragma unroll
-    for (int k = 0; k < ACC_INFLIGHT; ++k) {
-      const float g0 = BinRec<GT>::g0(q[k]) * s_lo, g1 = BinRec<GT>::g1(q[k]) * s_lo;
-      // records past the end: zero weights
-      const float w0 = (float)(q[k].y & W_MAX), w1 = (float)((q[k].x >> 26) << 13 | q[k].y >> W_BITS);
-      slot[k][0] = q[k].x & BIN_MASK;
-      slot[k][1] = (q[k].x >> BIN_ROWS_LOG2) & BIN_MASK;
-      f[k][0] = __float2int_rn(w0 * g0 * s_hi);
-      f[k][1] = __float2int_rn(w0 * g1 * s_hi);
-      f[k][2] = __float2int_rn(w1 * g0 * s_hi);
-      f[k][3] = __float2int_rn(w1 * g1 * s_hi);
-      if (nonfinite) {  // only mark the rows the level touches
-        f[k][0] = f[k][1] = w0 != 0.0f;
-        f[k][2] = f[k][3] = w1 != 0.0f;
+      for (int k = 0; k < ACC_INFLIGHT; ++k) {
+        const float g0 = BinRec<GT>::g0(q[k]) * s_lo, g1 = BinRec<GT>::g1(q[k]) * s_lo;
+        const float w0 = (float)(q[k].y & W_MAX), w1 = (float)((q[k].x >> 26) << 13 | q[k].y >> W_BITS);
+        slot[k][0] = q[k].x & BIN_MASK;
+        slot[k][1] = (q[k].x >> BIN_ROWS_LOG2) & BIN_MASK;
+        if constexpr (NONFINITE) {
+          f[k][0] = f[k][1] = w0 != 0.0f;
+          f[k][2] = f[k][3] = w1 != 0.0f;
+        } else {
+          f[k][0] = __float2int_rn(w0 * g0 * s_hi);
+          f[k][1] = __float2int_rn(w0 * g1 * s_hi);
+          f[k][2] = __float2int_rn(w1 * g0 * s_hi);
+          f[k][3] = __float2int_rn(w1 * g1 * s_hi);
+        }
       }
+#pragma unroll
+      for (int k = 0; k < ACC_INFLIGHT; ++k) q[k] = load_rec(i0 + ACC_THREADS * ACC_INFLIGHT + k * ACC_THREADS + tid);
+#pragma unroll
+      for (int k = 0; k < ACC_INFLIGHT; ++k)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (f[k][j]) atomicAdd(acc_tile + (uint32_t)(j & 1) * BIN_ROWS + slot[k][j >> 1], (unsigned long long)(long long)f[k][j]);
     }
-#pragma unroll
-    for (int k = 0; k < ACC_INFLIGHT; ++k) {
-      const uint32_t i = i0 + ACC_THREADS * ACC_INFLIGHT + k * ACC_THREADS + tid;
-      q[k] = i < task.z ? records[i] : BinRec<GT>::zero();
-    }
-#pragma unroll
-    for (int k = 0; k < ACC_INFLIGHT; ++k)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (f[k][j]) atomicAdd(acc_tile + (uint32_t)(j & 1) * BIN_ROWS + slot[k][j >> 1], (unsigned long long)(long long)f[k][j]);
-  }
+  };
+  if (nonfinite) accumulate(std::true_type{});
+  else accumulate(std::false_type{});
   lds_barrier();
   float* dst = dtable + (g.row_offset[l] + (int64_t)row0) * feat + f0;  // features f0, f0 + 1 of the bin's rows
   const float qnan = __uint_as_float(0x7fc00000u);
