@@ -487,3 +487,42 @@ def test_relu2_gradients_far_above_unit_scale():
     assert not bool(((y.view(-1, d_out).cpu().float() - ref).abs() > floor + RTOL * ref.abs()).any())
     for k in ("w_in", "w_out", "w_hid"):
         _close(leaves[k].grad, want["d" + k], "d" + k, scale_rel=True)
+
+
+@pytest.mark.parametrize("rows,d_in,d_out,bias,dtype,x_other,pad", [
+    (1, 32, 16, False, torch.bfloat16, False, 0),
+    (33, 4, 4, True, torch.float16, False, 4),
+    (383, 12, 8, False, torch.bfloat16, True, 8),
+    (385, 20, 12, True, torch.float16, True, 0),
+    (4097, 28, 16, True, torch.bfloat16, True, 4),
+    (70001, 32, 4, False, torch.bfloat16, False, 8),
+    (200003, 24, 16, True, torch.float16, False, 0),
+])
+def test_decoder_shape_kernels(rows, d_in, d_out, bias, dtype, x_other, pad):
+    """d_in <= 32 -> 64 -> 64 -> d_out <= 16 with ReLU takes kernels of its own in both directions (twelve / eight waves per
+    workgroup, rows behind buffer descriptors): row counts around the 32-row chunk and the 384 / 256 rows of a workgroup's
+    pass, widths that are multiples of four, x as a column slice of a wider tensor and stored in the other 16-bit type,
+    with and without biases."""
+    mk = _mk()
+    xdt = dtype if not x_other else (torch.float16 if dtype == torch.bfloat16 else torch.bfloat16)
+    torch.manual_seed(rows)
+    p = _params(d_in, 64, d_out, 2, bias, dtype, seed=rows)
+    xs = torch.randn(1, rows, d_in + pad).to(xdt)
+    dy = torch.randn(1, rows, d_out).to(dtype)
+    xr = xs[..., :d_in].to(dtype)  # what a cast in front of the kernel would hand over
+    args = (p["w_in"], p["b_in"], p["w_out"], p["b_out"], p["w_hid"], p["b_hid"], "relu")
+    want_y = M.mlp_forward(xr.float().reshape(-1, d_in), *args, round_to=dtype)
+    want = M.mlp_backward(xr.reshape(-1, d_in), dy.view(-1, d_out), *args, round_to=dtype)
+    leaves = {k: (None if v is None else v.to(DEV).requires_grad_(True)) for k, v in p.items()}
+    xsd = xs.to(DEV).requires_grad_(True)
+    y = mk.fully_fused_mlp(xsd[..., :d_in], leaves["w_in"], leaves["b_in"], leaves["w_out"], leaves["b_out"], leaves["w_hid"], leaves["b_hid"], "relu")
+    assert y.dtype == dtype
+    _close(y.view(-1, d_out), want_y, "y")
+    y.backward(dy.to(DEV))
+    assert xsd.grad.dtype == xdt
+    if pad:
+        assert float(xsd.grad[..., d_in:].abs().max()) == 0.0
+    _close(xsd.grad[..., :d_in].reshape(-1, d_in), want["dx"], "dx", outliers=1e-3)
+    for k in ("w_in", "b_in", "w_out", "b_out", "w_hid", "b_hid"):
+        if leaves[k] is not None:
+            _close(leaves[k].grad, want["d" + k], "d" + k, scale_rel=True)
