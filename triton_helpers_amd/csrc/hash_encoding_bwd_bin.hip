@@ -305,6 +305,7 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t x, uint32_t* w
 __global__ __launch_bounds__(1024) void hash_bwd_bin_offsets_k(const uint32_t* hist, uint32_t* cursor, uint32_t* n_tasks,
                                                                uint4* tasks, int NB, uint32_t max_tasks) {
   __shared__ uint32_t wave_sums[16];
+  __shared__ uint32_t first_task[1025], bin_start[1024], bin_count[1024];  // of the 1024 bins of a pass
   uint32_t rec_run = 0, task_run = 0;
   for (int b0 = 0; b0 < NB; b0 += 1024) {
     const int b = b0 + (int)threadIdx.x;
@@ -312,18 +313,31 @@ __global__ __launch_bounds__(1024) void hash_bwd_bin_offsets_k(const uint32_t* h
     const uint32_t slices = c <= SLICE_RECORDS ? (c ? 1u : 0u) : (c + SPLIT_RECORDS - 1u) / SPLIT_RECORDS;
     uint32_t rec_total, task_total;
     const uint32_t start = rec_run + block_exclusive_scan(c, wave_sums, &rec_total);
-    const uint32_t t0 = task_run + block_exclusive_scan(slices, wave_sums, &task_total);
-    if (b < NB) {
-      cursor[b] = start;
-      // equal slices, so that no workgroup gets a short tail
-      const uint32_t per = slices ? (c + slices - 1u) / slices : 0u;
-      for (uint32_t s = 0; s < slices; ++s) {
-        uint32_t lo = start + s * per, hi = start + (s + 1u) * per;
-        if (hi > start + c) hi = start + c;
-        if (lo > hi) lo = hi;
-        if (t0 + s < max_tasks) tasks[t0 + s] = make_uint4((uint32_t)b, lo, hi, slices > 1u ? 1u : 0u);
+    const uint32_t t0 = block_exclusive_scan(slices, wave_sums, &task_total);
+    if (b < NB) cursor[b] = start;
+    first_task[threadIdx.x] = t0;
+    bin_start[threadIdx.x] = start;
+    bin_count[threadIdx.x] = c;
+    if (threadIdx.x == 0) first_task[1024] = task_total;
+    __syncthreads();
+    // every task of the pass by a thread of its own (a coarse dense level is one bin cut into a hundred slices): the
+    // task's bin is the last one whose first task is not behind it
+    for (uint32_t t = threadIdx.x; t < task_total; t += 1024) {
+      uint32_t lo_b = 0, hi_b = 1023;
+      while (lo_b < hi_b) {
+        const uint32_t mid = (lo_b + hi_b + 1) >> 1;
+        if (first_task[mid] <= t) lo_b = mid; else hi_b = mid - 1;
       }
+      // bins without records share their first task with the bin behind them: the search lands on the last of the run
+      const uint32_t c_b = bin_count[lo_b], n_sl = first_task[lo_b + 1] - first_task[lo_b], sl = t - first_task[lo_b];
+      // equal slices, so that no workgroup gets a short tail
+      const uint32_t per = (c_b + n_sl - 1u) / n_sl;
+      uint32_t lo = bin_start[lo_b] + sl * per, hi = bin_start[lo_b] + (sl + 1u) * per;
+      if (hi > bin_start[lo_b] + c_b) hi = bin_start[lo_b] + c_b;
+      if (lo > hi) lo = hi;
+      if (task_run + t < max_tasks) tasks[task_run + t] = make_uint4((uint32_t)b0 + lo_b, lo, hi, n_sl > 1u ? 1u : 0u);
     }
+    __syncthreads();
     rec_run += rec_total;
     task_run += task_total;
   }
