@@ -144,7 +144,14 @@ def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def current_stream(device: torch.device) -> int:
+    """Handle of the current stream of ``device`` (the raw accessor saves the Stream object, two microseconds a call)."""
+    if _raw_stream is not None:
+        index = device.index
+        return _raw_stream(torch.cuda.current_device() if index is None else index)
     return torch.cuda.current_stream(device).cuda_stream
 
 

@@ -136,10 +136,18 @@ def _c(t: Optional[Tensor]) -> Optional[Tensor]:
     return None if t is None else (t if t.is_contiguous() else t.contiguous())
 
 
+_workspace_sizes: dict = {}
+
+
 def _workspace(lib, rows2d: Tensor, d_hidden: int, depth: int, activation: str, backward: bool, dtype: torch.dtype):
     """Scratch for networks that run as several launches (none for the usual depths) and for the float32 backward."""
-    n = lib.nf_mlp_workspace_bytes(rows2d.shape[0], d_hidden, depth, _lib.NF_ACT[activation], int(backward),
-                                   _lib.dtype_code(dtype))
+    key = (rows2d.shape[0], d_hidden, depth, activation, backward, dtype)
+    n = _workspace_sizes.get(key)
+    if n is None:
+        n = lib.nf_mlp_workspace_bytes(rows2d.shape[0], d_hidden, depth, _lib.NF_ACT[activation], int(backward),
+                                       _lib.dtype_code(dtype))
+        if len(_workspace_sizes) < 4096:
+            _workspace_sizes[key] = n
     if n == 0:
         return None, 0
     return torch.empty(n, dtype=torch.uint8, device=rows2d.device), n
