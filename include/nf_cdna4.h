@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define NF_ABI_VERSION 6
+#define NF_ABI_VERSION 7
 
 /* element types */
 enum { NF_F32 = 0, NF_F16 = 1, NF_BF16 = 2 };
@@ -176,6 +176,20 @@ int nf_mlp_bwd(const void* x, int64_t x_stride, const void* dy, int64_t dy_strid
                const void* b_out, float* dw_in, float* db_in, float* dw_hid, float* db_hid, float* dw_out,
                float* db_out, int64_t rows, int d_in, int d_hidden, int d_out, int depth, int act, int dtype,
                int x_dtype, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* nf_mlp_bwd with the weight and bias gradients delivered as the optimiser wants them: every dw_ / db_ buffer is in
+ * `dtype`, and is WRITTEN with the sum over all rows, rounded once -- nothing to clear before the call and nothing to
+ * cast after it (the reference's host-side sum(0) of per-program partials in the storage dtype,
+ * triton_helpers/layers/fully_fused_mlp/kernel.py:627-633, in one place).  The workgroups' partial sums are added in a
+ * fixed order, so the same inputs give the same bits on every run.  Built for the decoder shape -- depth == 2,
+ * d_hidden == 64, d_in <= 32, d_out <= 16 (both multiples of 4), ReLU, 8-byte aligned rows -- and NF_EUNSUPPORTED
+ * otherwise, before anything is launched.  workspace: 16-byte aligned, nf_mlp_bwd_rounded_workspace_bytes() bytes. */
+int nf_mlp_bwd_rounded(const void* x, int64_t x_stride, const void* dy, int64_t dy_stride, void* dx, int64_t dx_stride,
+                       const void* w_in, const void* b_in, const void* w_hid, const void* b_hid, const void* w_out,
+                       const void* b_out, void* dw_in, void* db_in, void* dw_hid, void* db_hid, void* dw_out,
+                       void* db_out, int64_t rows, int d_in, int d_hidden, int d_out, int depth, int act, int dtype,
+                       int x_dtype, void* workspace, int64_t workspace_bytes, void* stream);
+int64_t nf_mlp_bwd_rounded_workspace_bytes(int d_in, int d_hidden, int d_out);
 
 /* Reversible MLP of `blocks` additive couplings over rows of width 2*half:
  *   y1 = x1 + F_k(x2),  y2 = x2 + G_k(y1),  F/G(u) = act(u W1^T + b1) W2^T + b2.

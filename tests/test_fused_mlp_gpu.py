@@ -526,3 +526,57 @@ def test_decoder_shape_kernels(rows, d_in, d_out, bias, dtype, x_other, pad):
     for k in ("w_in", "b_in", "w_out", "b_out", "w_hid", "b_hid"):
         if leaves[k] is not None:
             _close(leaves[k].grad, want["d" + k], "d" + k, scale_rel=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("bias", [True, False])
+def test_rounded_weight_gradients_entry_point(dtype, bias):
+    """nf_mlp_bwd_rounded against nf_mlp_bwd on the same inputs: the same dx bit for bit, weight and bias gradients equal to
+    the float32 accumulators rounded once (one unit in the last place for the order of the sums), written into buffers
+    that held garbage, and the same bits on a second call."""
+    from triton_helpers_amd import _lib
+
+    lib = _lib.load()
+    rows, d_in, H, d_out = 50000, 32, 64, 16
+    code = _lib.dtype_code(dtype)
+    relu = _lib.NF_ACT["relu"]
+    p = {k: (None if v is None else v.to(DEV)) for k, v in _params(d_in, H, d_out, 2, bias, dtype, seed=5).items()}
+    torch.manual_seed(5)
+    x = torch.randn(rows, d_in, device=DEV).to(dtype)
+    dy = torch.randn(rows, d_out, device=DEV).to(dtype)
+    stream = _lib.current_stream(x.device)
+    names = ("w_in", "b_in", "w_hid", "b_hid", "w_out", "b_out")
+    acc = {k: (None if p[k] is None else torch.zeros(p[k].shape, dtype=torch.float32, device=DEV)) for k in names}
+    dx_a = torch.empty_like(x)
+    rc = lib.nf_mlp_bwd(x.data_ptr(), d_in, dy.data_ptr(), d_out, dx_a.data_ptr(), d_in,
+                        *(_lib.ptr(p[k]) for k in names), *(_lib.ptr(acc[k]) for k in names),
+                        rows, d_in, H, d_out, 2, relu, code, code, None, 0, stream)
+    _lib.check(rc, "nf_mlp_bwd")
+    n = lib.nf_mlp_bwd_rounded_workspace_bytes(d_in, H, d_out)
+    ws = torch.empty(n, dtype=torch.uint8, device=DEV)
+    runs = []
+    for _ in range(2):
+        out = {k: (None if p[k] is None else torch.full(p[k].shape, float("nan"), dtype=dtype, device=DEV)) for k in names}
+        dx_b = torch.empty_like(x)
+        rc = lib.nf_mlp_bwd_rounded(x.data_ptr(), d_in, dy.data_ptr(), d_out, dx_b.data_ptr(), d_in,
+                                    *(_lib.ptr(p[k]) for k in names), *(_lib.ptr(out[k]) for k in names),
+                                    rows, d_in, H, d_out, 2, relu, code, code, ws.data_ptr(), n, stream)
+        _lib.check(rc, "nf_mlp_bwd_rounded")
+        torch.cuda.synchronize()
+        runs.append((dx_b, out))
+    dx_b, out = runs[0]
+    assert torch.equal(dx_a, dx_b)
+    eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    for k in names:
+        if p[k] is None:
+            continue
+        want = acc[k].to(dtype).float()
+        got = out[k].float()
+        assert torch.isfinite(got).all(), k
+        assert float((got - want).abs().max()) <= eps * float(want.abs().max()), k
+        assert torch.equal(out[k], runs[1][1][k]), f"{k}: two calls differ"
+    # shapes it is not built for are refused before anything runs
+    rc = lib.nf_mlp_bwd_rounded(x.data_ptr(), d_in, dy.data_ptr(), d_out, None, d_in,
+                                *(_lib.ptr(p[k]) for k in names), *(_lib.ptr(out[k]) for k in names),
+                                rows, d_in, H, d_out, 2, _lib.NF_ACT["silu"], code, code, ws.data_ptr(), n, stream)
+    assert rc == _lib.NF_EUNSUPPORTED

@@ -14,7 +14,7 @@ import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "libnf_cdna4.so"
 
-NF_ABI_VERSION = 6
+NF_ABI_VERSION = 7
 NF_F32, NF_F16, NF_BF16 = 0, 1, 2
 NF_ACT = {"none": 0, "relu": 1, "silu": 2, "relu2": 3, "gelu": 4}
 NF_MAX_LEVELS = 32
@@ -41,6 +41,8 @@ EXPORTS = (
     "nf_mlp_fwd",
     "nf_mlp_bwd",
     "nf_mlp_workspace_bytes",
+    "nf_mlp_bwd_rounded",
+    "nf_mlp_bwd_rounded_workspace_bytes",
     "nf_revmlp_fwd",
     "nf_revmlp_bwd",
 )
@@ -99,6 +101,10 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.nf_table_adam_step.argtypes = [P, I, P, P, P, P, I64, I64, c_float, c_float, c_float, c_float, c_float, c_float, I, P]
     lib.nf_mlp_fwd.restype = c_int
     lib.nf_mlp_fwd.argtypes = [P, I64, P, I64, P, P, P, P, P, P, I64, I, I, I, I, I, I, I, P, I64, P]
+    lib.nf_mlp_bwd_rounded.restype = c_int
+    lib.nf_mlp_bwd_rounded.argtypes = [P, I64, P, I64, P, I64, P, P, P, P, P, P, P, P, P, P, P, P, I64, I, I, I, I, I, I, I, P, I64, P]
+    lib.nf_mlp_bwd_rounded_workspace_bytes.restype = I64
+    lib.nf_mlp_bwd_rounded_workspace_bytes.argtypes = [I, I, I]
     lib.nf_mlp_workspace_bytes.restype = I64
     lib.nf_mlp_workspace_bytes.argtypes = [I64, I, I, I, I, I]
     lib.nf_mlp_bwd.restype = c_int

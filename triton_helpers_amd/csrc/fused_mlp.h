@@ -22,6 +22,10 @@ struct MlpArgs {
   int waves;  // waves per workgroup
   int in_act; // activation applied to x as it is loaded (x holds pre-activations of a layer in front); dx = d/dx of that
   int x_conv; // 0: x / dx stored like the weights; 1: stored as float16 (weights bfloat16); 2: stored as bfloat16 (weights float16)
+  // eight-wave backward only: non-NULL = every workgroup stores its sums into partials + blockIdx.x * partial_stride
+  // ([dw_in | dw_hid | dw_out | db_in | db_hid | db_out], float32) instead of adding them to dw_* / db_*
+  float* partials;
+  int64_t partial_stride;
 };
 
 constexpr int FRAG_ELEMS = 64 * 8;  // 16-bit elements per fragment (1 KiB)
@@ -94,13 +98,18 @@ __device__ __forceinline__ Frag panel_frag(const uint16_t* panel, int t, int lan
 
 // dW tile (mt over output features, nt over input features): lane (n, g) reg r is
 // dW[16*mt + 4*g + r][16*nt + n].
-__device__ __forceinline__ void flush_dw_tile(float* dw, int out_dim, int in_dim, int mt, int nt, int lane, f32x4_t v) {
+// store: plain stores (the tile belongs to this workgroup alone) instead of atomic adds.
+__device__ __forceinline__ void flush_dw_tile(float* dw, int out_dim, int in_dim, int mt, int nt, int lane, f32x4_t v,
+                                              bool store = false) {
   const int c = 16 * nt + (lane & 15);
   const int r0 = 16 * mt + 4 * (lane >> 4);
   if (c >= in_dim) return;
 #pragma unroll
   for (int r = 0; r < 4; ++r)
-    if (r0 + r < out_dim) unsafeAtomicAdd(dw + (size_t)(r0 + r) * in_dim + c, v[r]);
+    if (r0 + r < out_dim) {
+      if (store) dw[(size_t)(r0 + r) * in_dim + c] = v[r];
+      else unsafeAtomicAdd(dw + (size_t)(r0 + r) * in_dim + c, v[r]);
+    }
 }
 
 // Compute units of the current device.  The count is cached per device ordinal (written once with the same value by
@@ -129,6 +138,10 @@ int launch_mlp_bwdn(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
 // The benchmark shape of launch_mlp_bwd2 (d_in <= 32, d_hidden = 64, d_out <= 16, ReLU, aligned rows, extents below
 // 2^31 bytes) on eight waves per workgroup (fused_mlp_bwd2_w8.hip).  *handled = false: not that shape.
 int launch_mlp_bwd2_w8(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
+// The same with the weight and bias gradients summed in a fixed order and written, rounded to `dtype`, into out[6]
+// (dw_in, db_in, dw_hid, db_hid, dw_out, db_out; NULL entries skipped); workspace: mlp_bwd2_w8_rounded_bytes().
+size_t mlp_bwd2_w8_rounded_bytes(int d_in, int d_hidden, int d_out);
+int launch_mlp_bwd2_w8_rounded(const MlpArgs& a, int dtype, void* const out[6], void* workspace, hipStream_t s, bool* handled);
 
 
 // The forward of that shape (fused_mlp_fwd2.hip).  *handled = false: not that shape, nothing was launched.

@@ -852,3 +852,39 @@ extern "C" int nf_mlp_bwd(const void* x, int64_t x_stride, const void* dy, int64
   return 0;
 }
 
+
+extern "C" int64_t nf_mlp_bwd_rounded_workspace_bytes(int d_in, int d_hidden, int d_out) {
+  if (d_in < 1 || d_hidden < 1 || d_out < 1) return 0;
+  return (int64_t)mlp_bwd2_w8_rounded_bytes(d_in, d_hidden, d_out);
+}
+
+extern "C" int nf_mlp_bwd_rounded(const void* x, int64_t x_stride, const void* dy, int64_t dy_stride, void* dx, int64_t dx_stride,
+                                  const void* w_in, const void* b_in, const void* w_hid, const void* b_hid, const void* w_out,
+                                  const void* b_out, void* dw_in, void* db_in, void* dw_hid, void* db_hid, void* dw_out,
+                                  void* db_out, int64_t rows, int d_in, int d_hidden, int d_out, int depth, int act, int dtype,
+                                  int x_dtype, void* workspace, int64_t workspace_bytes, void* stream) {
+  if (int rc = validate(rows, d_in, d_hidden, d_out, depth, act, dtype)) return rc;
+  NF_REQUIRE(dtype != NF_F32 && (x_dtype == NF_F16 || x_dtype == NF_BF16), NF_EUNSUPPORTED,
+             "rounded weight gradients: 16-bit tensors only (dtype code %d, x_dtype code %d)", dtype, x_dtype);
+  NF_REQUIRE(rows > 0, NF_EUNSUPPORTED, "rounded weight gradients: no rows (the buffers would stay unwritten)");
+  NF_REQUIRE(x && dy && w_in && w_hid && w_out && dw_in && dw_hid && dw_out, NF_EINVAL, "NULL pointer argument");
+  NF_REQUIRE(x_stride >= d_in && dy_stride >= d_out && (dx == nullptr || dx_stride >= d_in), NF_EINVAL,
+             "row stride smaller than row width");
+  const int64_t need = nf_mlp_bwd_rounded_workspace_bytes(d_in, d_hidden, d_out);
+  NF_REQUIRE(workspace != nullptr && workspace_bytes >= need && (uintptr_t)workspace % 16 == 0, NF_EINVAL,
+             "rounded weight gradients need a 16-byte aligned workspace of %lld bytes (nf_mlp_bwd_rounded_workspace_bytes)",
+             (long long)need);
+  MlpArgs a = {};
+  a.w_in = (const uint16_t*)w_in; a.b_in = (const uint16_t*)b_in; a.w_hid = (const uint16_t*)w_hid;
+  a.b_hid = (const uint16_t*)b_hid; a.w_out = (const uint16_t*)w_out; a.b_out = (const uint16_t*)b_out;
+  a.rows = rows; a.d_in = d_in; a.d_hidden = d_hidden; a.d_out = d_out; a.depth = depth; a.act = act;
+  a.in_act = NF_ACT_NONE;
+  a.x_conv = x_dtype == dtype ? 0 : (x_dtype == NF_F16 ? 1 : 2);
+  set_rows(a, (const uint16_t*)x, x_stride, nullptr, 0, (const uint16_t*)dy, dy_stride, (uint16_t*)dx, dx_stride);
+  void* const out[6] = {dw_in, db_in, dw_hid, db_hid, dw_out, db_out};
+  bool handled = false;
+  const int rc = launch_mlp_bwd2_w8_rounded(a, dtype, out, workspace, (hipStream_t)stream, &handled);
+  if (rc != 0 || handled) return rc;
+  return fail(NF_EUNSUPPORTED, "rounded weight gradients: built for one hidden-to-hidden layer, d_hidden = 64, d_in <= 32, d_out <= 16, "
+                               "ReLU and 8-byte aligned rows (nothing was launched; use nf_mlp_bwd)");
+}

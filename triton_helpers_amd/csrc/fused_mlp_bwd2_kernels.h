@@ -19,11 +19,14 @@
 namespace nf {
 
 // Bias gradient of feature 16*mt + n: the four lane groups hold partial sums over disjoint rows.
-__device__ __forceinline__ void flush_db(float* db, int dim, int mt, int lane, float v) {
+__device__ __forceinline__ void flush_db(float* db, int dim, int mt, int lane, float v, bool store = false) {
   v += __shfl_xor(v, 16);
   v += __shfl_xor(v, 32);
   const int f = 16 * mt + lane;
-  if (db != nullptr && lane < 16 && f < dim) unsafeAtomicAdd(db + f, v);
+  if (db != nullptr && lane < 16 && f < dim) {
+    if (store) db[f] = v;
+    else unsafeAtomicAdd(db + f, v);
+  }
 }
 
 typedef short s16x2_t __attribute__((ext_vector_type(2)));
@@ -657,26 +660,35 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd2_k(MlpArgs a) {
       return (p[0] + p[(size_t)NBIAS * 64]) + (p[(size_t)2 * NBIAS * 64] + p[(size_t)3 * NBIAS * 64]);
     };
     {
+      // where the sums go: the caller's accumulators (atomic adds), or this workgroup's own slot (plain stores)
+      const bool own = a.partials != nullptr;
+      float* slot = own ? a.partials + (size_t)blockIdx.x * a.partial_stride : nullptr;
+      float* p_dw_in = own ? slot : a.dw_in;
+      float* p_dw_hid = own ? p_dw_in + a.d_hidden * a.d_in : a.dw_hid;
+      float* p_dw_out = own ? p_dw_hid + a.d_hidden * a.d_hidden : a.dw_out;
+      float* p_db_in = own ? p_dw_out + a.d_out * a.d_hidden : a.db_in;
+      float* p_db_hid = own ? p_db_in + a.d_hidden : a.db_hid;
+      float* p_db_out = own ? p_db_hid + a.d_hidden : a.db_out;
       int t = 0, u = 0;
   #pragma unroll
       for (int i = 0; i < MT_H; ++i) {
   #pragma unroll
         for (int j = 0; j < MT_I; ++j, ++t)
-          if ((t & 3) == wave) flush_dw_tile(a.dw_in, a.d_hidden, a.d_in, i, j, lane, tile_sum(t));
+          if ((t & 3) == wave) flush_dw_tile(p_dw_in, a.d_hidden, a.d_in, i, j, lane, tile_sum(t), own);
   #pragma unroll
         for (int j = 0; j < MT_H; ++j, ++t)
-          if ((t & 3) == wave) flush_dw_tile(a.dw_hid, a.d_hidden, a.d_hidden, i, j, lane, tile_sum(t));
-        if ((u & 3) == wave) flush_db(a.db_in, a.d_hidden, i, lane, bias_sum(u));
+          if ((t & 3) == wave) flush_dw_tile(p_dw_hid, a.d_hidden, a.d_hidden, i, j, lane, tile_sum(t), own);
+        if ((u & 3) == wave) flush_db(p_db_in, a.d_hidden, i, lane, bias_sum(u), own);
         ++u;
-        if ((u & 3) == wave) flush_db(a.db_hid, a.d_hidden, i, lane, bias_sum(u));
+        if ((u & 3) == wave) flush_db(p_db_hid, a.d_hidden, i, lane, bias_sum(u), own);
         ++u;
       }
   #pragma unroll
       for (int i = 0; i < MT_O; ++i) {
   #pragma unroll
         for (int j = 0; j < MT_H; ++j, ++t)
-          if ((t & 3) == wave) flush_dw_tile(a.dw_out, a.d_out, a.d_hidden, i, j, lane, tile_sum(t));
-        if ((u & 3) == wave) flush_db(a.db_out, a.d_out, i, lane, bias_sum(u));
+          if ((t & 3) == wave) flush_dw_tile(p_dw_out, a.d_out, a.d_hidden, i, j, lane, tile_sum(t), own);
+        if ((u & 3) == wave) flush_db(p_db_out, a.d_out, i, lane, bias_sum(u), own);
         ++u;
       }
     }

@@ -232,6 +232,11 @@ class _fully_fused_mlp(Function):
             x = x.to(w_in.dtype)  # only the one-hidden-layer ReLU backward converts on the fly
         do2 = _rows2d(do, D_out)
         need_dx = ctx.needs_input_grad[0]
+        if (not wide and w_in.dtype != torch.float32 and ctx.depth == 2 and D_hidden == 64 and D_in <= 32 and D_out <= 16
+                and D_in % 4 == 0 and D_out % 4 == 0 and ctx.activation == "relu" and do2.shape[0] > 0):
+            done = _backward_rounded(x, do2, w_in, b_in, w_out, b_out, w_hid, b_hid, need_dx, D_in, D_hidden, D_out)
+            if done is not None:
+                return done
         grads = _lib.GradBuffers(w_in, b_in, w_out, b_out, w_hid, b_hid)
         p_dw_in, p_db_in, p_dw_out, p_db_out, p_dw_hid, p_db_hid = grads.pointers()
         lib = _lib.load()
@@ -257,6 +262,40 @@ class _fully_fused_mlp(Function):
         if wide and dx is not None:
             dx = dx.float()
         return dx, dw_in, db_in, dw_out, db_out, dw_hid, db_hid, None, None
+
+
+def _backward_rounded(x, do2, w_in, b_in, w_out, b_out, w_hid, b_hid, need_dx, D_in, D_hidden, D_out):
+    """Backward of the decoder shape through ``nf_mlp_bwd_rounded``: the weight gradients come back summed in a fixed
+    order and rounded to the parameters' dtype, into one uninitialised buffer (no clearing, no cast kernel).  ``None`` when
+    the library declines (rows not 8-byte aligned): the caller takes the general path."""
+    lib = _lib.load()
+    like = (w_in, b_in, w_out, b_out, w_hid, b_hid)
+    offsets, off = [], 0
+    for t in like:
+        offsets.append(off)
+        if t is not None:
+            off += (t.numel() + 7) // 8 * 8  # 16-byte aligned pieces
+    flat = torch.empty(off, dtype=w_in.dtype, device=w_in.device)
+    base, es = flat.data_ptr(), flat.element_size()
+    p = [None if t is None else base + es * o for t, o in zip(like, offsets)]
+    ws_bytes = lib.nf_mlp_bwd_rounded_workspace_bytes(D_in, D_hidden, D_out)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w_in.device)
+    x2 = _rows2d(x, D_in)
+    dx = x.new_empty(x.shape) if need_dx else None
+    rc = lib.nf_mlp_bwd_rounded(
+        x2.data_ptr(), x2.stride(0), do2.data_ptr(), do2.stride(0), _lib.ptr(dx), D_in,
+        w_in.data_ptr(), _lib.ptr(b_in), _lib.ptr(w_hid), _lib.ptr(b_hid), w_out.data_ptr(), _lib.ptr(b_out),
+        p[0], p[1], p[4], p[5], p[2], p[3],
+        x2.shape[0], D_in, D_hidden, D_out, 2, _lib.NF_ACT["relu"], _lib.dtype_code(w_in.dtype), _lib.dtype_code(x.dtype),
+        ws.data_ptr(), ws_bytes, _lib.current_stream(x.device),
+    )
+    if rc == _lib.NF_EUNSUPPORTED:
+        return None
+    _lib.check(rc, "nf_mlp_bwd_rounded")
+    g = [None if t is None else flat.as_strided(t.shape, t.stride(), o) if t.is_contiguous() else flat[o:o + t.numel()].view(t.shape)
+         for t, o in zip(like, offsets)]
+    dw_in, db_in, dw_out, db_out, dw_hid, db_hid = g
+    return dx, dw_in, db_in, dw_out, db_out, dw_hid, db_hid, None, None
 
 
 def fully_fused_mlp(
