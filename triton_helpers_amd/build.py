@@ -36,7 +36,7 @@ COMMON_FLAGS = [
 NO_CONTRACT = {"hash_encoding.hip", "hash_encoding_bwd_scan.hip", "hash_encoding_bwd_bin.hip", "hash_encoding_bwd_static.hip", "hash_check_host.hip"}
 # Files whose MFMA results feed vector ALU work directly: keep them in architectural VGPRs instead of
 # bouncing every result through an accumulation register.
-MFMA_VGPR_FORM = {"fused_mlp.hip", "fused_mlp_bwd2.hip", "fused_mlp_bwdn.hip", "fused_mlp_bwd2_w8.hip", "fused_mlp_fwd2.hip", "reversible_mlp.hip"}
+MFMA_VGPR_FORM = {"fused_mlp.hip", "fused_mlp_bwd2.hip", "fused_mlp_bwdn.hip", "fused_mlp_bwd2_w8.hip", "fused_mlp_bwd2_ws.hip", "fused_mlp_fwd2.hip", "reversible_mlp.hip"}
 
 
 def _hipcc() -> str:

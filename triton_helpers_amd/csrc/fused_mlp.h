@@ -144,6 +144,10 @@ size_t mlp_bwd2_w8_rounded_bytes(int d_in, int d_hidden, int d_out);
 int launch_mlp_bwd2_w8_rounded(const MlpArgs& a, int dtype, void* const out[6], void* workspace, hipStream_t s, bool* handled);
 
 
+// One hidden layer, width 64, ReLU, with d_in > 32 or d_out > 16 (aligned rows, extents below 2^31 bytes): chain and
+// gradient waves (fused_mlp_bwd2_ws.hip).  *handled = false: not such a call, nothing was launched.
+int launch_mlp_bwd2_ws(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
+
 // The forward of that shape (fused_mlp_fwd2.hip).  *handled = false: not that shape, nothing was launched.
 int launch_mlp_fwd2(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
 

@@ -76,7 +76,9 @@ static int dispatch2(const MlpArgs& a, hipStream_t s, bool* handled) {
 int launch_mlp_bwd2(const MlpArgs& a, int dtype, hipStream_t s, bool* handled) {
   *handled = false;
   if (a.depth == 2) {
-    const int rc = launch_mlp_bwd2_w8(a, dtype, s, handled);
+    int rc = launch_mlp_bwd2_w8(a, dtype, s, handled);
+    if (rc != 0 || *handled) return rc;
+    rc = launch_mlp_bwd2_ws(a, dtype, s, handled);
     if (rc != 0 || *handled) return rc;
     return dtype == NF_BF16 ? dispatch2<BF16>(a, s, handled) : dispatch2<F16>(a, s, handled);
   }
