@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define NF_ABI_VERSION 7
+#define NF_ABI_VERSION 8
 
 /* element types */
 enum { NF_F32 = 0, NF_F16 = 1, NF_BF16 = 2 };
@@ -119,6 +119,15 @@ int64_t nf_hash_encode_bwd_static_bytes(void);
 int nf_hash_encode_indices(const void* coords, int coords_dtype, int64_t coords_stride_n, int64_t coords_stride_d,
                            int64_t* out_rows, float* out_w, int64_t n_points, const nf_hash_geom* geom,
                            const int64_t* primes, float scale, void* stream);
+
+/* The same output computed with the index arithmetic of the fast kernels (the forward sweep / tiled kernels and the
+ * binned backward): 32-bit wrap-around products and the level's mask instead of 64-bit products and a remainder.
+ * D = 2 or 3, hashed levels with a power-of-two row count (NF_EUNSUPPORTED otherwise).  Same reference interface as
+ * nf_hash_encode_indices (embedding_lookup, triton_helpers/layers/hash_encoding/kernel.py:88-152, whose device form
+ * is this 32-bit one, :143-145); the two entry points must agree bit for bit. */
+int nf_hash_encode_indices_fast(const void* coords, int coords_dtype, int64_t coords_stride_n, int64_t coords_stride_d,
+                                int64_t* out_rows, float* out_w, int64_t n_points, const nf_hash_geom* geom,
+                                const int64_t* primes, float scale, void* stream);
 
 /* Host-side range check, the counterpart of the reference's debug-build asserts (tl.device_assert under
  * TRITON_DEBUG, triton_helpers/layers/hash_encoding/kernel.py:109-122, 151, 227-228).  Runs on the CPU, launches

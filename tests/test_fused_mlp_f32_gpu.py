@@ -162,3 +162,69 @@ def test_float32_gradients_accumulate_and_strided_rows():
     _close(dxs[:, :d_in], want["dx"], "dx")
     for k in g:
         _close(g[k], 2 * want["d" + k], "d" + k)
+
+
+def _float64_relu_net(p, x, dy):
+    """float64 evaluation of the ReLU network written out with torch ops: gradients, and per row the smallest
+    |pre-activation| relative to the row's largest one (a row whose smallest is ~1e-7 has a gate that float32
+    rounding, i.e. the order of a sum, can flip)."""
+    H = p["w_in"].shape[0]
+    depth = 1 if p["w_hid"] is None else p["w_hid"].shape[0] // H + 1
+    leaves = {k: (None if v is None else v.double().clone().requires_grad_(True)) for k, v in p.items()}
+    xx = x.double().clone().requires_grad_(True)
+    margin = None
+    h = xx
+    for k in range(depth):
+        w = leaves["w_in"] if k == 0 else leaves["w_hid"][(k - 1) * H:k * H]
+        b = leaves["b_in"] if k == 0 else (None if leaves["b_hid"] is None else leaves["b_hid"][k - 1])
+        z = h @ w.t() if b is None else h @ w.t() + b
+        rel = (z.detach().abs() / z.detach().abs().amax(1, keepdim=True).clamp_min(1e-300)).amin(1)
+        margin = rel if margin is None else torch.minimum(margin, rel)
+        h = torch.relu(z)
+    y = h @ leaves["w_out"].t() if leaves["b_out"] is None else h @ leaves["w_out"].t() + leaves["b_out"]
+    y.backward(dy.double())
+    out = {"y": y.detach(), "dx": xx.grad}
+    out.update({"d" + k: v.grad for k, v in leaves.items() if v is not None})
+    return out, margin
+
+
+@pytest.mark.parametrize("case,rows,d_in,d_hidden,depth,d_out,bias", [
+    (67, 33333, 25, 64, 9, 50, False),
+    (141, 4097, 45, 64, 4, 21, True),
+])
+def test_deep_relu_float32_many_rows(case, rows, d_in, d_hidden, depth, d_out, bias):
+    """The two cases of a randomized sweep in which 33 % / 49 % of the elements of dW_in missed rtol 1e-4.  Cause: ONE
+    row of the batch has a pre-activation within float32 rounding of zero, its ReLU gate opens or closes with the order
+    of the sum, and a single row carries more than 1e-4 of every weight-gradient element.  On the CPU, float32 against
+    float64 reproduces the same fraction for the second case (0.4906 of dW_in) and a permuted float32 summation makes it
+    vanish.  So the kernels are held to: (1) rows whose dx is grossly off are rows with such a pre-activation, and
+    there are only a handful; (2) with those rows taken out of the batch every gradient matches float64 at rtol 1e-4
+    with no outlier."""
+    mk = _mk()
+    torch.manual_seed(case)
+    p = _params(d_in, d_hidden, d_out, depth, bias, torch.float32, seed=case, gain=1.7)
+    x = torch.randn(rows, d_in)
+    dy = torch.randn(rows, d_out)
+
+    def run(xr, dyr):
+        leaves = {k: (None if v is None else v.to(DEV).requires_grad_(True)) for k, v in p.items()}
+        xd = xr.view(1, -1, d_in).to(DEV).requires_grad_(True)
+        y = mk.fully_fused_mlp(xd, leaves["w_in"], leaves["b_in"], leaves["w_out"], leaves["b_out"], leaves["w_hid"], leaves["b_hid"], "relu")
+        y.backward(dyr.view(1, -1, d_out).to(DEV))
+        out = {"y": y.detach().view(-1, d_out), "dx": xd.grad.view(-1, d_in)}
+        out.update({"d" + k: v.grad for k, v in leaves.items() if v is not None})
+        return {k: v.cpu() for k, v in out.items()}
+
+    want, margin = _float64_relu_net(p, x, dy)
+    got = run(x, dy)
+    _close(got["y"], want["y"], "y")
+    gross = (got["dx"].double() - want["dx"]).abs().amax(1) > 1e-3 * float(want["dx"].abs().max())
+    fragile = margin < 1e-5
+    assert int(gross.sum()) <= 8, f"{int(gross.sum())} rows with a gross dx error"
+    assert bool((fragile | ~gross).all()), "a row without a pre-activation near zero has a gross dx error"
+    keep = ~fragile
+    assert int(keep.sum()) >= 0.98 * rows  # nine layers x 64 units x 33333 rows: a few hundred rows come that close
+    want2, _ = _float64_relu_net(p, x[keep], dy[keep])
+    got2 = run(x[keep].contiguous(), dy[keep].contiguous())
+    for k in want2:
+        _close(got2[k], want2[k], k)

@@ -65,6 +65,22 @@ def test_corner_rows_bit_exact(N, D, F, T, L, lo, hi, scale):
     res = O.level_resolutions(L, lo, hi)
     wref = torch.stack([O.corner_weights(x, D, r) for r in res], 1)
     torch.testing.assert_close(w.cpu(), wref, rtol=1e-6, atol=1e-7)
+    # the 32-bit index arithmetic of the fast kernels, evaluated on the device, where it applies
+    if D in (2, 3) and (T & (T - 1)) == 0:
+        fast, wf = _hk().hash_encoding_indices(xs.to(DEV), None, T, lo, hi, L, scale=scale, return_weights=True, fast=True)
+        assert torch.equal(fast.cpu(), want)
+        assert torch.equal(wf, w), "the fast kernels' weights are the generic kernels' weights, bit for bit"
+
+
+def test_corner_rows_fast_path_upper_edge():
+    """x == scale in every dimension: the fast kernels' index functions keep the zero-weight corner inside the level,
+    like the 64-bit form."""
+    for D in (2, 3):
+        x = torch.ones(5, D, device=DEV)
+        x[1:] = torch.rand(4, D, device=DEV)
+        a = _hk().hash_encoding_indices(x, None, 2**12, 16, 64, 4)
+        b = _hk().hash_encoding_indices(x, None, 2**12, 16, 64, 4, fast=True)
+        assert torch.equal(a, b)
 
 
 def test_corner_rows_reference_literals():
@@ -77,6 +93,11 @@ def test_corner_rows_reference_literals():
     hashed = _hk().hash_encoding_indices(x, None, 7, 2, 4, 2)[:, 0]
     assert dense.cpu().tolist() == DENSE_ROWS
     assert hashed.cpu().tolist() == HASHED_ROWS
+    # the dense table again from the fast kernels' 32-bit arithmetic: T = 16 leaves level 0 (resolution 2, nine rows)
+    # dense and gives the hashed level 1 the power-of-two size that form needs (the hashed literal table uses T = 7,
+    # which only the 64-bit remainder form covers)
+    dense_fast = _hk().hash_encoding_indices(x, None, 16, 2, 4, 2, fast=True)[:, 0]
+    assert dense_fast.cpu().tolist() == DENSE_ROWS
 
 
 @pytest.mark.parametrize("N,D,F,T,L,lo,hi,scale", CASES)
@@ -203,8 +224,11 @@ def test_forward_config0_full_size():
     want = O.encode_forward(x, table, None, g["T"], 16, 16, 7006)
     got = _hk().hash_encoding(x.to(DEV), table.to(DEV), None, None, g["T"], 16, 7006, 16)
     torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-9)
+    want_rows = O.encode_indices(x, None, g["T"], 16, 16, 7006)
     rows = _hk().hash_encoding_indices(x.to(DEV), None, g["T"], 16, 7006, 16)
-    assert torch.equal(rows.cpu(), O.encode_indices(x, None, g["T"], 16, 16, 7006))
+    assert torch.equal(rows.cpu(), want_rows)
+    fast = _hk().hash_encoding_indices(x.to(DEV), None, g["T"], 16, 7006, 16, fast=True)
+    assert torch.equal(fast.cpu(), want_rows), "the fast kernels' device index arithmetic differs from the oracle"
 
 
 @pytest.mark.parametrize("N,D,F,T,L,lo,hi,scale", CASES + [(65536, 3, 2, 2**20, 16, 16, 512, 1.0), (131072, 3, 2, 2**14, 16, 16, 512, 1.0)])
@@ -381,6 +405,39 @@ def test_backward_binned_nonfinite_gradient(do_dtype):
     keep = torch.ones(E, dtype=torch.bool)
     keep[lvl2] = False
     torch.testing.assert_close(got[keep], clean[keep], rtol=1e-3, atol=1e-4)
+
+
+@pytest.mark.parametrize("feat", [1, 3])
+def test_backward_binned_nonfinite_gradient_odd_feature_count(feat):
+    """With an odd number of features the last feature is a pair with an empty partner: an inf in a level's gradient
+    must mark that level's rows only -- not feature 0 of the following row, the first row of the next level, or the
+    memory behind the table (a guard region after the gradient table stays untouched)."""
+    hk = _hk()
+    torch.manual_seed(7)
+    N, T, L, lo, hi = 40000, 2**16, 4, 16, 256
+    x = torch.rand(N, 3)
+    offs = O.level_row_offsets(L, T, 3, lo, hi)
+    E = offs[-1]
+    do = torch.randn(N, L * feat).half()
+    clean = O.encode_backward(x, do, E, feat, None, T, L, lo, hi)
+    do[123, 3 * feat + feat - 1] = float("inf")  # the last level, its last feature
+    guard = 4096
+    buf = torch.zeros(E * feat + guard, dtype=torch.float32, device=DEV)
+    out = buf[: E * feat].view(E, feat)
+    got = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, feat, None, T, lo, hi, L, out=out).cpu()
+    assert torch.count_nonzero(buf[E * feat:]).item() == 0, "wrote behind the gradient table"
+    last = slice(offs[3], offs[4])
+    assert not torch.isfinite(got[last, feat - 1]).all()
+    # the other features of the poisoned level and every other level are exact
+    if feat > 1:
+        torch.testing.assert_close(got[last, : feat - 1], clean[last, : feat - 1], rtol=1e-3, atol=1e-4)
+    torch.testing.assert_close(got[: offs[3]], clean[: offs[3]], rtol=1e-3, atol=1e-4)
+    # ... and with the inf in the first level the first row of the next level stays clean
+    do2 = torch.randn(N, L * feat).half()
+    clean2 = O.encode_backward(x, do2, E, feat, None, T, L, lo, hi)
+    do2[77, feat - 1] = float("inf")
+    got2 = hk.hash_encoding_table_grad(x.to(DEV), do2.to(DEV), E, feat, None, T, lo, hi, L).cpu()
+    torch.testing.assert_close(got2[offs[1]:], clean2[offs[1]:], rtol=1e-3, atol=1e-4)
 
 
 def test_autograd_round_trip_fp16_table():

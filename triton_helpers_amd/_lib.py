@@ -14,7 +14,7 @@ import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "libnf_cdna4.so"
 
-NF_ABI_VERSION = 7
+NF_ABI_VERSION = 8
 NF_F32, NF_F16, NF_BF16 = 0, 1, 2
 NF_ACT = {"none": 0, "relu": 1, "silu": 2, "relu2": 3, "gelu": 4}
 NF_MAX_LEVELS = 32
@@ -36,6 +36,7 @@ EXPORTS = (
     "nf_hash_encode_bwd_static",
     "nf_hash_encode_bwd_static_bytes",
     "nf_hash_encode_indices",
+    "nf_hash_encode_indices_fast",
     "nf_hash_check_host",
     "nf_table_adam_step",
     "nf_mlp_fwd",
@@ -95,6 +96,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.nf_hash_encode_bwd_static_bytes.argtypes = []
     lib.nf_hash_encode_indices.restype = c_int
     lib.nf_hash_encode_indices.argtypes = [P, I, I64, I64, P, P, I64, POINTER(HashGeom), P, c_float, P]
+    lib.nf_hash_encode_indices_fast.restype = c_int
+    lib.nf_hash_encode_indices_fast.argtypes = [P, I, I64, I64, P, P, I64, POINTER(HashGeom), P, c_float, P]
     lib.nf_hash_check_host.restype = c_int
     lib.nf_hash_check_host.argtypes = [P, I64, POINTER(HashGeom), P, c_float, I, P, P, P]
     lib.nf_table_adam_step.restype = c_int

@@ -104,6 +104,52 @@ __global__ __launch_bounds__(256) void hash_indices_k(const void* coords, int cd
   }
 }
 
+// The same table through the index arithmetic of the fast kernels (sweep, tiled, binned backward): cells from
+// cell_index(), rows from rows_d3() / rows_d2() in 32-bit wrap-around arithmetic with the level's mask, weights from
+// weights_d3() / weights_d2() -- the very inline functions those kernels call, here with their results written out.
+template <int D>
+__global__ __launch_bounds__(256) void hash_indices_fast_k(const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                           int64_t* out_rows, float* out_w, int64_t N, DevGeom g,
+                                                           const int64_t* primes, float scale) {
+  static_assert(D == 2 || D == 3, "the fast kernels cover two and three dimensions");
+  constexpr int CN = 1 << D;
+  const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int l = blockIdx.y;
+  if (n >= N) return;
+  uint32_t pi[3] = {0u, 0u, 0u};
+#pragma unroll
+  for (int d = 0; d < D; ++d) pi[d] = (uint32_t)primes[d];
+  float x[3] = {0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    x[d] = load_as_f32(coords, n * csn + d * csd, cdt);
+    if (scale != 1.0f) x[d] = x[d] / scale;
+  }
+  const bool hashed = l >= g.first_hash;
+  const uint32_t res = (uint32_t)g.res[l];
+  const float fres = (float)g.res[l];
+  const uint32_t mask = g.rows[l] - 1;
+  uint32_t c[3] = {0u, 0u, 0u};
+  float fr[3] = {0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    const float pos = x[d] * fres;
+    const float fl = floorf(pos);
+    c[d] = cell_index(fl, fres);
+    fr[d] = pos - fl;
+  }
+  const Corner8 r = D == 3 ? rows_d3(c, hashed, res, mask, pi) : rows_d2(c, hashed, res, mask, pi);
+  float w[8];
+  if (D == 3) weights_d3(fr, w);
+  else weights_d2(fr, w);
+  const int64_t base = (n * g.levels + l) * CN;
+#pragma unroll
+  for (int j = 0; j < CN; ++j) {
+    out_rows[base + j] = (int64_t)r.row[j];
+    if (out_w) out_w[base + j] = w[j];
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Tiled path: D = 3, F = 2, 16-bit tables (one table row = one dword), L % 4 == 0.
 //
@@ -695,6 +741,27 @@ extern "C" int nf_hash_encode_bwd(const void* coords, int coords_dtype, int64_t 
     default: hipLaunchKernelGGL((hash_bwd_generic_k<4>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, g, primes, scale); break;
   }
   return check_launch("hash_bwd_generic");
+}
+
+extern "C" int nf_hash_encode_indices_fast(const void* coords, int coords_dtype, int64_t csn, int64_t csd,
+                                           int64_t* out_rows, float* out_w, int64_t n_points, const nf_hash_geom* geom,
+                                           const int64_t* primes, float scale, void* stream) {
+  DevGeom g;
+  if (int rc = make_dev_geom(geom, &g)) return rc;
+  NF_REQUIRE(dtype_ok(coords_dtype), NF_EINVAL, "unknown dtype code");
+  NF_REQUIRE(n_points >= 0, NF_EINVAL, "n_points negative");
+  NF_REQUIRE(scale > 0.0f, NF_EINVAL, "scale must be positive");
+  NF_REQUIRE(g.dims == 2 || g.dims == 3, NF_EUNSUPPORTED, "the 32-bit index form covers 2 and 3 dimensions, got %d", g.dims);
+  for (int l = g.first_hash < 0 ? 0 : g.first_hash; l < g.levels; ++l)
+    NF_REQUIRE((g.rows[l] & (g.rows[l] - 1u)) == 0u, NF_EUNSUPPORTED,
+               "the 32-bit index form needs power-of-two hashed levels (level %d has %u rows)", l, g.rows[l]);
+  if (n_points == 0) return 0;
+  NF_REQUIRE(coords && out_rows && primes, NF_EINVAL, "NULL pointer argument");
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid((unsigned)((n_points + 255) / 256), (unsigned)g.levels);
+  if (g.dims == 3) hipLaunchKernelGGL((hash_indices_fast_k<3>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, out_rows, out_w, n_points, g, primes, scale);
+  else hipLaunchKernelGGL((hash_indices_fast_k<2>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, out_rows, out_w, n_points, g, primes, scale);
+  return check_launch("hash_indices_fast");
 }
 
 extern "C" int nf_hash_encode_indices(const void* coords, int coords_dtype, int64_t csn, int64_t csd,

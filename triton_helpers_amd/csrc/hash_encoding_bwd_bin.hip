@@ -605,6 +605,8 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const typena
     return r;
   };
   const uint32_t n_rec = task.z - task.y;
+  // an odd feature count leaves the last pass with one feature: plane 1 then has no column in the table
+  const bool has_pair = f0 + 1 < feat;
   // the next round's records are loaded before this round's adds; a level with an inf or a nan in its gradient only
   // marks the rows it touches (its own copy of the loop, so that the usual one has no test per record)
   auto accumulate = [&](auto nonfinite_c) {
@@ -622,8 +624,10 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const typena
         slot[k][0] = q[k].x & BIN_MASK;
         slot[k][1] = (q[k].x >> BIN_ROWS_LOG2) & BIN_MASK;
         if constexpr (NONFINITE) {
-          f[k][0] = f[k][1] = w0 != 0.0f;
-          f[k][2] = f[k][3] = w1 != 0.0f;
+          f[k][0] = w0 != 0.0f;
+          f[k][2] = w1 != 0.0f;
+          f[k][1] = has_pair && f[k][0];
+          f[k][3] = has_pair && f[k][2];
         } else {
           f[k][0] = __float2int_rn(w0 * g0 * s_hi);
           f[k][1] = __float2int_rn(w0 * g1 * s_hi);
@@ -652,7 +656,7 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const typena
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t i = i0 + u * ACC_THREADS + tid;
-      const long long a = i < nvals ? (long long)acc_tile[(i & 1u) * BIN_ROWS + (i >> 1)] : 0ll;
+      const long long a = (i < nvals && (has_pair || !(i & 1u))) ? (long long)acc_tile[(i & 1u) * BIN_ROWS + (i >> 1)] : 0ll;
       // |a| < 2^48 is exact in double and so is the division by 2^se: one rounding, to float, at the end
       x[u] = a == 0 ? 0.0f : (float)ldexp((double)a, -se);
       if (nonfinite && a != 0) x[u] = qnan;

@@ -318,11 +318,14 @@ def hash_encoding_indices(
     levels: int = 16,
     scale: float = 1.0,
     return_weights: bool = False,
+    fast: bool = False,
 ):
     """Level-local table rows ``(N, L, 2**D)`` int64 (and float32 weights) computed by the device code.
 
     The device-side counterpart of the reference's ``embedding_lookup`` test kernels
-    (reference tests/test_layers/test_hash_encoding.py:178-215).
+    (reference tests/test_layers/test_hash_encoding.py:178-215).  ``fast=True`` evaluates the 32-bit index arithmetic
+    of the fast kernels (forward sweep, binned backward; 2-D / 3-D, power-of-two hashed levels) instead of the 64-bit
+    form of the per-(point, level) kernels; the two must agree bit for bit.
     """
     coords2d = _flat_coords(coord)
     N, D = coords2d.shape
@@ -332,9 +335,10 @@ def hash_encoding_indices(
     rows = torch.empty(N, levels, 2**D, dtype=torch.int64, device=coord.device)
     w = torch.empty(N, levels, 2**D, dtype=torch.float32, device=coord.device) if return_weights else None
     lib = _lib.load()
-    rc = lib.nf_hash_encode_indices(
+    entry = lib.nf_hash_encode_indices_fast if fast else lib.nf_hash_encode_indices
+    rc = entry(
         coords2d.data_ptr(), _lib.dtype_code(coords2d.dtype), coords2d.stride(0), coords2d.stride(1),
         rows.data_ptr(), _lib.ptr(w), N, geom, pi.data_ptr(), float(scale), _lib.current_stream(coord.device),
     )
-    _lib.check(rc, "nf_hash_encode_indices")
+    _lib.check(rc, "nf_hash_encode_indices_fast" if fast else "nf_hash_encode_indices")
     return (rows, w) if return_weights else rows
