@@ -15,7 +15,10 @@ Extra objects in the same line:
   roofline      the dominant kernel of the step (the forward gather kernel: the backward is a
                 chain of five shorter kernels), algorithmic bytes per launch / launch time measured
                 here with events against the 8 TB/s HBM peak; ``traffic`` (HBM bytes per launch) and
-                the L2 request count come from the counters in the committed profile summary;
+                the L2 request count are counter figures of a separate profiler run, kept in the
+                committed profile summary together with that run's kernel time: they are quoted
+                (``traffic_source`` says from where) only while this run's launch time is within 10 %
+                of it, and are null otherwise;
   cpu_baseline  the CPU oracle (a port of the reference's PyTorch path) timed on this host
                 on a 65536-point sample of the same workload; ``cpu_baselines`` holds the same for
                 the other configurations (configs[0] is the reference's own CPU-runnable case);
@@ -57,17 +60,28 @@ E2E_LOSS_SCALE = 2.0**20
 CPU_SAMPLE = 65536
 
 
-def profile_figures():
-    """Counter-derived figures of the forward kernel, kept in the committed profile summary as a line
-    ``<!-- bench-figures: key=value ... -->`` next to the tables they come from (None when absent)."""
+def profile_figures(kernel, launch_ms):
+    """Counter-derived figures of the forward kernel.  They cannot be measured in this run (hardware counters need
+    the profiler), so the committed profile summary keeps them in a line
+    ``<!-- bench-figures: kernel=<name> kernel_us=<its duration in the counter run> key=value ... -->`` next to the
+    tables they come from.  Returns (figures, source): the figures are used only when the line names the kernel this
+    run launches and its duration then is within 10 % of the duration measured now; otherwise ({}, why)."""
+    rel = os.path.relpath(PROFILE_SUMMARY, ROOT)
     try:
         text = open(PROFILE_SUMMARY).read()
     except OSError:
-        return {}
+        return {}, f"{rel} is missing"
     m = re.search(r"<!--\s*bench-figures:(.*?)-->", text, flags=re.S)
     if not m:
-        return {}
-    return {k: float(v) for k, v in re.findall(r"(\w+)=([0-9.eE+-]+)", m.group(1))}
+        return {}, f"{rel} holds no bench-figures line"
+    name = re.search(r"kernel=(\S+)", m.group(1))
+    figs = {k: float(v) for k, v in re.findall(r"(\w+)=([0-9.eE+-]+)(?=\s|$)", m.group(1))}
+    if name is None or name.group(1) != kernel or "kernel_us" not in figs:
+        return {}, f"{rel}: the counter figures are for {name.group(1) if name else 'an unnamed kernel'}, this run launches {kernel}"
+    then_us, now_us = figs["kernel_us"], launch_ms * 1e3
+    if abs(then_us - now_us) > 0.10 * now_us:
+        return {}, f"{rel}: stale -- {kernel} took {then_us:.1f} us in the counter run and {now_us:.1f} us now"
+    return figs, f"{rel}: rocprofv3 --pmc run of {kernel} ({then_us:.1f} us per launch there, {now_us:.1f} us here)"
 
 
 def quantiles(ms):
@@ -435,10 +449,10 @@ def main():
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
     bwd_achieved = BWD_BYTES_PER_POINT * N_POINTS / (t_bwd * 1e-3) / 1e9
     step_bytes = (FWD_BYTES_PER_POINT + BWD_BYTES_PER_POINT) * N_POINTS + h["E"] * F * 4
-    figs = profile_figures() if not args.hash_kernel_flags else {}
+    figs, figs_source = profile_figures(dom, dom_ms)
     roofline = {
         "bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": achieved / HBM_PEAK_GBS, "traffic": figs.get("fwd_traffic_bytes"),
+        "frac": achieved / HBM_PEAK_GBS, "traffic": figs.get("fwd_traffic_bytes"), "traffic_source": figs_source,
         "launch_ms": dom_ms, "launch_ms_p20_p80": [h["fwd_ev"]["p20"], h["fwd_ev"]["p80"]],
         "algorithmic_bytes_per_launch": dom_bytes,
     }
@@ -446,7 +460,8 @@ def main():
         # the gathers are served by L2 (90 % hits): requests that leave the CUs x 128-byte lines over the launch time
         l2 = figs["fwd_l2_read_requests"] * 128 / (dom_ms * 1e-3) / 1e9
         roofline["l2"] = {"read_requests": figs["fwd_l2_read_requests"], "achieved": l2, "peak": L2_PEAK_GBS, "unit": "GB/s",
-                          "frac": l2 / L2_PEAK_GBS, "peak_how": "16 channels x 128 B/clk x 8 XCDs x 2.4 GHz"}
+                          "frac": l2 / L2_PEAK_GBS, "peak_how": "16 channels x 128 B/clk x 8 XCDs x 2.4 GHz",
+                          "source": "request count from the same counter run as traffic, time from this run"}
     out = {
         "metric": "Mpoints/s fwd+bwd: hash-enc+fused MLP @2^20 pts; % HBM / MFMA peak",
         "value": N_POINTS / h["ms"] / 1e3,
@@ -493,8 +508,8 @@ def main():
         s, w = max(5, args.steps // 2), max(3, args.warmup // 2)
         out["workloads"] = {
             "configs[2]": bench_mlp(s, w, 16),
-            "configs[3]": bench_rev(max(3, s // 2), 3),
-            "configs[4]": bench_e2e(max(3, s // 2), 3),
+            "configs[3]": bench_rev(max(20, s // 2), 5),
+            "configs[4]": bench_e2e(max(20, s // 2), 5),
         }
     if args.calibrate_copy:
         a = torch.zeros(64 * 2**20, dtype=torch.float32, device="cuda")

@@ -107,7 +107,10 @@ int64_t nf_hash_encode_bwd_workspace_bytes(int64_t n_points, const nf_hash_geom*
  * held until the process ends; the call allocates and frees nothing.  Batches whose scratch does not fit take the
  * smaller bit-plane variant where that applies (3-D points, 16-bit gradients: up to about 1.1 M points at L = 16) and
  * are refused with NF_EINVAL beyond that.  All calls on one GPU share the array: calls that overlap in time on one
- * GPU race on it.  Same arguments and results as nf_hash_encode_bwd otherwise. */
+ * GPU race on it.  The first call on a device resolves the array's address and sets the kernels' LDS attribute (it
+ * may load the library's code object): make one warm-up call per device before recording calls into a HIP graph or
+ * entering a region that may not touch the runtime's memory management.  Same arguments and results as
+ * nf_hash_encode_bwd otherwise. */
 #define NF_HASH_BWD_STATIC_BYTES (128 * 1024 * 1024)
 int nf_hash_encode_bwd_static(const void* coords, int coords_dtype, int64_t coords_stride_n, int64_t coords_stride_d,
                               const void* dout, int dout_dtype, int64_t dout_stride_n, float* dtable, int64_t n_points,
@@ -144,11 +147,16 @@ int nf_hash_check_host(const float* coords, int64_t n_points, const nf_hash_geom
  * float32 gradient nf_hash_encode_bwd accumulated for it.  No counterpart in the reference, which ships no
  * optimiser: the natural neighbour of its scatter-add, triton_helpers/layers/hash_encoding/kernel.py:432, 636.
  * table [n_elems] in table_dtype; master: float32 copy of the parameters (NULL: the table itself is the parameter);
- * grad is divided by grad_scale (the loss scale) before use and, with clear_grad != 0, zeroed for the next backward;
- * exp_avg / exp_avg_sq: float32 moments; step counts from 1. */
+ * grad is divided by grad_scale (the loss scale) before use; exp_avg / exp_avg_sq: float32 moments; step counts from 1.
+ * flags: NF_ADAM_CLEAR_GRAD zeroes grad for the next backward; NF_ADAM_SKIP_NONFINITE leaves the parameter and the
+ * moments of an element untouched when its gradient is inf or NaN (an overflowed loss-scaled step; the binned backward
+ * marks the rows of an overflowed level with NaN).  found_nonfinite (device int, may be NULL; cleared by the caller) is
+ * set to 1 when any gradient element was inf or NaN, with or without the skip. */
+#define NF_ADAM_CLEAR_GRAD 1
+#define NF_ADAM_SKIP_NONFINITE 2
 int nf_table_adam_step(void* table, int table_dtype, float* master, float* grad, float* exp_avg, float* exp_avg_sq,
                        int64_t n_elems, int64_t step, float lr, float beta1, float beta2, float eps, float weight_decay,
-                       float grad_scale, int clear_grad, void* stream);
+                       float grad_scale, int flags, int* found_nonfinite, void* stream);
 
 /* Fully fused MLP.  x [rows, d_in] (row stride x_stride) in x_dtype, y [rows, d_out] (row stride y_stride) in `dtype`;
  * w_in [d_hidden, d_in], w_hid [(depth-1)*d_hidden, d_hidden], w_out [d_out, d_hidden], all

@@ -72,3 +72,39 @@ def test_training_loop_keeps_one_gradient_buffer():
         opt.step(grad, grad_scale=65536.0)
         assert not bool(grad.any())
     assert losses[2] < losses[1] < losses[0]
+
+
+def test_nonfinite_gradient_elements_are_skipped_and_reported():
+    """An inf and a NaN in the gradient (an overflowed loss-scaled step): those elements keep their parameter and moments,
+    the others get the ordinary update, the flag is raised, and the gradient is cleared; without the skip the same
+    elements turn non-finite (torch.optim.Adam's behaviour), and the flag is raised all the same."""
+    from triton_helpers_amd.optim import TableAdam
+
+    torch.manual_seed(3)
+    n = (5000, 2)
+    p0 = ((torch.rand(n) * 2 - 1) * 1e-2).half()
+    g = torch.randn(n) * 0.1
+    bad = g.clone()
+    bad[17, 1] = float("inf")
+    bad[4000, 0] = float("nan")
+    clean_opt = TableAdam(p0.clone().to(DEV), lr=1e-3)
+    clean_opt.step(g.to(DEV))
+    assert int(clean_opt.found_nonfinite.item()) == 0
+    opt = TableAdam(p0.clone().to(DEV), lr=1e-3)
+    grad = bad.to(DEV)
+    opt.step(grad)
+    assert int(opt.found_nonfinite.item()) == 1
+    assert not bool(grad.any())
+    want = clean_opt.table.cpu().clone()
+    want[17, 1] = p0[17, 1]
+    want[4000, 0] = p0[4000, 0]
+    assert torch.equal(opt.table.cpu(), want)
+    assert float(opt.exp_avg[17, 1]) == 0.0 and float(opt.exp_avg_sq[4000, 0]) == 0.0
+    assert torch.isfinite(opt.master).all() and torch.isfinite(opt.exp_avg).all() and torch.isfinite(opt.exp_avg_sq).all()
+    # a later clean step clears the flag again
+    opt.step(g.to(DEV))
+    assert int(opt.found_nonfinite.item()) == 0
+    raw = TableAdam(p0.clone().to(DEV), lr=1e-3)
+    raw.step(bad.to(DEV), skip_nonfinite=False)
+    assert int(raw.found_nonfinite.item()) == 1
+    assert not torch.isfinite(raw.master[4000, 0]) and torch.isfinite(raw.master[0, 0])

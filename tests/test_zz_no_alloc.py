@@ -21,8 +21,16 @@ def _call(lib, L_, static, x, do, E, geom, pi, flags=0):
     de = torch.zeros(E, F, dtype=torch.float32, device=DEV)
     stream = L_.current_stream(x.device)
     if static:
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
         rc = lib.nf_hash_encode_bwd_static(x.data_ptr(), L_.dtype_code(x.dtype), x.stride(0), x.stride(1), do.data_ptr(), L_.dtype_code(do.dtype),
                                            do.stride(0), de.data_ptr(), x.shape[0], geom, pi.data_ptr(), 1.0, flags, stream)
+        torch.cuda.synchronize()
+        # after the first call on a device (which may load the code object and resolve the array's address) the entry
+        # point leaves the device's free memory exactly as it found it
+        if _call.warm:
+            assert torch.cuda.mem_get_info()[0] == free_before, "the allocation-free entry point changed the free device memory"
+        _call.warm = True
     else:
         n = lib.nf_hash_encode_bwd_workspace_bytes(x.shape[0], geom, L_.dtype_code(do.dtype), flags)
         ws = torch.empty(max(n, 16), dtype=torch.uint8, device=DEV)
@@ -30,6 +38,9 @@ def _call(lib, L_, static, x, do, E, geom, pi, flags=0):
                                     do.stride(0), de.data_ptr(), x.shape[0], geom, pi.data_ptr(), 1.0, ws.data_ptr(), n, flags, stream)
     torch.cuda.synchronize()
     return rc, de
+
+
+_call.warm = False
 
 
 def test_static_scratch_backward_matches_the_workspace_backward():

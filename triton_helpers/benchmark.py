@@ -1,4 +1,4 @@
-from triton_helpers_amd.benchmark import *  # noqa: F401,F403
-from triton_helpers_amd import benchmark as _impl
-
-globals().update({k: v for k, v in vars(_impl).items() if not k.startswith('__')})
+"""Alias of ``triton_helpers_amd.benchmark`` (the benchmark / profile command line of the layers)."""
+from triton_helpers_amd.benchmark import (  # noqa: F401
+    DTYPES, MODES, Table, Timing, Workload, axis_values, profile_once, run_cli, step_closure, sweep, time_calls,
+)

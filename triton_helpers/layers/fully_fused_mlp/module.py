@@ -1,3 +1,2 @@
-from triton_helpers_amd.layers.fully_fused_mlp import module as _impl
-
-globals().update({k: v for k, v in vars(_impl).items() if not k.startswith('__')})
+"""Alias of ``triton_helpers_amd.layers.fully_fused_mlp.module``."""
+from triton_helpers_amd.layers.fully_fused_mlp.module import FullyFusedMLP  # noqa: F401

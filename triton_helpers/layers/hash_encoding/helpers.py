@@ -1,4 +1,5 @@
-from triton_helpers_amd.layers.hash_encoding.helpers import *  # noqa: F401,F403
-from triton_helpers_amd.layers.hash_encoding import helpers as _impl
-
-globals().update({k: v for k, v in vars(_impl).items() if not k.startswith('__')})
+"""Alias of ``triton_helpers_amd.layers.hash_encoding.helpers`` (level geometry under the reference's names)."""
+from triton_helpers_amd.layers.hash_encoding.helpers import (  # noqa: F401
+    compute_b, compute_embedding_counts, compute_level_embedding_offset, compute_resolutions, get_first_hash_level,
+    level_geometry, seek_to_level_embeddings, total_rows,
+)

@@ -24,6 +24,7 @@ NF_HASH_FORCE_GENERIC = 1
 NF_HASH_FORCE_ATOMIC = 2
 NF_HASH_FORCE_PLANES = 4
 NF_HASH_FWD_STAGED = 8
+NF_ADAM_CLEAR_GRAD, NF_ADAM_SKIP_NONFINITE = 1, 2
 
 _DTYPE_CODE = {torch.float32: NF_F32, torch.float16: NF_F16, torch.bfloat16: NF_BF16}
 
@@ -101,7 +102,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.nf_hash_check_host.restype = c_int
     lib.nf_hash_check_host.argtypes = [P, I64, POINTER(HashGeom), P, c_float, I, P, P, P]
     lib.nf_table_adam_step.restype = c_int
-    lib.nf_table_adam_step.argtypes = [P, I, P, P, P, P, I64, I64, c_float, c_float, c_float, c_float, c_float, c_float, I, P]
+    lib.nf_table_adam_step.argtypes = [P, I, P, P, P, P, I64, I64, c_float, c_float, c_float, c_float, c_float, c_float, I, P, P]
     lib.nf_mlp_fwd.restype = c_int
     lib.nf_mlp_fwd.argtypes = [P, I64, P, I64, P, P, P, P, P, P, I64, I, I, I, I, I, I, I, P, I64, P]
     lib.nf_mlp_bwd_rounded.restype = c_int

@@ -140,15 +140,16 @@ int launch_mlp_bwdn(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
 int launch_mlp_bwd2_w8(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
 // The same with the weight and bias gradients summed in a fixed order and written, rounded to `dtype`, into out[6]
 // (dw_in, db_in, dw_hid, db_hid, dw_out, db_out; NULL entries skipped); workspace: mlp_bwd2_w8_rounded_bytes().
+// Also covers the shapes of launch_mlp_bwd2_ws.
 size_t mlp_bwd2_w8_rounded_bytes(int d_in, int d_hidden, int d_out);
 int launch_mlp_bwd2_w8_rounded(const MlpArgs& a, int dtype, void* const out[6], void* workspace, hipStream_t s, bool* handled);
 
 
 // One hidden layer, width 64, ReLU, with d_in > 32 or d_out > 16 (aligned rows, extents below 2^31 bytes): chain and
 // gradient waves (fused_mlp_bwd2_ws.hip).  *handled = false: not such a call, nothing was launched.
-int launch_mlp_bwd2_ws(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
+int launch_mlp_bwd2_ws(const MlpArgs& a, int dtype, hipStream_t s, bool* handled, int* blocks_out = nullptr);
 
-// The forward of that shape (fused_mlp_fwd2.hip).  *handled = false: not that shape, nothing was launched.
+// The forward of one-hidden-layer ReLU networks of width 64 with aligned rows (fused_mlp_fwd2.hip).  *handled = false: not that shape, nothing was launched.
 int launch_mlp_fwd2(const MlpArgs& a, int dtype, hipStream_t s, bool* handled);
 
 // float32 storage and float32 products (fused_mlp_f32.hip).  The backward needs mlp32_bwd_workspace_bytes of scratch.

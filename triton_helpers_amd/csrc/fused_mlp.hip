@@ -885,6 +885,6 @@ extern "C" int nf_mlp_bwd_rounded(const void* x, int64_t x_stride, const void* d
   bool handled = false;
   const int rc = launch_mlp_bwd2_w8_rounded(a, dtype, out, workspace, (hipStream_t)stream, &handled);
   if (rc != 0 || handled) return rc;
-  return fail(NF_EUNSUPPORTED, "rounded weight gradients: built for one hidden-to-hidden layer, d_hidden = 64, d_in <= 32, d_out <= 16, "
-                               "ReLU and 8-byte aligned rows (nothing was launched; use nf_mlp_bwd)");
+  return fail(NF_EUNSUPPORTED, "rounded weight gradients: built for one hidden-to-hidden layer, d_hidden = 64, d_in <= 64, d_out <= 64, "
+                               "ReLU, 8-byte aligned rows and (beyond d_in 32 / d_out 16) x stored like the weights (nothing was launched; use nf_mlp_bwd)");
 }

@@ -124,6 +124,14 @@ constexpr uint32_t OUT_OF_RANGE = 0x80000000u;
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t rows_rsrc(const void* base, int64_t rows, int64_t stride) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)(rows * stride * 2), 0x00020000);
 }
+// What a launch needs of a tensor's extent for these 32-bit offsets to be safe: the tensor itself below 2^31 bytes
+// (the descriptor's range check then catches every row past the end), and the furthest row any lane ever addresses
+// -- the rows a partly filled last chunk pads to, and the chunk the prefetch asks for one grid-stride ahead (at most
+// 256 workgroups x 12 waves x 32 rows) -- still below 2^32 bytes, so that no offset wraps back into range.
+inline bool rows_in_reach(int64_t rows, int64_t stride) {
+  const int64_t ahead = (int64_t)256 * 12 * 32 + 64;
+  return rows * stride * 2 <= (((int64_t)1 << 31) - 1) && (rows + ahead) * stride * 2 + 128 < ((int64_t)1 << 32);
+}
 // byte offset of the piece (columns col .. col + 3) of row `row` of the first chunk
 __device__ __forceinline__ uint32_t piece_offset(int row, int col, int width, int64_t stride) {
   return col < width ? (uint32_t)(((int64_t)row * stride + col) * 2) : OUT_OF_RANGE;

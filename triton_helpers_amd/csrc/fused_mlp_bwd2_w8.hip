@@ -95,12 +95,11 @@ static int launch2_w8(const MlpArgs& a0, hipStream_t s, int* blocks_out = nullpt
 static bool w8_shape(const MlpArgs& a, int dtype) {
   const int xc_other = dtype == NF_BF16 ? 1 : 2;
   const auto rows8 = [](const void* p, int64_t stride) { return (uintptr_t)p % 8 == 0 && stride % 4 == 0; };
-  const int64_t limit = ((int64_t)1 << 31) - 1;  // bytes a buffer descriptor's 32-bit offsets reach
   const bool shape = a.depth == 2 && a.d_hidden == 64 && a.d_in <= 32 && a.d_out <= 16 && a.act == NF_ACT_RELU && a.in_act == NF_ACT_NONE &&
                      (a.x_conv == 0 || a.x_conv == xc_other);
   const bool aligned = a.d_in % 4 == 0 && a.d_out % 4 == 0 && rows8(a.x, a.x_stride) && rows8(a.dy, a.dy_stride) &&
                        (a.dx == nullptr || rows8(a.dx, a.dx_stride));
-  const bool in_reach = a.rows * a.x_stride * 2 <= limit && a.rows * a.dy_stride * 2 <= limit && (a.dx == nullptr || a.rows * a.dx_stride * 2 <= limit);
+  const bool in_reach = rows_in_reach(a.rows, a.x_stride) && rows_in_reach(a.rows, a.dy_stride) && (a.dx == nullptr || rows_in_reach(a.rows, a.dx_stride));
   return shape && aligned && in_reach;
 }
 
@@ -113,8 +112,7 @@ int launch_mlp_bwd2_w8(const MlpArgs& a, int dtype, hipStream_t s, bool* handled
 
 int launch_mlp_bwd2_w8_rounded(const MlpArgs& a0, int dtype, void* const out[6], void* workspace, hipStream_t s, bool* handled) {
   *handled = false;
-  if (!w8_shape(a0, dtype)) return 0;
-  *handled = true;
+  const bool decoder = w8_shape(a0, dtype);
   MlpArgs a = a0;
   const size_t stride = slot_floats(a.d_in, a.d_hidden, a.d_out);
   a.partials = reinterpret_cast<float*>(workspace);
@@ -126,7 +124,14 @@ int launch_mlp_bwd2_w8_rounded(const MlpArgs& a0, int dtype, void* const out[6],
   a.db_hid = out[3] ? any : nullptr;
   a.db_out = out[5] ? any : nullptr;
   int blocks = 0;
-  if (int rc = dtype == NF_BF16 ? launch2_w8<BF16>(a, s, &blocks) : launch2_w8<F16>(a, s, &blocks)) return rc;
+  if (decoder) {
+    *handled = true;
+    if (int rc = dtype == NF_BF16 ? launch2_w8<BF16>(a, s, &blocks) : launch2_w8<F16>(a, s, &blocks)) return rc;
+  } else {
+    // the 64-wide inputs / outputs: chain and gradient waves, at most one workgroup per CU (fewer than ROUNDED_SLOTS)
+    const int rc = launch_mlp_bwd2_ws(a, dtype, s, handled, &blocks);
+    if (rc != 0 || !*handled) return rc;
+  }
   RoundedPieces pc;
   const int H = a.d_hidden;
   const int sizes[6] = {H * a.d_in, H * H, a.d_out * H, H, H, a.d_out};

@@ -34,12 +34,12 @@ static int dispatch_ws(const MlpArgs& a, hipStream_t s, int* blocks_out) {
 }
 
 // Covers depth 2, d_hidden 64, ReLU, x stored like the weights, 8-byte aligned rows, extents a buffer descriptor
-// reaches, and d_in > 32 or d_out > 16 (the decoder shape has a kernel of its own).
-int launch_mlp_bwd2_ws(const MlpArgs& a, int dtype, hipStream_t s, bool* handled) {
+// reaches, and d_in > 32 or d_out > 16 (the decoder shape has a kernel of its own).  *blocks_out: workgroups launched
+// (with MlpArgs::partials set, each stores its sums into the slot of its index).
+int launch_mlp_bwd2_ws(const MlpArgs& a, int dtype, hipStream_t s, bool* handled, int* blocks_out) {
   *handled = false;
   const auto rows8 = [](const void* p, int64_t stride) { return (uintptr_t)p % 8 == 0 && stride % 4 == 0; };
-  // byte offsets are 32 bits: the rows of the last, partly filled chunk and one piece beyond stay below 2^31
-  const auto reach = [&](int64_t stride) { return (a.rows + 32) * stride * 2 + 128 < ((int64_t)1 << 31); };
+  const auto reach = [&](int64_t stride) { return rows_in_reach(a.rows, stride); };
   const bool shape = a.depth == 2 && a.d_hidden == 64 && a.d_in <= 64 && a.d_out <= 64 && (a.d_in > 32 || a.d_out > 16) &&
                      a.act == NF_ACT_RELU && a.in_act == NF_ACT_NONE && a.x_conv == 0;
   const bool aligned = a.d_in % 4 == 0 && a.d_out % 4 == 0 && rows8(a.x, a.x_stride) && rows8(a.dy, a.dy_stride) &&
@@ -47,7 +47,7 @@ int launch_mlp_bwd2_ws(const MlpArgs& a, int dtype, hipStream_t s, bool* handled
   const bool in_reach = reach(a.x_stride) && reach(a.dy_stride) && (a.dx == nullptr || reach(a.dx_stride));
   if (!(shape && aligned && in_reach)) return 0;
   *handled = true;
-  return dtype == NF_BF16 ? dispatch_ws<BF16>(a, s, nullptr) : dispatch_ws<F16>(a, s, nullptr);
+  return dtype == NF_BF16 ? dispatch_ws<BF16>(a, s, blocks_out) : dispatch_ws<F16>(a, s, blocks_out);
 }
 
 }  // namespace nf

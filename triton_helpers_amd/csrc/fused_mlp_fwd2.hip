@@ -1,5 +1,6 @@
-// The forward of the decoder / benchmark shape -- d_in <= 32, d_hidden = 64, one hidden-to-hidden layer, d_out <= 16,
-// ReLU, 8-byte aligned rows -- as a kernel of its own: eight waves per workgroup, the chunk body one basic block (no
+// The forward of one-hidden-layer ReLU networks of width 64 (d_in <= 64, d_out <= 64; the decoder / benchmark shape
+// 32 -> 64 -> 64 -> 16 and the 64-wide shapes of the reference's own benchmark), 8-byte aligned rows, as a kernel of
+// its own per (input, output) width class: twelve waves per workgroup, the chunk body one basic block (no
 // run-time tests of activation, depth, alignment or row count inside it), rows addressed through buffer descriptors
 // (reads past the end return zero, stores past it are dropped), the next chunk's rows requested before this one's
 // products.  Everything else stays on mlp_fwd_k (fused_mlp.hip), which loops over a run-time depth.
@@ -16,10 +17,14 @@ namespace nf {
 #define NF_FWD2_WAVES 12
 #endif
 
-// XC: how x is stored (MlpArgs::x_conv).
-template <typename T, int XC>
-__global__ __launch_bounds__(64 * NF_FWD2_WAVES) void mlp_fwd2_k(MlpArgs a) {
-  constexpr int KIN = 32, HP = 64, OUTP = 16, NT = 2, WAVES = NF_FWD2_WAVES;
+// XC: how x is stored (MlpArgs::x_conv); KIN / OUTP: d_in / d_out rounded up to 32 or 64 / 16 or 64.
+// Twelve waves where the weight fragments (held in registers across chunks) leave room for three waves per SIMD,
+// eight for the 64-wide inputs / outputs.
+constexpr int fwd2_waves(int kin, int outp) { return (kin == 32 && outp == 16) ? NF_FWD2_WAVES : 8; }
+
+template <typename T, int XC, int KIN = 32, int OUTP = 16>
+__global__ __launch_bounds__(64 * fwd2_waves(KIN, OUTP)) void mlp_fwd2_k(MlpArgs a) {
+  constexpr int HP = 64, NT = 2, WAVES = fwd2_waves(KIN, OUTP);
   constexpr int KC_IN = KIN / 32, KC_H = HP / 32, MT_H = HP / 16, MT_O = OUTP / 16;
   constexpr int ROWS = 16 * NT;
   constexpr int nthreads = 64 * WAVES;
@@ -34,7 +39,9 @@ __global__ __launch_bounds__(64 * NF_FWD2_WAVES) void mlp_fwd2_k(MlpArgs a) {
   for (int kc = 0; kc < KC_IN; ++kc)
 #pragma unroll
     for (int h = 0; h < 2; ++h) off_x[kc][h] = piece_offset(lane & 15, 32 * kc + 16 * h + 4 * (lane >> 4), a.d_in, a.x_stride);
-  const uint32_t off_y = piece_offset(lane & 15, 4 * (lane >> 4), a.d_out, a.y_stride);
+  uint32_t off_y[MT_O];
+#pragma unroll
+  for (int mt = 0; mt < MT_O; ++mt) off_y[mt] = piece_offset(lane & 15, 16 * mt + 4 * (lane >> 4), a.d_out, a.y_stride);
   auto load_x = [&](int64_t chunk, int nt, int kc) {
     const uint32_t at = (uint32_t)((chunk * ROWS + 16 * nt) * a.x_stride * 2);
     const buf_v2u lo = __builtin_amdgcn_raw_buffer_load_b64(rs_x, off_x[kc][0] + at, 0, 0);
@@ -91,27 +98,29 @@ __global__ __launch_bounds__(64 * NF_FWD2_WAVES) void mlp_fwd2_k(MlpArgs a) {
       }
     layer_nt<T, NT, MT_O, KC_H, 1>(acc, h, f_out, bias_out, lane);
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      buf_v2u o;
-      o[0] = pack2<T>(acc[nt][0][0], acc[nt][0][1]);
-      o[1] = pack2<T>(acc[nt][0][2], acc[nt][0][3]);
-      __builtin_amdgcn_raw_buffer_store_b64(o, rs_y, off_y + (uint32_t)((chunk * ROWS + 16 * nt) * a.y_stride * 2), 0, 0);
-    }
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT_O; ++mt) {
+        buf_v2u o;
+        o[0] = pack2<T>(acc[nt][mt][0], acc[nt][mt][1]);
+        o[1] = pack2<T>(acc[nt][mt][2], acc[nt][mt][3]);
+        __builtin_amdgcn_raw_buffer_store_b64(o, rs_y, off_y[mt] + (uint32_t)((chunk * ROWS + 16 * nt) * a.y_stride * 2), 0, 0);
+      }
   }
 }
 
-template <typename T>
+template <typename T, int KIN, int OUTP>
 static int launch_fwd2(const MlpArgs& a0, hipStream_t s) {
   MlpArgs a = a0;
-  constexpr int WAVES = NF_FWD2_WAVES, ROWS = 32;
-  constexpr size_t LDS = ((size_t)4 * 1 + 4 * 2 + 1 * 2) * 1024 + (size_t)(64 + 64 + 16) * 4;
+  constexpr int WAVES = fwd2_waves(KIN, OUTP), ROWS = 32;
+  constexpr size_t LDS = ((size_t)4 * (KIN / 32) + 4 * 2 + (OUTP / 16) * 2) * 1024 + (size_t)(64 + 64 + OUTP) * 4;
   a.waves = WAVES;
   const int64_t chunks = (a.rows + ROWS - 1) / ROWS;
   int64_t blocks = (chunks + WAVES - 1) / WAVES;
   const int64_t cap = (int64_t)device_cus() * NF_FWD2_WG_PER_CU;
   if (blocks > cap) blocks = cap;
   constexpr int XC_OTHER = T::code == NF_BF16 ? 1 : 2;
-  const void* kern = a.x_conv == 0 ? (const void*)mlp_fwd2_k<T, 0> : (const void*)mlp_fwd2_k<T, XC_OTHER>;
+  const void* kern = a.x_conv == 0 ? (const void*)mlp_fwd2_k<T, 0, KIN, OUTP> : (const void*)mlp_fwd2_k<T, XC_OTHER, KIN, OUTP>;
   void* args[] = {(void*)&a};
   const hipError_t e = hipLaunchKernel(kern, dim3((unsigned)blocks), dim3(64 * WAVES), args, LDS, s);
   if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(mlp_fwd2): %s", hipGetErrorString(e));
@@ -122,14 +131,18 @@ int launch_mlp_fwd2(const MlpArgs& a, int dtype, hipStream_t s, bool* handled) {
   *handled = false;
   const int xc_other = dtype == NF_BF16 ? 1 : 2;
   const auto rows8 = [](const void* p, int64_t stride) { return (uintptr_t)p % 8 == 0 && stride % 4 == 0; };
-  const int64_t limit = ((int64_t)1 << 31) - 1;  // bytes a buffer descriptor's 32-bit offsets reach
-  const bool shape = a.depth == 2 && a.d_hidden == 64 && a.d_in <= 32 && a.d_out <= 16 && a.act == NF_ACT_RELU && a.in_act == NF_ACT_NONE &&
+  const bool shape = a.depth == 2 && a.d_hidden == 64 && a.d_in <= 64 && a.d_out <= 64 && a.act == NF_ACT_RELU && a.in_act == NF_ACT_NONE &&
                      (a.x_conv == 0 || a.x_conv == xc_other);
   const bool aligned = a.d_in % 4 == 0 && a.d_out % 4 == 0 && rows8(a.x, a.x_stride) && rows8(a.y, a.y_stride);
-  const bool in_reach = a.rows * a.x_stride * 2 <= limit && a.rows * a.y_stride * 2 <= limit;
+  const bool in_reach = rows_in_reach(a.rows, a.x_stride) && rows_in_reach(a.rows, a.y_stride);
   if (!shape || !aligned || !in_reach) return 0;
   *handled = true;
-  return dtype == NF_BF16 ? launch_fwd2<BF16>(a, s) : launch_fwd2<F16>(a, s);
+  const bool wide_in = a.d_in > 32, wide_out = a.d_out > 16;
+#define NF_FWD2_DISPATCH(T)                                          \
+  (wide_in ? (wide_out ? launch_fwd2<T, 64, 64>(a, s) : launch_fwd2<T, 64, 16>(a, s)) \
+           : (wide_out ? launch_fwd2<T, 32, 64>(a, s) : launch_fwd2<T, 32, 16>(a, s)))
+  return dtype == NF_BF16 ? NF_FWD2_DISPATCH(BF16) : NF_FWD2_DISPATCH(F16);
+#undef NF_FWD2_DISPATCH
 }
 
 }  // namespace nf

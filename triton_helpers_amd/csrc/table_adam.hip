@@ -8,6 +8,9 @@
 // Arithmetic is torch.optim.Adam's (no amsgrad, L2 weight decay added to the gradient):
 //   g = grad / grad_scale (+ weight_decay * p);  m = b1 m + (1 - b1) g;  v = b2 v + (1 - b2) g g
 //   p -= (lr / (1 - b1^t)) * m / (sqrt(v) / sqrt(1 - b2^t) + eps)
+// Loss-scaled fp16 training meets overflowed gradients (the binned backward marks the rows of such a level with NaN):
+// with NF_ADAM_SKIP_NONFINITE an element whose gradient is inf or NaN keeps its parameter and moments (what a skipped
+// step does for it), and *found_nonfinite, when given, is set so that the caller can lower its loss scale.
 // A pure stream: 34 bytes per element with a master copy and a 16-bit table.
 #include "nf_common.h"
 
@@ -16,11 +19,18 @@ namespace nf {
 template <typename TT, bool MASTER>
 __global__ __launch_bounds__(256) void table_adam_k(typename TT::storage* table, float* master, float* grad, float* m, float* v,
                                                     int64_t n, float step_size, float inv_sqrt_bc2, float b1, float b2, float eps,
-                                                    float weight_decay, float inv_scale, int clear_grad) {
+                                                    float weight_decay, float inv_scale, int flags, int* found_nonfinite) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
     float p = MASTER ? master[i] : TT::to_f32(table[i]);
     float g = grad[i] * inv_scale;
+    if (!(fabsf(g) <= 3.4028234e38f)) {  // inf or NaN
+      if (found_nonfinite != nullptr) *found_nonfinite = 1;
+      if (flags & NF_ADAM_SKIP_NONFINITE) {
+        if (flags & NF_ADAM_CLEAR_GRAD) grad[i] = 0.0f;
+        continue;
+      }
+    }
     if (weight_decay != 0.0f) g = fmaf(weight_decay, p, g);
     const float mi = fmaf(b1, m[i], (1.0f - b1) * g);
     const float vi = fmaf(b2, v[i], (1.0f - b2) * g * g);
@@ -30,7 +40,7 @@ __global__ __launch_bounds__(256) void table_adam_k(typename TT::storage* table,
     v[i] = vi;
     if (MASTER) master[i] = p;
     table[i] = TT::from_f32(p);
-    if (clear_grad) grad[i] = 0.0f;
+    if (flags & NF_ADAM_CLEAR_GRAD) grad[i] = 0.0f;
   }
 }
 
@@ -40,7 +50,7 @@ using namespace nf;
 
 extern "C" int nf_table_adam_step(void* table, int table_dtype, float* master, float* grad, float* exp_avg, float* exp_avg_sq,
                                   int64_t n_elems, int64_t step, float lr, float beta1, float beta2, float eps, float weight_decay,
-                                  float grad_scale, int clear_grad, void* stream) {
+                                  float grad_scale, int flags, int* found_nonfinite, void* stream) {
   NF_REQUIRE(dtype_ok(table_dtype), NF_EINVAL, "unknown dtype code %d", table_dtype);
   NF_REQUIRE(n_elems >= 0, NF_EINVAL, "n_elems negative");
   NF_REQUIRE(step >= 1, NF_EINVAL, "step=%lld: steps count from 1", (long long)step);
@@ -58,10 +68,10 @@ extern "C" int nf_table_adam_step(void* table, int table_dtype, float* master, f
   do {                                                                                                                             \
     if (master != nullptr)                                                                                                         \
       hipLaunchKernelGGL((table_adam_k<TT, true>), grid, block, 0, s, (TT::storage*)table, master, grad, exp_avg, exp_avg_sq, n_elems, \
-                         step_size, inv_sqrt_bc2, beta1, beta2, eps, weight_decay, inv_scale, clear_grad);                          \
+                         step_size, inv_sqrt_bc2, beta1, beta2, eps, weight_decay, inv_scale, flags, found_nonfinite);          \
     else                                                                                                                           \
       hipLaunchKernelGGL((table_adam_k<TT, false>), grid, block, 0, s, (TT::storage*)table, master, grad, exp_avg, exp_avg_sq, n_elems, \
-                         step_size, inv_sqrt_bc2, beta1, beta2, eps, weight_decay, inv_scale, clear_grad);                          \
+                         step_size, inv_sqrt_bc2, beta1, beta2, eps, weight_decay, inv_scale, flags, found_nonfinite);          \
   } while (0)
   if (table_dtype == NF_F32) NF_ADAM_LAUNCH(F32);
   else if (table_dtype == NF_F16) NF_ADAM_LAUNCH(F16);

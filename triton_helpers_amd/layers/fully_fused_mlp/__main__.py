@@ -3,46 +3,40 @@
 Dimensions as in the reference: ``x (32, L, D)``, every layer ``D`` wide, ``H`` hidden-to-hidden layers.  Providers: a
 chain of ``F.linear`` + ReLU calls (``baseline``) and the fused kernels (``fully-fused``).
 """
-from dataclasses import dataclass
-from typing import Dict, Optional
-
 import torch
 import torch.nn.functional as F
-from torch import Tensor
 
-from ...benchmark import CLI, KernelExecutor
+from ...benchmark import Workload, run_cli
 from .kernel import fully_fused_mlp
 
 
-@dataclass
-class Baseline(KernelExecutor):
-    def prepare_inputs(self, L: int, D: int, H: int, **kwargs) -> Dict[str, Optional[Tensor]]:
-        device, dtype, grad = kwargs.get("device", "cuda"), kwargs.get("dtype", torch.float32), kwargs.get("requires_grad", False)
-        mk = lambda *shape: (self.randn(shape, device=device) / D**0.5).to(dtype).requires_grad_(grad)  # noqa: E731
-        x = self.randn((32, L, D), device=device).to(dtype).requires_grad_(grad)
-        return {
-            "x": x, "w_in": mk(D, D), "b_in": mk(D), "w_out": mk(D, D), "b_out": mk(D),
-            "w_hid": mk(D * H, D) if H >= 1 else None, "b_hid": mk(H, D) if H >= 1 else None, "H": H,
-        }
+def _inputs(L, D, H, device="cuda", dtype=torch.float32, requires_grad=False):
+    def leaf(*shape, scale=1.0):
+        return (torch.randn(shape, device=device) * scale).to(dtype).requires_grad_(requires_grad)
 
-    def forward(self, x, w_in, b_in, w_out, b_out, w_hid, b_hid, H) -> Tensor:
-        x = F.relu(F.linear(x, w_in, b_in))
-        D = w_in.shape[0]
-        for i in range(H):
-            x = F.relu(F.linear(x, w_hid[D * i : D * (i + 1)], b_hid[i]))
-        return F.linear(x, w_out, b_out)
+    s = D**-0.5
+    return {
+        "x": leaf(32, L, D), "w_in": leaf(D, D, scale=s), "b_in": leaf(D, scale=s), "w_out": leaf(D, D, scale=s), "b_out": leaf(D, scale=s),
+        "w_hid": leaf(D * H, D, scale=s) if H >= 1 else None, "b_hid": leaf(H, D, scale=s) if H >= 1 else None,
+    }
 
 
-@dataclass
-class Native(Baseline):
-    def forward(self, x, w_in, b_in, w_out, b_out, w_hid, b_hid, H) -> Tensor:
-        return fully_fused_mlp(x, w_in, b_in, w_out, b_out, w_hid, b_hid)
+def _linear_chain(x, w_in, b_in, w_out, b_out, w_hid, b_hid):
+    D = w_in.shape[0]
+    h = F.relu(F.linear(x, w_in, b_in))
+    for k in range(0 if w_hid is None else w_hid.shape[0] // D):
+        h = F.relu(F.linear(h, w_hid[D * k : D * (k + 1)], b_hid[k]))
+    return F.linear(h, w_out, b_out)
+
+
+def _fused(x, w_in, b_in, w_out, b_out, w_hid, b_hid):
+    return fully_fused_mlp(x, w_in, b_in, w_out, b_out, w_hid, b_hid)
 
 
 def main(argv=None):
-    return CLI.entrypoint(
+    return run_cli(
         "MLP",
-        [Baseline("baseline"), Native("fully-fused")],
+        [Workload("baseline", _inputs, _linear_chain), Workload("fully-fused", _inputs, _fused)],
         dims={
             "L": ((512, 2048, 8192, 16384, 32768, 65536), "values"),
             "D": (64, "values"),

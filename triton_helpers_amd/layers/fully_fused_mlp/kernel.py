@@ -232,7 +232,9 @@ class _fully_fused_mlp(Function):
             x = x.to(w_in.dtype)  # only the one-hidden-layer ReLU backward converts on the fly
         do2 = _rows2d(do, D_out)
         need_dx = ctx.needs_input_grad[0]
-        if (not wide and w_in.dtype != torch.float32 and ctx.depth == 2 and D_hidden == 64 and D_in <= 32 and D_out <= 16
+        decoder = D_in <= 32 and D_out <= 16  # the wider shapes need x in the parameters' dtype
+        if (not wide and w_in.dtype != torch.float32 and ctx.depth == 2 and D_hidden == 64 and D_in <= 64 and D_out <= 64
+                and (decoder or x.dtype == w_in.dtype)
                 and D_in % 4 == 0 and D_out % 4 == 0 and ctx.activation == "relu" and do2.shape[0] > 0):
             done = _backward_rounded(x, do2, w_in, b_in, w_out, b_out, w_hid, b_hid, need_dx, D_in, D_hidden, D_out)
             if done is not None:

@@ -4,38 +4,31 @@ Dimensions as in the reference: a batch of ``(32, L, D)`` points, ``F`` features
 levels with resolutions ``X .. Y``.  The provider is this package's kernel; the reference's comparison provider
 (tiny-cuda-nn) does not exist for this GPU.
 """
-from dataclasses import dataclass
-from typing import Any, Dict
-
 import torch
-from torch import Tensor
 
-from ...benchmark import CLI, KernelExecutor
+from ...benchmark import Workload, run_cli
 from .kernel import hash_encoding
 from .module import HashEncoding
 
 
-@dataclass
-class Native(KernelExecutor):
-    @torch.no_grad()
-    def prepare_inputs(self, L: int, D: int, F: int, T: int, N: int, X: int, Y: int, **kwargs) -> Dict[str, Any]:
-        device = kwargs.get("device", "cuda")
-        torch.random.manual_seed(0)
-        x = self.rand((32, L, D), device=device)
-        layer = HashEncoding(T, N, D, F, X, Y).to(device)
-        e = layer.embeddings.detach().to(kwargs.get("dtype", torch.float32))
-        e.requires_grad = kwargs.get("requires_grad", False)
-        return {"x": x, "e": e, "pi": layer.pi.detach(), "geometry": (T, X, Y, N)}
+@torch.no_grad()
+def _inputs(L, D, F, T, N, X, Y, device="cuda", dtype=torch.float32, requires_grad=False):
+    torch.random.manual_seed(0)
+    layer = HashEncoding(T, N, D, F, X, Y).to(device)
+    table = layer.embeddings.detach().to(dtype)
+    table.requires_grad = requires_grad
+    return {"x": torch.rand((32, L, D), device=device), "table": table, "pi": layer.pi.detach(), "geometry": (T, X, Y, N)}
 
-    def forward(self, x: Tensor, e: Tensor, pi: Tensor, geometry) -> Tensor:
-        T, X, Y, N = geometry
-        return hash_encoding(x, e, None, pi, T, X, Y, N)
+
+def _encode(x, table, pi, geometry):
+    T, X, Y, N = geometry
+    return hash_encoding(x, table, None, pi, T, X, Y, N)
 
 
 def main(argv=None):
-    return CLI.entrypoint(
+    return run_cli(
         "InstantNGP Hash Encoding",
-        [Native("hip-hash")],
+        [Workload("hip-hash", _inputs, _encode)],
         dims={
             "L": ((512, 2048, 8192, 16384, 32768, 65536, 65536 * 2), "values"),
             "D": (3, "values"),

@@ -48,48 +48,6 @@ _FLAGS = 0  # test hook: _lib.NF_HASH_FORCE_GENERIC / NF_HASH_FORCE_ATOMIC / NF_
 
 
 # ---------------------------------------------------------------------------
-# CPU checking utilities with the reference's names (reference kernel.py:443-502).
-# No operator of this package calls them; tests of user code import them.
-# ---------------------------------------------------------------------------
-def _cpu_create_corner_offsets(d: int, **kwargs) -> Tensor:
-    bits = torch.arange(2**d, dtype=torch.int32)[:, None] >> torch.arange(d, dtype=torch.int32)[None, :]
-    return (bits & 1).to(**kwargs)
-
-
-@torch.no_grad()
-def _cpu_embedding_lookup(x: Tensor, pi: Tensor, D: int, T_l: int, N_l: int) -> Tensor:
-    cell = torch.floor(x * N_l).to(torch.int64)
-    corners = cell[:, None, :] + _cpu_create_corner_offsets(D, device=cell.device, dtype=torch.int64)[None]
-    if (N_l + 1) ** D <= T_l:
-        strides = N_l ** torch.arange(D, device=pi.device)
-        return (corners * strides).sum(-1)
-    terms = corners * pi
-    h = terms[..., 0]
-    for i in range(1, D):
-        h = torch.bitwise_xor(h, terms[..., i])
-    return h % T_l
-
-
-def _cpu_interpolate(x: Tensor, e: Tensor, D: int, N_l: int) -> Tensor:
-    pos = x * N_l
-    frac = (pos - torch.floor(pos).to(torch.int64))[:, None, :]
-    offsets = _cpu_create_corner_offsets(D, device=x.device, dtype=torch.int64)
-    w = torch.where(offsets == 0, 1 - frac, frac).prod(-1)
-    return (w[..., None] * e).sum(1)
-
-
-def _cpu_hash_encoding(x: Tensor, e: Tensor, pi: Tensor, o: Tensor, D: int, F: int, T: int, L: int, N_min: int, N_max: int) -> Tensor:
-    assert 1 <= D <= 3, "D must be 1, 2, or 3"
-    res = compute_resolutions(L, N_min, N_max)
-    counts = compute_embedding_counts(L, T, D, N_min, N_max)
-    for l in range(L):
-        rows = _cpu_embedding_lookup(x, pi, D, counts[l], res[l])
-        level = seek_to_level_embeddings(e, l, L, T, D, N_min, N_max)
-        o[..., l * F : (l + 1) * F] = _cpu_interpolate(x, level[rows], D, res[l])
-    return o
-
-
-# ---------------------------------------------------------------------------
 # Launch helpers
 # ---------------------------------------------------------------------------
 _default_primes: Dict[torch.device, Tensor] = {}
