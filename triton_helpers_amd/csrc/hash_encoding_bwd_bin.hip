@@ -22,6 +22,12 @@
 // bit of x.  When they do not (bin border, 13 trailing ones in x) the pair becomes two records with one zero weight
 // each.  The count and fill kernels apply the same rule, so their record counts agree.
 //
+// Dense levels whose cells span less than a bin (3-D, 16-bit gradients) take ONE record per point and level instead
+// of four: {row of corner 0 relative to the bin, the three cell fractions in 18 / 16 / 16-bit fixed point, gradient
+// pair}, still 12 bytes.  All eight corners lie within  res^2 + res + 1  rows of the first, so they fall into one bin
+// or two neighbouring ones; a cell on a bin border is sent to both, and each accumulation takes the corners inside its
+// own bin.  The accumulation rebuilds the eight trilinear weights from the fractions (each off by at most 2^-17).
+//
 // Integer accumulation: fill also finds max |dout| per level; with 2^e the power of two above it, a contribution
 // w * g is accumulated as round(w * g * 2^(30 - e)), below 2^30 in magnitude, so a task's records cannot
 // overflow 64 bits, the rounding is 2^-30 of the level's largest gradient per contribution, and a task's sum does
@@ -52,7 +58,16 @@ struct BinPlan {
   int n_levels;
   int nbins[NF_MAX_LEVELS];
   int binbase[NF_MAX_LEVELS + 1];  // first global bin of the level
+  int cell[NF_MAX_LEVELS];         // the level's records are cells (one per point) instead of x-pairs
 };
+
+// cell record = {u | qx << 14,  qy | qz << 16,  packed gradient pair}: u = row of corner 0 minus the bin's first row,
+// plus BIN_ROWS (the cell may start in the bin below); q* = the cell fractions in 18 / 16 / 16-bit fixed point
+constexpr float CELL_QX = 262143.0f, CELL_QYZ = 65535.0f;
+__device__ __forceinline__ uint3 make_cell_record(int32_t rel_row, const float (&fr)[3], uint32_t packed) {
+  const uint32_t qx = (uint32_t)(fr[0] * CELL_QX + 0.5f), qy = (uint32_t)(fr[1] * CELL_QYZ + 0.5f), qz = (uint32_t)(fr[2] * CELL_QYZ + 0.5f);
+  return make_uint3((uint32_t)(rel_row + BIN_ROWS) | qx << 14, qy | qz << 16, packed);
+}
 
 // workspace (32-bit words): hist[NB] | gmax[32] | cursor[NB] | n_tasks, pad[3] | tasks[max_tasks][4] |
 // wg_counts[workgroups][NB] | records[R][3]      (hist and gmax are cleared together)
@@ -248,12 +263,30 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_count_k(const void* 
   for (int l = 0; l < bp.n_levels; ++l) {
     uint32_t* cnt = lh + bp.binbase[l];
     const int nb = bp.nbins[l];
+    const bool cells = D == 3 && bp.cell[l];
     if (nb == 1) {
       if (valid) {
         const unsigned long long m = __ballot(true);
-        if (lane == __ffsll((long long)m) - 1) atomicAdd(cnt, (uint32_t)PAIRS * (uint32_t)__popcll(m));
+        if (lane == __ffsll((long long)m) - 1) atomicAdd(cnt, (cells ? 1u : (uint32_t)PAIRS) * (uint32_t)__popcll(m));
       }
       continue;
+    }
+    if constexpr (D == 3) {
+      if (cells) {
+        // one record in the bin of corner 0 and, when the cell reaches into the next bin, one there
+        const uint32_t res = (uint32_t)g.res[l];
+        const Located3 q = locate(v, (float)g.res[l]);
+        const uint32_t b = q.c[0] + q.c[1] * res + q.c[2] * res * res;
+        const uint32_t k0 = b >> BIN_ROWS_LOG2, k1 = (b + res * res + res + 1u) >> BIN_ROWS_LOG2;
+        if (nb <= AGG_MAX_BINS) {
+          wave_rank(cnt, k0, valid, lane);
+          if (__any(valid && k1 != k0)) wave_rank(cnt, k1, valid && k1 != k0, lane);
+        } else if (valid) {
+          atomicAdd(cnt + k0, 1u);
+          if (k1 != k0) atomicAdd(cnt + k1, 1u);
+        }
+        continue;
+      }
     }
     uint32_t row[1 << D];
     cell_rows<D>(v, (float)g.res[l], l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi, primes, row, nullptr);
@@ -463,7 +496,33 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
       const uint32_t m = wave_max_u32((pk & 0xffffu) > (pk >> 16) ? (pk & 0xffffu) : (pk >> 16));
       if (lane == 63 && m) atomicMax(lmax + l, m);
     }
-    {
+    bool cells = false;
+    if constexpr (D == 3 && !G32) cells = bp.cell[l] != 0;
+    if (cells) {
+      const uint32_t res = (uint32_t)g.res[l];
+      const Located3 q = locate(v, (float)g.res[l]);
+      const uint32_t b = q.c[0] + q.c[1] * res + q.c[2] * res * res;
+      const uint32_t k0 = b >> BIN_ROWS_LOG2, k1 = (b + res * res + res + 1u) >> BIN_ROWS_LOG2;
+      const bool two = k1 != k0;
+      uint32_t pos0;
+      if (nb == 1) pos0 = (uint32_t)tid;  // the valid points are the first of the workgroup
+      else if (nb <= AGG_MAX_BINS) pos0 = wave_rank(lcur, k0, valid, lane);
+      else pos0 = valid ? atomicAdd(lcur + k0, 1u) : 0u;
+      if (valid) {
+        const uint3 rec = make_cell_record((int32_t)(b - (k0 << BIN_ROWS_LOG2)), q.fr, packed);
+        stage[pos0] = make_uint4(rec.x, rec.y, rec.z, pos0 + ldelta[k0]);
+      }
+      if (nb > 1 && __any(valid && two)) {
+        const bool on = valid && two;
+        uint32_t pos1;
+        if (nb <= AGG_MAX_BINS) pos1 = wave_rank(lcur, k1, on, lane);
+        else pos1 = on ? atomicAdd(lcur + k1, 1u) : 0u;
+        if (on) {
+          const uint3 rec = make_cell_record((int32_t)b - (int32_t)(k1 << BIN_ROWS_LOG2), q.fr, packed);
+          stage[pos1] = make_uint4(rec.x, rec.y, rec.z, pos1 + ldelta[k1]);
+        }
+      }
+    } else {
       uint32_t row[1 << D];
       float w[1 << D];
       cell_rows<D>(v, (float)g.res[l], l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi, primes, row, w);
@@ -644,7 +703,55 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const typena
           if (f[k][j]) atomicAdd(acc_tile + (uint32_t)(j & 1) * BIN_ROWS + slot[k][j >> 1], (unsigned long long)(long long)f[k][j]);
     }
   };
-  if (nonfinite) accumulate(std::true_type{});
+  // cell records (dense levels): the eight corners' rows and weights are rebuilt from the record; a corner outside this
+  // bin belongs to the copy of the record in the neighbouring bin
+  auto accumulate_cells = [&](auto nonfinite_c) {
+    constexpr bool NONFINITE = decltype(nonfinite_c)::value;
+    const uint32_t res = (uint32_t)g.res[l], r2 = res * res;
+    const float s_cell = ldexpf(1.0f, se - se / 2);
+    Rec q[ACC_INFLIGHT];
+#pragma unroll
+    for (int k = 0; k < ACC_INFLIGHT; ++k) q[k] = load_rec(k * ACC_THREADS + tid);
+    for (uint32_t i0 = 0; i0 < n_rec; i0 += ACC_THREADS * ACC_INFLIGHT) {
+      Rec cur[ACC_INFLIGHT];
+#pragma unroll
+      for (int k = 0; k < ACC_INFLIGHT; ++k) cur[k] = q[k];
+#pragma unroll
+      for (int k = 0; k < ACC_INFLIGHT; ++k) q[k] = load_rec(i0 + ACC_THREADS * ACC_INFLIGHT + k * ACC_THREADS + tid);
+#pragma unroll
+      for (int k = 0; k < ACC_INFLIGHT; ++k) {
+        const bool live = (cur[k].x & 0x3fffu) != 0u;  // reads past the task's end return zero words
+        const int32_t rel = (int32_t)(cur[k].x & 0x3fffu) - BIN_ROWS;
+        const float fx = (float)(cur[k].x >> 14) * (1.0f / CELL_QX), fy = (float)(cur[k].y & 0xffffu) * (1.0f / CELL_QYZ),
+                    fz = (float)(cur[k].y >> 16) * (1.0f / CELL_QYZ);
+        const float fr[3] = {fx, fy, fz};
+        float w[8];
+        weights_d3(fr, w);
+        const float g0 = BinRec<GT>::g0(cur[k]) * s_lo, g1 = BinRec<GT>::g1(cur[k]) * s_lo;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int32_t slot = rel + (j & 1) + ((j >> 1) & 1) * (int32_t)res + (j >> 2) * (int32_t)r2;
+          if (!live || slot < 0 || slot >= BIN_ROWS) continue;
+          int32_t f0v, f1v;
+          if constexpr (NONFINITE) {
+            f0v = w[j] != 0.0f;
+            f1v = has_pair && f0v;
+          } else {
+            f0v = __float2int_rn(w[j] * g0 * s_cell);
+            f1v = __float2int_rn(w[j] * g1 * s_cell);
+          }
+          if (f0v) atomicAdd(acc_tile + (uint32_t)slot, (unsigned long long)(long long)f0v);
+          if (f1v) atomicAdd(acc_tile + (uint32_t)BIN_ROWS + (uint32_t)slot, (unsigned long long)(long long)f1v);
+        }
+      }
+    }
+  };
+  bool cells = false;
+  if constexpr (sizeof(Rec) == 12) cells = bp.cell[l] != 0;
+  if (cells) {
+    if (nonfinite) accumulate_cells(std::true_type{});
+    else accumulate_cells(std::false_type{});
+  } else if (nonfinite) accumulate(std::true_type{});
   else accumulate(std::false_type{});
   lds_barrier();
   float* dst = dtable + (g.row_offset[l] + (int64_t)row0) * feat + f0;  // features f0, f0 + 1 of the bin's rows
@@ -678,7 +785,9 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const typena
 // Host side
 // ---------------------------------------------------------------------------------------
 // Plan for levels la .. lb-1 (the kernels see them as levels 0 .. lb-la-1 of a shifted geometry).
-static bool bin_plan(int64_t N, const nf_hash_geom* geom, int la, int lb, BinPlan* bp, int64_t* records, uint32_t* max_tasks) {
+// cells: dense 3-D levels whose eight corners span less than a bin take one record per point (16-bit gradients)
+static bool bin_plan(int64_t N, const nf_hash_geom* geom, int la, int lb, BinPlan* bp, int64_t* records, uint32_t* max_tasks,
+                     bool cells = false) {
   bp->n_levels = lb - la;
   int nb_total = 0;
   for (int l = la; l < lb; ++l) {
@@ -687,6 +796,8 @@ static bool bin_plan(int64_t N, const nf_hash_geom* geom, int la, int lb, BinPla
     if (nb > MAX_BINS_PER_LEVEL) return false;
     bp->nbins[l - la] = (int)nb;
     bp->binbase[l - la] = nb_total;
+    const int64_t res = geom->res[l];
+    bp->cell[l - la] = cells && geom->dims == 3 && l < geom->first_hash_level && res * res + res + 1 < BIN_ROWS;
     nb_total += (int)nb;
   }
   bp->binbase[lb - la] = nb_total;
@@ -806,7 +917,7 @@ static int launch_bwd_bin_piece(const void* coords, int cdt, int64_t csn, int64_
     BinPlan bp;
     int64_t R;
     uint32_t max_tasks;
-    bin_plan(N, geom, la, lb, &bp, &R, &max_tasks);
+    bin_plan(N, geom, la, lb, &bp, &R, &max_tasks, ddt != NF_F32);
     // the group's levels as levels 0 .. of a geometry of their own; their gradient columns start at la * feat
     DevGeom gg = g;
     gg.levels = lb - la;
