@@ -386,24 +386,49 @@ def test_backward_binned_clustered_points(do_dtype):
     torch.testing.assert_close(got, again, rtol=1e-5, atol=1e-6 * float(want.abs().max()))
 
 
+@pytest.mark.parametrize("do_dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_backward_binned_dense_levels_of_several_bins(do_dtype):
+    """Dense 3-D levels of 2 to 48 bins (resolutions 24 .. 72 in a table of 2^19 rows): with 16-bit gradients a point
+    leaves one record per level, and a second one where its cell reaches into the next bin.  Points on grid nodes
+    (weights exactly 0 and 1), on the upper edge and clustered in one cell are part of the input."""
+    hk = _hk()
+    torch.manual_seed(11)
+    N, T, L, lo, hi = 120000, 2**19, 6, 24, 72
+    x = torch.rand(N, 3)
+    x[:5000] = torch.randint(0, 73, (5000, 3)).float() / 72.0          # nodes of the finest level
+    x[5000:10000] = torch.randint(0, 25, (5000, 3)).float() / 24.0     # nodes of the coarsest level
+    x[10000:30000] = torch.tensor([0.71, 0.33, 0.52]) + 1e-3 * torch.rand(20000, 3)
+    x[30000:30100] = 1.0
+    offs = O.level_row_offsets(L, T, 3, lo, hi)
+    E = offs[-1]
+    assert all(offs[i + 1] - offs[i] < T for i in range(L)), "every level is dense"
+    do = torch.randn(N, L * 2).to(do_dtype)
+    want = O.encode_backward(x, do, E, 2, None, T, L, lo, hi)
+    got = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, 2, None, T, lo, hi, L)
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-3, atol=1e-4 * float(want.abs().max()))
+    # rows that no point's cell touches stay exactly zero
+    assert float(got.cpu()[want == 0].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("level", [1, 2])
 @pytest.mark.parametrize("do_dtype", [torch.float16, torch.float32])
-def test_backward_binned_nonfinite_gradient(do_dtype):
+def test_backward_binned_nonfinite_gradient(do_dtype, level):
     """An inf in one level's upstream gradient turns the rows that level touches into nan and leaves the other
-    levels exact."""
+    levels exact (level 1: dense, five bins; level 2: hashed)."""
     hk = _hk()
     torch.manual_seed(6)
-    N, T, L, lo, hi = 40000, 2**16, 4, 16, 256
+    N, T, L, lo, hi = 40000, 2**16, 4, 16, 128
     x = torch.rand(N, 3)
     E = O.level_row_offsets(L, T, 3, lo, hi)[-1]
     offs = O.level_row_offsets(L, T, 3, lo, hi)
     do = torch.randn(N, L * 2).to(do_dtype)
     clean = O.encode_backward(x, do, E, 2, None, T, L, lo, hi)
-    do[123, 2 * 2] = float("inf")  # level 2, feature 0
+    do[123, 2 * level] = float("inf")  # feature 0 of the level
     got = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, 2, None, T, lo, hi, L).cpu()
-    lvl2 = slice(offs[2], offs[3])
-    assert not torch.isfinite(got[lvl2]).all()
+    lvl = slice(offs[level], offs[level + 1])
+    assert not torch.isfinite(got[lvl]).all()
     keep = torch.ones(E, dtype=torch.bool)
-    keep[lvl2] = False
+    keep[lvl] = False
     torch.testing.assert_close(got[keep], clean[keep], rtol=1e-3, atol=1e-4)
 
 
