@@ -8,6 +8,13 @@ width ``2*H`` are split into halves ``x1, x2`` and pass through ``blocks`` coupl
 ``w1, w2 : (blocks*2*H, H)`` hold, per block, F's matrix then G's; ``b1, b2 : (blocks*2, H)``
 or ``None``.  The autograd Function saves only the OUTPUT: the backward kernel rebuilds each
 block's input from its output while it back-propagates, so no activation is stored.
+
+Choice of activation.  The rebuilt inputs come from 16-bit outputs, so a pre-activation that the forward saw within
+rounding of zero can land on the other side of zero in the backward.  Smooth activations (``"gelu"``, ``"silu"``) do not
+notice: at 65 536 rows, width 128, four couplings, no element of ``dx`` or of the weight gradients is outside rtol 2e-2 /
+atol 1e-2 of a float32 evaluation.  ``"relu"`` and ``"relu2"`` take their gates from the rebuilt inputs: a gate that flips
+moves a gradient by a whole weight, and 12 % of the elements of ``dx`` are outside that tolerance in the same measurement
+(largest error 7 % of the largest entry).  Use a smooth activation when the gradients matter to that level.
 """
 from __future__ import annotations
 
