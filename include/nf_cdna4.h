@@ -49,7 +49,7 @@ enum {
 };
 
 #define NF_MAX_LEVELS 32
-#define NF_MAX_DIMS 4
+#define NF_MAX_DIMS 6
 
 /* Level geometry of a hash encoding, computed on the host
  * (triton_helpers/layers/hash_encoding/helpers.py:26-115). */

@@ -129,7 +129,7 @@ def encode_forward(
     """
     n, dims = x.shape
     feat = table.shape[-1]
-    assert 1 <= dims <= 3
+    assert dims >= 1 and (dims <= 3 or primes is not None), "more than three dimensions need their own primes (kernel.py:537-540)"
     if primes is None:
         primes = PRIMES
     primes = torch.as_tensor(primes, dtype=torch.int64)

@@ -72,6 +72,41 @@ def test_corner_rows_bit_exact(N, D, F, T, L, lo, hi, scale):
         assert torch.equal(wf, w), "the fast kernels' weights are the generic kernels' weights, bit for bit"
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("D,T,L,lo,hi", [(4, 2**12, 4, 2, 16), (5, 2**12, 4, 2, 12), (6, 2**13, 4, 2, 8), (4, 3000, 2, 3, 9)])
+def test_four_to_six_dimensions(D, T, L, lo, hi, dtype):
+    """More than three dimensions (the reference takes any D once the caller brings the primes, kernel.py:537-545): the
+    per-(point, level) kernels with 16, 32 and 64 corners per cell, dense and hashed levels, one table size that is not a
+    power of two.  Corner rows bit for bit, forward and table gradient against the oracle."""
+    hk = _hk()
+    torch.manual_seed(D)
+    N, F = 500, 2
+    pi = torch.tensor([1, 2654435761, 805459861, 3674653429, 2097192037, 1434869437], dtype=torch.int64)
+    x = torch.rand(N, D)
+    x[0] = 0.0
+    x[1] = 1.0
+    offs = O.level_row_offsets(L, T, D, lo, hi)
+    E = offs[-1]
+    assert any(offs[i + 1] - offs[i] < T for i in range(L)) and any(offs[i + 1] - offs[i] == T for i in range(L)), "dense and hashed levels"
+    keep = torch.ones(N, dtype=torch.bool)
+    keep[1] = False  # x == 1 in every dimension: the reference's CPU path indexes one row past a dense level there
+    want_rows = O.encode_indices(x[keep], pi, T, L, lo, hi)
+    got_rows = hk.hash_encoding_indices(x.to(DEV), pi.to(DEV), T, lo, hi, L)
+    assert got_rows.shape == (N, L, 2**D)
+    assert torch.equal(got_rows.cpu()[keep], want_rows)
+    assert int(got_rows.max()) < T and int(got_rows.min()) >= 0
+    table = ((torch.rand(E, F) * 2 - 1)).to(dtype)
+    want = O.encode_forward(x[keep], table.float(), pi, T, L, lo, hi)
+    got = hk.hash_encoding(x.to(DEV), table.to(DEV), None, pi.to(DEV), T, lo, hi, L)
+    rtol, atol = (1e-5, 1e-6) if dtype == torch.float32 else (2.0**-10, 1e-4)
+    torch.testing.assert_close(got.cpu().float()[keep], want, rtol=rtol, atol=atol)
+    do = torch.randn(N, L * F).to(dtype)
+    do[1] = 0
+    want_g = O.encode_backward(x[keep], do[keep], E, F, pi, T, L, lo, hi)
+    got_g = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, F, pi.to(DEV), T, lo, hi, L)
+    torch.testing.assert_close(got_g.cpu(), want_g, rtol=1e-4, atol=1e-5 * max(1.0, float(want_g.abs().max())))
+
+
 def test_corner_rows_fast_path_upper_edge():
     """x == scale in every dimension: the fast kernels' index functions keep the zero-weight corner inside the level,
     like the 64-bit form."""

@@ -18,7 +18,7 @@ NF_ABI_VERSION = 8
 NF_F32, NF_F16, NF_BF16 = 0, 1, 2
 NF_ACT = {"none": 0, "relu": 1, "silu": 2, "relu2": 3, "gelu": 4}
 NF_MAX_LEVELS = 32
-NF_MAX_DIMS = 4
+NF_MAX_DIMS = 6
 NF_EINVAL, NF_EUNSUPPORTED, NF_EALIGN = -1, -2, -3
 NF_HASH_FORCE_GENERIC = 1
 NF_HASH_FORCE_ATOMIC = 2

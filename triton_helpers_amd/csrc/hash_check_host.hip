@@ -79,7 +79,9 @@ extern "C" int nf_hash_check_host(const float* coords, int64_t n_points, const n
     case 1: check_points<1>(coords, n_points, g, primes, scale, variant, rows_out, n_bad_rows); break;
     case 2: check_points<2>(coords, n_points, g, primes, scale, variant, rows_out, n_bad_rows); break;
     case 3: check_points<3>(coords, n_points, g, primes, scale, variant, rows_out, n_bad_rows); break;
-    default: check_points<4>(coords, n_points, g, primes, scale, variant, rows_out, n_bad_rows); break;
+    case 4: check_points<4>(coords, n_points, g, primes, scale, variant, rows_out, n_bad_rows); break;
+    case 5: check_points<5>(coords, n_points, g, primes, scale, variant, rows_out, n_bad_rows); break;
+    default: check_points<6>(coords, n_points, g, primes, scale, variant, rows_out, n_bad_rows); break;
   }
   return 0;
 }

@@ -680,7 +680,9 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
     case 1: return dispatch_fwd_generic<1>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
     case 2: return dispatch_fwd_generic<2>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
     case 3: return dispatch_fwd_generic<3>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
-    default: return dispatch_fwd_generic<4>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
+    case 4: return dispatch_fwd_generic<4>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
+    case 5: return dispatch_fwd_generic<5>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
+    default: return dispatch_fwd_generic<6>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
   }
 }
 
@@ -738,7 +740,9 @@ extern "C" int nf_hash_encode_bwd(const void* coords, int coords_dtype, int64_t 
     case 1: hipLaunchKernelGGL((hash_bwd_generic_k<1>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, g, primes, scale); break;
     case 2: hipLaunchKernelGGL((hash_bwd_generic_k<2>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, g, primes, scale); break;
     case 3: hipLaunchKernelGGL((hash_bwd_generic_k<3>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, g, primes, scale); break;
-    default: hipLaunchKernelGGL((hash_bwd_generic_k<4>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, g, primes, scale); break;
+    case 4: hipLaunchKernelGGL((hash_bwd_generic_k<4>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, g, primes, scale); break;
+    case 5: hipLaunchKernelGGL((hash_bwd_generic_k<5>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, g, primes, scale); break;
+    default: hipLaunchKernelGGL((hash_bwd_generic_k<6>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, g, primes, scale); break;
   }
   return check_launch("hash_bwd_generic");
 }
@@ -780,7 +784,9 @@ extern "C" int nf_hash_encode_indices(const void* coords, int coords_dtype, int6
     case 1: hipLaunchKernelGGL((hash_indices_k<1>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, out_rows, out_w, n_points, g, primes, scale); break;
     case 2: hipLaunchKernelGGL((hash_indices_k<2>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, out_rows, out_w, n_points, g, primes, scale); break;
     case 3: hipLaunchKernelGGL((hash_indices_k<3>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, out_rows, out_w, n_points, g, primes, scale); break;
-    default: hipLaunchKernelGGL((hash_indices_k<4>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, out_rows, out_w, n_points, g, primes, scale); break;
+    case 4: hipLaunchKernelGGL((hash_indices_k<4>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, out_rows, out_w, n_points, g, primes, scale); break;
+    case 5: hipLaunchKernelGGL((hash_indices_k<5>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, out_rows, out_w, n_points, g, primes, scale); break;
+    default: hipLaunchKernelGGL((hash_indices_k<6>), grid, dim3(256), 0, s, coords, coords_dtype, csn, csd, out_rows, out_w, n_points, g, primes, scale); break;
   }
   return check_launch("hash_indices");
 }

@@ -127,6 +127,7 @@ def hash_encoding_table_grad(
     """
     if pi is None:
         pi = _primes_for(coords.device)
+    assert pi.numel() >= coords.shape[-1], "Pi must have at least D_in elements"
     de = out if out is not None else torch.zeros(num_embeddings, d_embed, dtype=torch.float32, device=coords.device)
     assert de.dtype == torch.float32 and de.is_contiguous() and de.shape == (num_embeddings, d_embed)
     coords2d = _flat_coords(coords)
@@ -289,6 +290,7 @@ def hash_encoding_indices(
     N, D = coords2d.shape
     if pi is None:
         pi = _primes_for(coord.device)
+    assert pi.numel() >= D, "Pi must have at least D_in elements"
     geom = level_geometry(max_entries_per_level, levels, D, 1, min_res, max_res)
     rows = torch.empty(N, levels, 2**D, dtype=torch.int64, device=coord.device)
     w = torch.empty(N, levels, 2**D, dtype=torch.float32, device=coord.device) if return_weights else None
