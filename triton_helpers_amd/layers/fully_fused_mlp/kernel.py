@@ -156,7 +156,6 @@ def _workspace(lib, rows2d: Tensor, d_hidden: int, depth: int, activation: str, 
 class _fully_fused_mlp(Function):
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.float16)
-    @torch.no_grad()
     def forward(
         ctx,
         x: Tensor,
@@ -217,7 +216,6 @@ class _fully_fused_mlp(Function):
 
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
-    @torch.no_grad()
     def backward(ctx, do: Tensor):
         x, w_in, b_in, w_out, b_out, w_hid, b_hid = ctx.saved_tensors
         B, L, D_in = x.shape
@@ -266,21 +264,37 @@ class _fully_fused_mlp(Function):
         return dx, dw_in, db_in, dw_out, db_out, dw_hid, db_hid, None, None
 
 
+_rounded_plans: dict = {}
+
+
+def _rounded_plan(lib, like, D_in, D_hidden, D_out):
+    """Where each gradient sits in the flat buffer (16-byte aligned pieces), its length and the scratch size, per
+    combination of parameter shapes (a handful per process)."""
+    key = tuple(None if t is None else (tuple(t.shape), t.stride(), t.dtype) for t in like)
+    plan = _rounded_plans.get(key)
+    if plan is None:
+        offsets, off = [], 0
+        for t in like:
+            offsets.append(off)
+            if t is not None:
+                off += (t.numel() + 7) // 8 * 8
+        plan = (tuple(offsets), off, lib.nf_mlp_bwd_rounded_workspace_bytes(D_in, D_hidden, D_out))
+        if len(_rounded_plans) < 4096:
+            _rounded_plans[key] = plan
+    return plan
+
+
 def _backward_rounded(x, do2, w_in, b_in, w_out, b_out, w_hid, b_hid, need_dx, D_in, D_hidden, D_out):
-    """Backward of the decoder shape through ``nf_mlp_bwd_rounded``: the weight gradients come back summed in a fixed
-    order and rounded to the parameters' dtype, into one uninitialised buffer (no clearing, no cast kernel).  ``None`` when
-    the library declines (rows not 8-byte aligned): the caller takes the general path."""
+    """Backward of the one-hidden-layer ReLU shapes through ``nf_mlp_bwd_rounded``: the weight gradients come back summed
+    in a fixed order and rounded to the parameters' dtype, into one uninitialised buffer (no clearing, no cast kernel).
+    ``None`` when the library declines (rows not 8-byte aligned): the caller takes the general path.  The buffer is
+    allocated per call: its pieces become the ``.grad`` tensors, which a later backward must not overwrite."""
     lib = _lib.load()
     like = (w_in, b_in, w_out, b_out, w_hid, b_hid)
-    offsets, off = [], 0
-    for t in like:
-        offsets.append(off)
-        if t is not None:
-            off += (t.numel() + 7) // 8 * 8  # 16-byte aligned pieces
-    flat = torch.empty(off, dtype=w_in.dtype, device=w_in.device)
+    offsets, total, ws_bytes = _rounded_plan(lib, like, D_in, D_hidden, D_out)
+    flat = torch.empty(total, dtype=w_in.dtype, device=w_in.device)
     base, es = flat.data_ptr(), flat.element_size()
     p = [None if t is None else base + es * o for t, o in zip(like, offsets)]
-    ws_bytes = lib.nf_mlp_bwd_rounded_workspace_bytes(D_in, D_hidden, D_out)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w_in.device)
     x2 = _rows2d(x, D_in)
     dx = x.new_empty(x.shape) if need_dx else None
