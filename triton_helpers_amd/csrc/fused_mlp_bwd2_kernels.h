@@ -126,10 +126,10 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t rows_rsrc(const void* base, in
 }
 // What a launch needs of a tensor's extent for these 32-bit offsets to be safe: the tensor itself below 2^31 bytes
 // (the descriptor's range check then catches every row past the end), and the furthest row any lane ever addresses
-// -- the rows a partly filled last chunk pads to, and the chunk the prefetch asks for one grid-stride ahead (at most
-// 256 workgroups x 12 waves x 32 rows) -- still below 2^32 bytes, so that no offset wraps back into range.
+// -- the rows a partly filled last chunk pads to, and the chunks the prefetch asks for up to two grid-strides ahead (a
+// stride is at most 256 workgroups x 12 waves x 32 rows) -- still below 2^32 bytes, so that no offset wraps back into range.
 inline bool rows_in_reach(int64_t rows, int64_t stride) {
-  const int64_t ahead = (int64_t)256 * 12 * 32 + 64;
+  const int64_t ahead = (int64_t)2 * 256 * 12 * 32 + 64;
   return rows * stride * 2 <= (((int64_t)1 << 31) - 1) && (rows + ahead) * stride * 2 + 128 < ((int64_t)1 << 32);
 }
 // byte offset of the piece (columns col .. col + 3) of row `row` of the first chunk
