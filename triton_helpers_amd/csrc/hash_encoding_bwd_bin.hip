@@ -790,6 +790,7 @@ static bool bin_plan(int64_t N, const nf_hash_geom* geom, int la, int lb, BinPla
                      bool cells = false) {
   bp->n_levels = lb - la;
   int nb_total = 0;
+  int64_t R = 0;
   for (int l = la; l < lb; ++l) {
     const int64_t r = geom->rows[l];
     const int64_t nb = (r + BIN_ROWS - 1) / BIN_ROWS;
@@ -798,12 +799,13 @@ static bool bin_plan(int64_t N, const nf_hash_geom* geom, int la, int lb, BinPla
     bp->binbase[l - la] = nb_total;
     const int64_t res = geom->res[l];
     bp->cell[l - la] = cells && geom->dims == 3 && l < geom->first_hash_level && res * res + res + 1 < BIN_ROWS;
+    // a cell level leaves at most two records per point; an x-pair level has room for every pair to be split in two
+    // (normally half of it is used)
+    R += N * (bp->cell[l - la] ? 2 : geom->dims == 3 ? 8 : 4);
     nb_total += (int)nb;
   }
   bp->binbase[lb - la] = nb_total;
   if (nb_total > MAX_BINS_TOTAL) return false;
-  // room for every pair to be split in two; normally half of it is used
-  const int64_t R = N * (lb - la) * (geom->dims == 3 ? 8 : 4);
   if (R >= ((int64_t)1 << 32) - 4 * ACC_THREADS * ACC_INFLIGHT) return false;  // 32-bit record positions
   *records = R;
   *max_tasks = (uint32_t)(nb_total + R / SPLIT_RECORDS + 1);
@@ -878,7 +880,7 @@ int64_t bwd_bin_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int 
     BinPlan bp;
     int64_t R;
     uint32_t max_tasks;
-    bin_plan(n_points, geom, first[k], first[k + 1], &bp, &R, &max_tasks);
+    bin_plan(n_points, geom, first[k], first[k + 1], &bp, &R, &max_tasks, dout_dtype != NF_F32);
     BinWs ws;
     const int64_t b = bin_ws(nullptr, bp, n_points, R, dout_dtype == NF_F32 ? 4 : 3, max_tasks, &ws);
     if (b > bytes) bytes = b;
