@@ -1,19 +1,24 @@
 // One-hidden-layer ReLU backward (d_in <= 64, d_hidden = 64, d_out <= 64) with the work of a workgroup split by ROLE:
-// twelve waves, one "chain" wave and two "gradient" waves per SIMD.
+// sixteen waves, two "chain" waves and two "gradient" waves per SIMD.
 //
 // What the split is for.  A wave issues in order and its vector instructions do not start while one of its own matrix
 // products is in flight (measured: a product followed by eight independent vector instructions takes 16 + 8 x 4
 // clocks), so a SIMD's matrix core and vector ALU only overlap across waves; and the weight gradients of a 64-wide
 // network (up to 48 tiles = 192 accumulator registers) leave no room for the rest of the backward in the same wave.
 //
-//   * a chain wave owns a 32-row chunk per round: it recomputes the forward, carries the gradient back through the
-//     three layers (all the packing / gating vector work) and writes dx.  It holds no weight-gradient accumulator.
-//   * the two gradient waves of a chain wave hold its weight-gradient accumulators for the whole launch, half of the
-//     output features each (at most 24 tiles = 96 registers, so three waves fit a SIMD).  The chain wave parks the
-//     operands of dW = dz^T h (row-major, 16 bit) in LDS panels; the gradient waves read them back transposed
-//     (ds_read_b64_tr_b16) and run the products of the chunk while the chain wave is busy with vector work.
+//   * a round covers four 32-row panels.  A chain wave owns 16 rows of a panel per round (two chain waves per panel, so
+//     that a SIMD has a second chain to run while the first waits for weight fragments or a barrier): it recomputes the
+//     forward, carries the gradient back through the three layers (all the packing / gating vector work) and writes dx.
+//     It holds no weight-gradient accumulator.
+//   * the two gradient waves of a panel hold its weight-gradient accumulators for the whole launch, half of the
+//     output features each (at most 24 tiles = 96 of the 128 registers a wave has at four waves per SIMD; the B operands
+//     of a section's products are therefore taken two at a time).  The chain waves park the operands of dW = dz^T h
+//     (row-major, 16 bit) in the panel; the gradient waves read them back transposed (ds_read_b64_tr_b16) and run the
+//     products of the panel while the chain waves are busy with vector work.
+//   (With four chain waves of 32 rows each -- twelve waves, 168 registers -- the same kernel takes 12 - 15 % longer:
+//   64 -> 64 -> 64 -> 64 with biases 160 against 139 us per 2^20 rows.  The template keeps both.)
 //
-// The roles meet at three workgroup barriers per round.  A chain wave has one panel area per section ({h2, dy},
+// The roles meet at three workgroup barriers per round.  A panel has one area per section ({h2, dy},
 // {h1, dz2}, {dz1, x}); a section is announced by the barrier in front of the NEXT section's stores, by which time its
 // own stores have long landed, and it is overwritten a full round later, after the gradient wave has passed three more
 // barriers.  Rows past the end of the batch read as zero through the buffer descriptors (a zero dy row contributes
@@ -24,7 +29,8 @@
 
 namespace nf {
 
-constexpr int WS_CHAIN = 4, WS_GRAD = 8, WS_WAVES = WS_CHAIN + WS_GRAD;
+// panels per round, gradient waves, chain waves (one or two per panel)
+constexpr int WS_CHAIN = 4, WS_GRAD = 8, WS_CHAIN_WAVES = 8, WS_WAVES = WS_CHAIN_WAVES + WS_GRAD;
 // dwords per panel row for 64 / 32 / 16 features: the features plus padding that spreads the rows over the banks
 constexpr int ws_stride(int features) { return features == 64 ? 34 : features == 32 ? 20 : 12; }
 constexpr int ws_panel(int features) { return 32 * ws_stride(features); }  // dwords per 32-row panel
@@ -80,17 +86,24 @@ struct WsShape {
 
 // XC: how x / dx are stored (MlpArgs::x_conv, 0 or the other 16-bit type); B: the network has biases or bias
 // gradients are wanted (false: accumulators start at zero and no row sums are kept).
-template <typename T, int KIN, int OUTP, int XC, bool B>
-__global__ __launch_bounds__(64 * WS_WAVES, 1) void mlp_bwd2_ws_k(MlpArgs a) {
+template <typename T, int KIN, int OUTP, int XC, bool B, int CH = WS_CHAIN_WAVES>
+__global__ __launch_bounds__(64 * (CH + WS_GRAD), 1) void mlp_bwd2_ws_k(MlpArgs a) {
   using SH = WsShape<KIN, OUTP>;
-  constexpr int KC_IN = SH::KC_IN, KC_O = SH::KC_O, MT_H = SH::MT_H, MT_I = SH::MT_I, MT_O = SH::MT_O, NT = 2;
+  // CH chain waves share the WS_CHAIN panels of a round: four own a 32-row panel each, eight a 16-row half each
+  static_assert(CH == WS_CHAIN || CH == 2 * WS_CHAIN, "four or eight chain waves");
+  constexpr int NT = CH == WS_CHAIN ? 2 : 1, WAVES = CH + WS_GRAD;
+  // B operands of a section's products held at a time: all four with 168 registers per wave, two with 128
+  constexpr int JB = CH == WS_CHAIN ? 4 : 2;
+  constexpr int KC_IN = SH::KC_IN, KC_O = SH::KC_O, MT_H = SH::MT_H, MT_I = SH::MT_I, MT_O = SH::MT_O;
   constexpr int TILES = SH::TILES, NBIAS = SH::NBIAS;
   constexpr int S_H = ws_stride(64), S_X = ws_stride(KIN), S_Y = ws_stride(OUTP), P_H = ws_panel(64);
   constexpr int DY_HALVES = OUTP > 16 ? 2 : 1;
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x;
-  constexpr int nthreads = 64 * WS_WAVES;
+  constexpr int nthreads = 64 * WAVES;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // a chain wave's panel and the first 16-row tile it owns there
+  const int pd = CH == WS_CHAIN ? wave : wave >> 1, pt0 = CH == WS_CHAIN ? 0 : wave & 1;
 
   uint16_t* f_in = reinterpret_cast<uint16_t*>(smem);       // W_in    [MT_H][KC_IN]
   uint16_t* f_hid = f_in + MT_H * KC_IN * FRAG_ELEMS;       // W_hid   [MT_H][2]
@@ -104,7 +117,7 @@ __global__ __launch_bounds__(64 * WS_WAVES, 1) void mlp_bwd2_ws_k(MlpArgs a) {
   const int64_t n_chunks = (a.rows + 31) / 32;
   const int64_t per_round = (int64_t)gridDim.x * WS_CHAIN;
   const int rounds = (int)((n_chunks + per_round - 1) / per_round);
-  const bool chain = wave < WS_CHAIN;
+  const bool chain = wave < CH;
 
   // the chain waves ask for their first rows before the weights are staged
   const __amdgpu_buffer_rsrc_t rs_x = rows_rsrc(a.x, a.rows, a.x_stride), rs_dy = rows_rsrc(a.dy, a.rows, a.dy_stride),
@@ -141,15 +154,15 @@ __global__ __launch_bounds__(64 * WS_WAVES, 1) void mlp_bwd2_ws_k(MlpArgs a) {
     }
     return f;
   };
-  const int64_t first_chunk = (int64_t)blockIdx.x * WS_CHAIN + wave;
+  const int64_t first_chunk = (int64_t)blockIdx.x * WS_CHAIN + pd;
   Frag nx[NT][KC_IN], ndy[NT][KC_O];
   if (chain) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
-      for (int kc = 0; kc < KC_IN; ++kc) nx[nt][kc] = load_x(first_chunk, nt, kc);
+      for (int kc = 0; kc < KC_IN; ++kc) nx[nt][kc] = load_x(first_chunk, pt0 + nt, kc);
 #pragma unroll
-      for (int kc = 0; kc < KC_O; ++kc) ndy[nt][kc] = load_dy(first_chunk, nt, kc);
+      for (int kc = 0; kc < KC_O; ++kc) ndy[nt][kc] = load_dy(first_chunk, pt0 + nt, kc);
     }
   }
 
@@ -169,7 +182,7 @@ __global__ __launch_bounds__(64 * WS_WAVES, 1) void mlp_bwd2_ws_k(MlpArgs a) {
 
   if (chain) {
     // ------------------------------------------------------------------ chain waves
-    uint32_t* area_a = panels + (size_t)wave * SH::WAVE_DWORDS;
+    uint32_t* area_a = panels + (size_t)pd * SH::WAVE_DWORDS;
     uint32_t* area_b = area_a + SH::AREA_A;
     uint32_t* area_c = area_b + SH::AREA_B;
     for (int round = 0; round < rounds; ++round) {
@@ -181,12 +194,12 @@ __global__ __launch_bounds__(64 * WS_WAVES, 1) void mlp_bwd2_ws_k(MlpArgs a) {
 #pragma unroll
         for (int kc = 0; kc < KC_IN; ++kc) {
           in[nt][kc] = XC == 0 ? nx[nt][kc] : convert_frag(nx[nt][kc], XC);
-          nx[nt][kc] = load_x(chunk + per_round, nt, kc);
+          nx[nt][kc] = load_x(chunk + per_round, pt0 + nt, kc);
         }
 #pragma unroll
         for (int kc = 0; kc < KC_O; ++kc) {
           dz[nt][kc] = ndy[nt][kc];
-          ndy[nt][kc] = load_dy(chunk + per_round, nt, kc);
+          ndy[nt][kc] = load_dy(chunk + per_round, pt0 + nt, kc);
         }
       }
       // ---- forward recompute ----
@@ -220,9 +233,9 @@ __global__ __launch_bounds__(64 * WS_WAVES, 1) void mlp_bwd2_ws_k(MlpArgs a) {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
-        for (int kc = 0; kc < 2; ++kc) ws_park<S_H, true>(area_a, h2[nt][kc], nt, kc, lane);
+        for (int kc = 0; kc < 2; ++kc) ws_park<S_H, true>(area_a, h2[nt][kc], pt0 + nt, kc, lane);
 #pragma unroll
-        for (int kc = 0; kc < KC_O; ++kc) ws_park<S_Y, (OUTP > 16)>(area_a + P_H, dz[nt][kc], nt, kc, lane);
+        for (int kc = 0; kc < KC_O; ++kc) ws_park<S_Y, (OUTP > 16)>(area_a + P_H, dz[nt][kc], pt0 + nt, kc, lane);
       }
       layer_nt<T, NT, MT_H, KC_O, 0>(acc, dz, t_out, nullptr, lane);  // dh2 = W_out^T dy
       gates(h2);                                                      // dz2
@@ -232,8 +245,8 @@ __global__ __launch_bounds__(64 * WS_WAVES, 1) void mlp_bwd2_ws_k(MlpArgs a) {
       for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int kc = 0; kc < 2; ++kc) {
-          ws_park<S_H, true>(area_b, h1[nt][kc], nt, kc, lane);
-          ws_park<S_H, true>(area_b + P_H, dz[nt][kc], nt, kc, lane);
+          ws_park<S_H, true>(area_b, h1[nt][kc], pt0 + nt, kc, lane);
+          ws_park<S_H, true>(area_b + P_H, dz[nt][kc], pt0 + nt, kc, lane);
         }
       layer_nt<T, NT, MT_H, 2, 0>(acc, dz, t_hid, nullptr, lane);  // dh1 = W_hid^T dz2
       gates(h1);                                                   // dz1
@@ -242,9 +255,9 @@ __global__ __launch_bounds__(64 * WS_WAVES, 1) void mlp_bwd2_ws_k(MlpArgs a) {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
-        for (int kc = 0; kc < 2; ++kc) ws_park<S_H, true>(area_c, dz[nt][kc], nt, kc, lane);
+        for (int kc = 0; kc < 2; ++kc) ws_park<S_H, true>(area_c, dz[nt][kc], pt0 + nt, kc, lane);
 #pragma unroll
-        for (int kc = 0; kc < KC_IN; ++kc) ws_park<S_X, true>(area_c + P_H, in[nt][kc], nt, kc, lane);
+        for (int kc = 0; kc < KC_IN; ++kc) ws_park<S_X, true>(area_c + P_H, in[nt][kc], pt0 + nt, kc, lane);
       }
       if (a.dx != nullptr) {
         layer_nt<T, NT, MT_I, 2, 0>(acc, dz, t_in, nullptr, lane);  // dx = W_in^T dz1
@@ -256,14 +269,14 @@ __global__ __launch_bounds__(64 * WS_WAVES, 1) void mlp_bwd2_ws_k(MlpArgs a) {
             if (XC == 1) { o[0] = pack2<F16>(acc[nt][mt][0], acc[nt][mt][1]); o[1] = pack2<F16>(acc[nt][mt][2], acc[nt][mt][3]); }
             else if (XC == 2) { o[0] = pack2<BF16>(acc[nt][mt][0], acc[nt][mt][1]); o[1] = pack2<BF16>(acc[nt][mt][2], acc[nt][mt][3]); }
             else { o[0] = pack2<T>(acc[nt][mt][0], acc[nt][mt][1]); o[1] = pack2<T>(acc[nt][mt][2], acc[nt][mt][3]); }
-            __builtin_amdgcn_raw_buffer_store_b64(o, rs_dx, at(chunk, nt, a.dx_stride, off_dx[mt]), 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b64(o, rs_dx, at(chunk, pt0 + nt, a.dx_stride, off_dx[mt]), 0, 0);
           }
       }
     }
     ws_barrier();  // announces {dz1, x} of the last round
   } else {
     // ------------------------------------------------------------------ gradient waves
-    const int d = (wave - WS_CHAIN) & (WS_CHAIN - 1), half = (wave - WS_CHAIN) / WS_CHAIN;
+    const int d = (wave - CH) & (WS_CHAIN - 1), half = (wave - CH) / WS_CHAIN;
     const bool has_out = MT_O == 4 || half == 0;
     const f32x4_t zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -274,17 +287,23 @@ __global__ __launch_bounds__(64 * WS_WAVES, 1) void mlp_bwd2_ws_k(MlpArgs a) {
     const uint32_t* area_b = area_a + SH::AREA_A;
     const uint32_t* area_c = area_b + SH::AREA_B;
     auto section_c = [&]() {  // dW_in += dz1^T x, rows 32 half ..
-      Frag xb[MT_I];
+      constexpr int JC = JB < MT_I ? JB : MT_I;
 #pragma unroll
-      for (int j = 0; j < MT_I; ++j) xb[j] = ws_operand<S_X>(area_c + P_H, j, lane);
+      for (int j0 = 0; j0 < MT_I; j0 += JC) {
+        Frag xb[JC];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const Frag da = ws_operand<S_H>(area_c, 2 * half + i, lane);
+        for (int j = 0; j < JC; ++j) xb[j] = ws_operand<S_X>(area_c + P_H, j0 + j, lane);
 #pragma unroll
-        for (int j = 0; j < MT_I; ++j) acc_dw[SH::T_IN + i * MT_I + j] = mfma16<T>(da, xb[j], acc_dw[SH::T_IN + i * MT_I + j]);
-        if constexpr (B) {
+        for (int i = 0; i < 2; ++i) {
+          const Frag da = ws_operand<S_H>(area_c, 2 * half + i, lane);
 #pragma unroll
-          for (int q = 0; q < 4; ++q) acc_db[i] = dot2_ones<T>(da.w[q], acc_db[i]);
+          for (int j = 0; j < JC; ++j) acc_dw[SH::T_IN + i * MT_I + j0 + j] = mfma16<T>(da, xb[j], acc_dw[SH::T_IN + i * MT_I + j0 + j]);
+          if constexpr (B) {
+            if (j0 == 0) {
+#pragma unroll
+              for (int q = 0; q < 4; ++q) acc_db[i] = dot2_ones<T>(da.w[q], acc_db[i]);
+            }
+          }
         }
       }
     };
@@ -293,33 +312,43 @@ __global__ __launch_bounds__(64 * WS_WAVES, 1) void mlp_bwd2_ws_k(MlpArgs a) {
       if (round > 0) section_c();
       ws_barrier();
       if (has_out) {  // dW_out += dy^T h2
-        Frag hb[MT_H];
 #pragma unroll
-        for (int j = 0; j < MT_H; ++j) hb[j] = ws_operand<S_H>(area_a, j, lane);
+        for (int j0 = 0; j0 < MT_H; j0 += JB) {
+          Frag hb[JB];
 #pragma unroll
-        for (int i = 0; i < SH::RO; ++i) {
-          const Frag da = ws_operand<S_Y>(area_a + P_H, MT_O == 4 ? 2 * half + i : 0, lane);
+          for (int j = 0; j < JB; ++j) hb[j] = ws_operand<S_H>(area_a, j0 + j, lane);
 #pragma unroll
-          for (int j = 0; j < MT_H; ++j) acc_dw[SH::T_OUT + i * MT_H + j] = mfma16<T>(da, hb[j], acc_dw[SH::T_OUT + i * MT_H + j]);
-          if constexpr (B) {
+          for (int i = 0; i < SH::RO; ++i) {
+            const Frag da = ws_operand<S_Y>(area_a + P_H, MT_O == 4 ? 2 * half + i : 0, lane);
 #pragma unroll
-            for (int q = 0; q < 4; ++q) acc_db[4 + i] = dot2_ones<T>(da.w[q], acc_db[4 + i]);
+            for (int j = 0; j < JB; ++j) acc_dw[SH::T_OUT + i * MT_H + j0 + j] = mfma16<T>(da, hb[j], acc_dw[SH::T_OUT + i * MT_H + j0 + j]);
+            if constexpr (B) {
+              if (j0 == 0) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) acc_db[4 + i] = dot2_ones<T>(da.w[q], acc_db[4 + i]);
+              }
+            }
           }
         }
       }
       ws_barrier();
       {  // dW_hid += dz2^T h1
-        Frag hb[MT_H];
 #pragma unroll
-        for (int j = 0; j < MT_H; ++j) hb[j] = ws_operand<S_H>(area_b, j, lane);
+        for (int j0 = 0; j0 < MT_H; j0 += JB) {
+          Frag hb[JB];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          const Frag da = ws_operand<S_H>(area_b + P_H, 2 * half + i, lane);
+          for (int j = 0; j < JB; ++j) hb[j] = ws_operand<S_H>(area_b, j0 + j, lane);
 #pragma unroll
-          for (int j = 0; j < MT_H; ++j) acc_dw[SH::T_HID + i * MT_H + j] = mfma16<T>(da, hb[j], acc_dw[SH::T_HID + i * MT_H + j]);
-          if constexpr (B) {
+          for (int i = 0; i < 2; ++i) {
+            const Frag da = ws_operand<S_H>(area_b + P_H, 2 * half + i, lane);
 #pragma unroll
-            for (int q = 0; q < 4; ++q) acc_db[2 + i] = dot2_ones<T>(da.w[q], acc_db[2 + i]);
+            for (int j = 0; j < JB; ++j) acc_dw[SH::T_HID + i * MT_H + j0 + j] = mfma16<T>(da, hb[j], acc_dw[SH::T_HID + i * MT_H + j0 + j]);
+            if constexpr (B) {
+              if (j0 == 0) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) acc_db[2 + i] = dot2_ones<T>(da.w[q], acc_db[2 + i]);
+              }
+            }
           }
         }
       }
@@ -344,8 +373,8 @@ __global__ __launch_bounds__(64 * WS_WAVES, 1) void mlp_bwd2_ws_k(MlpArgs a) {
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     __syncthreads();
-    if (!chain && (wave - WS_CHAIN) / WS_CHAIN == h) {
-      const int d = (wave - WS_CHAIN) & (WS_CHAIN - 1);
+    if (!chain && (wave - CH) / WS_CHAIN == h) {
+      const int d = (wave - CH) & (WS_CHAIN - 1);
 #pragma unroll
       for (int t = 0; t < TILES; ++t) red[((size_t)d * TILES + t) * 64 + lane] = acc_dw[t];
 #pragma unroll
@@ -355,7 +384,7 @@ __global__ __launch_bounds__(64 * WS_WAVES, 1) void mlp_bwd2_ws_k(MlpArgs a) {
     constexpr int T_LAST = TILES;
 #pragma unroll
     for (int t = 0; t < T_LAST; ++t) {
-      if (t % WS_WAVES != wave) continue;
+      if (t % WAVES != wave) continue;
       if (t >= SH::T_OUT && MT_O != 4 && h != 0) continue;  // a 16-row dW_out was summed with half 0
       const f32x4_t* p = red + (size_t)t * 64 + lane;
       const f32x4_t v = (p[0] + p[(size_t)TILES * 64]) + (p[(size_t)2 * TILES * 64] + p[(size_t)3 * TILES * 64]);
@@ -366,7 +395,7 @@ __global__ __launch_bounds__(64 * WS_WAVES, 1) void mlp_bwd2_ws_k(MlpArgs a) {
     if constexpr (B) {
 #pragma unroll
       for (int u = 0; u < NBIAS; ++u) {
-        if (u % WS_WAVES != wave) continue;
+        if (u % WAVES != wave) continue;
         if (u >= 4 && MT_O != 4 && h != 0) continue;
         const float* p = redb + (size_t)u * 64 + lane;
         const float v = (p[0] + p[(size_t)NBIAS * 64]) + (p[(size_t)2 * NBIAS * 64] + p[(size_t)3 * NBIAS * 64]);

@@ -4,11 +4,12 @@
 
 namespace nf {
 
-template <typename T, int KIN, int OUTP>
+template <typename T, int KIN, int OUTP, int CH = WS_CHAIN_WAVES>
 static int launch_ws(const MlpArgs& a0, hipStream_t s, int* blocks_out) {
   MlpArgs a = a0;
   constexpr size_t LDS = WsShape<KIN, OUTP>::LDS;
-  a.waves = WS_WAVES;
+  constexpr int WAVES = CH + WS_GRAD;
+  a.waves = WAVES;
   a.x_vec = a.dy_vec = a.dx_vec = 1;
   const int64_t chunks = (a.rows + 31) / 32;
   int64_t blocks = (chunks + WS_CHAIN - 1) / WS_CHAIN;
@@ -16,11 +17,11 @@ static int launch_ws(const MlpArgs& a0, hipStream_t s, int* blocks_out) {
   if (blocks > cap) blocks = cap;
   if (blocks_out != nullptr) *blocks_out = (int)blocks;
   const bool b = a.db_in != nullptr || a.db_hid != nullptr || a.db_out != nullptr || a.b_in != nullptr || a.b_hid != nullptr;
-  const void* kern = b ? (const void*)mlp_bwd2_ws_k<T, KIN, OUTP, 0, true> : (const void*)mlp_bwd2_ws_k<T, KIN, OUTP, 0, false>;
+  const void* kern = b ? (const void*)mlp_bwd2_ws_k<T, KIN, OUTP, 0, true, CH> : (const void*)mlp_bwd2_ws_k<T, KIN, OUTP, 0, false, CH>;
   const hipError_t ea = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
   if (ea != hipSuccess) return fail((int)ea, "hipFuncSetAttribute: %s", hipGetErrorString(ea));
   void* args[] = {(void*)&a};
-  const hipError_t e = hipLaunchKernel(kern, dim3((unsigned)blocks), dim3(64 * WS_WAVES), args, LDS, s);
+  const hipError_t e = hipLaunchKernel(kern, dim3((unsigned)blocks), dim3(64 * WAVES), args, LDS, s);
   if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(mlp_bwd2, role split): %s", hipGetErrorString(e));
   return check_launch("mlp_bwd2 (role split)");
 }
