@@ -48,6 +48,9 @@ __device__ __forceinline__ f32x4_t mfma16<F16>(const Frag& a, const Frag& b, f32
 // K-slot -> feature maps (kc = 32-wide chunk, g = lane group, j = element 0..7)
 __host__ __device__ __forceinline__ int k_nat(int kc, int g, int j) { return 32 * kc + 8 * g + j; }
 __host__ __device__ __forceinline__ int k_chain(int kc, int g, int j) { return 32 * kc + 16 * (j >> 2) + 4 * g + (j & 3); }
+// "Wide order" of the 16 outputs of accumulator tile mt: lane group g's four outputs of tiles 2p and 2p + 1 are the eight
+// consecutive features 32p + 8g .. + 7 (one 16-byte access per lane and tile pair instead of two 8-byte ones); m = 4g + r.
+__host__ __device__ __forceinline__ int wide_feature(int mt, int m) { return 32 * (mt >> 1) + 8 * (m >> 2) + 4 * (mt & 1) + (m & 3); }
 
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
@@ -209,11 +212,12 @@ __device__ __forceinline__ void gate_apply(const f32x4_t dh, uint32_t g01, uint3
 
 // ---- staging weights into LDS as A fragments ------------------------------------------
 // dst: fragment array [MT][KC][64 lanes][8 elements]; element (mt, kc, lane(m,g), j) =
-//   transposed ? W[kmap(kc,g,j)][16*mt+m] : W[16*mt+m][kmap(kc,g,j)]
-// where W is [w_rows][w_cols] row-major; out-of-range entries are zero.
+//   transposed ? W[kmap(kc,g,j)][mmap(mt,m)] : W[mmap(mt,m)][kmap(kc,g,j)]
+// where W is [w_rows][w_cols] row-major, mmap(mt, m) = 16*mt + m, or wide_feature(mt, m) with WIDE_M; out-of-range
+// entries are zero.
 // NTHREADS > 0: the workgroup size is that compile-time constant, the loop is unrolled and all loads of a matrix
 // are in flight together.
-template <bool CHAIN, bool TRANSPOSED, int NTHREADS = 0>
+template <bool CHAIN, bool TRANSPOSED, int NTHREADS = 0, bool WIDE_M = false>
 __device__ __forceinline__ void stage_weight_frags(uint16_t* dst, const uint16_t* w, int w_rows, int w_cols, int MT,
                                                    int KC, int tid, int nthreads) {
   // one unit = the 8 elements of one lane of one fragment; the 8 loads of a unit are independent
@@ -223,7 +227,7 @@ __device__ __forceinline__ void stage_weight_frags(uint16_t* dst, const uint16_t
     const int lane = u & 63;
     const int frag = u >> 6;
     const int kc = frag % KC, mt = frag / KC;
-    const int m = 16 * mt + (lane & 15);
+    const int m = WIDE_M ? wide_feature(mt, lane & 15) : 16 * mt + (lane & 15);
     const int g = lane >> 4;
     uint16_t v[8];
     if (vec_ok && m < w_rows) {

@@ -35,14 +35,17 @@ struct RevArgs {
   int64_t rows;
   int half, nblocks, act;
   int vec_in, vec_out, vec_dy, vec_dx;
+  int wide_ok;  // backward: every tensor allows 16-byte accesses to its rows
 };
 
 // accumulator-layout load: lane (n,g) gets features 16*mt + 4*g + r of row row0 + n as two packed dwords
+// (WIDE: features wide_feature(mt, 4*g + r) instead)
+template <bool WIDE = false>
 __device__ __forceinline__ uint2 load_tile_packed(const uint16_t* base, int64_t stride, int64_t row0, int64_t rows, int col0,
                                                   int width, int mt, int lane, bool vec_ok) {
   uint2 v = make_uint2(0u, 0u);
   const int64_t r = row0 + (lane & 15);
-  const int c = 16 * mt + 4 * (lane >> 4);
+  const int c = WIDE ? wide_feature(mt, 4 * (lane >> 4)) : 16 * mt + 4 * (lane >> 4);
   if (r < rows && c < width) {
     const uint16_t* p = base + r * stride + col0 + c;
     if (vec_ok && c + 4 <= width) {
@@ -57,10 +60,11 @@ __device__ __forceinline__ uint2 load_tile_packed(const uint16_t* base, int64_t 
   }
   return v;
 }
+template <bool WIDE = false>
 __device__ __forceinline__ void store_tile_packed(uint16_t* base, int64_t stride, int64_t row0, int64_t rows, int col0,
                                                   int width, int mt, int lane, uint2 v, bool vec_ok) {
   const int64_t r = row0 + (lane & 15);
-  const int c = 16 * mt + 4 * (lane >> 4);
+  const int c = WIDE ? wide_feature(mt, 4 * (lane >> 4)) : 16 * mt + 4 * (lane >> 4);
   if (r >= rows || c >= width) return;
   uint16_t* p = base + r * stride + col0 + c;
   if (vec_ok && c + 4 <= width) {
@@ -79,7 +83,7 @@ template <bool FAST>
 __device__ __forceinline__ uint2 ld_tile(const uint16_t* base, int64_t stride, int64_t row0, int64_t rows, int col0,
                                          int width, int mt, int lane, bool vec_ok) {
   if (FAST) return *reinterpret_cast<const uint2*>(base + (row0 + (lane & 15)) * stride + 4 * (lane >> 4) + col0 + 16 * mt);
-  return load_tile_packed(base, stride, row0, rows, col0, width, mt, lane, vec_ok);
+  return load_tile_packed<false>(base, stride, row0, rows, col0, width, mt, lane, vec_ok);
 }
 template <bool FAST>
 __device__ __forceinline__ void st_tile(uint16_t* base, int64_t stride, int64_t row0, int64_t rows, int col0, int width,
@@ -88,7 +92,20 @@ __device__ __forceinline__ void st_tile(uint16_t* base, int64_t stride, int64_t 
     *reinterpret_cast<uint2*>(base + (row0 + (lane & 15)) * stride + 4 * (lane >> 4) + col0 + 16 * mt) = v;
     return;
   }
-  store_tile_packed(base, stride, row0, rows, col0, width, mt, lane, v, vec_ok);
+  store_tile_packed<false>(base, stride, row0, rows, col0, width, mt, lane, v, vec_ok);
+}
+
+// Tiles 2p and 2p + 1 of a row tile in wide order (wide_feature()): lane (n, g) holds features 32p + 8g .. + 7 of row
+// row0 + n, one 16-byte access.  Only for full-width, 16-byte aligned, unragged tensors.
+__device__ __forceinline__ void ld_tile_pair(const uint16_t* base, int64_t stride, int64_t row0, int col0, int p, int lane,
+                                             uint2& t0, uint2& t1) {
+  const uint4 v = *reinterpret_cast<const uint4*>(base + (row0 + (lane & 15)) * stride + col0 + 32 * p + 8 * (lane >> 4));
+  t0 = make_uint2(v.x, v.y);
+  t1 = make_uint2(v.z, v.w);
+}
+__device__ __forceinline__ void st_tile_pair(uint16_t* base, int64_t stride, int64_t row0, int col0, int p, int lane, uint2 t0,
+                                             uint2 t1) {
+  *reinterpret_cast<uint4*>(base + (row0 + (lane & 15)) * stride + col0 + 32 * p + 8 * (lane >> 4)) = make_uint4(t0.x, t0.y, t1.x, t1.y);
 }
 
 template <typename T>
@@ -134,9 +151,13 @@ __device__ __forceinline__ void rev_layer(f32x4_t (&acc)[2][4], const Frag (&in)
     }
 }
 
-template <typename T>
+// WIDE: position 16*mt + m of the staged row holds the bias of feature wide_feature(mt, m)
+template <typename T, bool WIDE = false>
 __device__ __forceinline__ void stage_bias_row(float* dst, const uint16_t* b, int n_valid, int n_pad, int tid, int nthreads) {
-  for (int i = tid; i < n_pad; i += nthreads) dst[i] = (b != nullptr && i < n_valid) ? T::to_f32(b[i]) : 0.0f;
+  for (int i = tid; i < n_pad; i += nthreads) {
+    const int f = WIDE ? wide_feature(i >> 4, i & 15) : i;
+    dst[i] = (b != nullptr && f < n_valid) ? T::to_f32(b[f]) : 0.0f;
+  }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -335,16 +356,20 @@ __device__ __forceinline__ void sub_backward(const uint2 (&u)[2][4], const uint2
 }
 
 // Bias gradient of feature 16*mt + n: the four lane groups hold partial sums over disjoint rows.
+// WIDE: the tile's features are in wide order (wide_feature())
+template <bool WIDE = false>
 __device__ __forceinline__ void flush_db_rev(float* db, int dim, int mt, int lane, float v) {
   v += __shfl_xor(v, 16);
   v += __shfl_xor(v, 32);
-  const int f = 16 * mt + lane;
+  const int f = WIDE ? wide_feature(mt, lane & 15) : 16 * mt + lane;
   if (db != nullptr && lane < 16 && f < dim) unsafeAtomicAdd(db + f, v);
 }
 
+// WIDE_ROWS / WIDE_COLS: the tile's rows (mt) / columns (nt) are features in wide order
+template <bool WIDE_ROWS = false, bool WIDE_COLS = false>
 __device__ __forceinline__ void flush_tile(float* dw, int dim, int mt, int nt, int lane, f32x4_t v) {
-  const int c = 16 * nt + (lane & 15);
-  const int r0 = 16 * mt + 4 * (lane >> 4);
+  const int c = WIDE_COLS ? wide_feature(nt, lane & 15) : 16 * nt + (lane & 15);
+  const int r0 = WIDE_ROWS ? wide_feature(mt, 4 * (lane >> 4)) : 16 * mt + 4 * (lane >> 4);
   if (c >= dim) return;
 #pragma unroll
   for (int r = 0; r < 4; ++r)
@@ -354,6 +379,10 @@ __device__ __forceinline__ void flush_tile(float* dw, int dim, int mt, int nt, i
 template <typename T, int HP, int ACT, bool FAST>
 __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
   constexpr int MT = HP / 16, KC = HP / 32, LAYER = MT * KC * RFRAG;
+  // The backward keeps the stream's features in wide order: the unchecked variant then reaches its rows with 16-byte
+  // accesses, half as many of them (a tile access has one lane per row and line, so the vector memory pipeline sees every
+  // lane as an access of its own); the checked variant uses the same order, so both do the same arithmetic.
+  constexpr bool WIDE = true;
   const int act = ACT >= 0 ? ACT : a.act;
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, nthreads = blockDim.x, lane = tid & 63, wave = tid >> 6;
@@ -389,12 +418,13 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
   if (G2_LDS)
     for (int i = lane; i < MT * MT * 64; i += 64) g2acc[i] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
   for (int s = 0; s < 2; ++s) {
-    stage_weight_frags<true, false>(fw + (2 * s) * LAYER, w1 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
-    stage_weight_frags<true, false>(fw + (2 * s + 1) * LAYER, w2 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
-    stage_weight_frags<true, true>(tw + (2 * s) * LAYER, w1 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
-    stage_weight_frags<true, true>(tw + (2 * s + 1) * LAYER, w2 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
+    // WIDE: the stream's features are contracted in natural order and produced in wide order (the hidden ones as ever)
+    stage_weight_frags<!WIDE, false>(fw + (2 * s) * LAYER, w1 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
+    stage_weight_frags<true, false, 0, WIDE>(fw + (2 * s + 1) * LAYER, w2 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
+    stage_weight_frags<true, true, 0, WIDE>(tw + (2 * s) * LAYER, w1 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
+    stage_weight_frags<!WIDE, true>(tw + (2 * s + 1) * LAYER, w2 + (size_t)s * H * H, H, H, MT, KC, tid, nthreads);
     stage_bias_row<T>(bias + (2 * s) * HP, b1 ? b1 + (size_t)s * H : nullptr, H, HP, tid, nthreads);
-    stage_bias_row<T>(bias + (2 * s + 1) * HP, b2 ? b2 + (size_t)s * H : nullptr, H, HP, tid, nthreads);
+    stage_bias_row<T, WIDE>(bias + (2 * s + 1) * HP, b2 ? b2 + (size_t)s * H : nullptr, H, HP, tid, nthreads);
   }
   __syncthreads();
 
@@ -415,20 +445,37 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
     f32x4_t sout[2][4], du[2][4];
     {
       uint2 y1[2][4], d2[2][4], y2[2][4], dy1[2][4];
+      if constexpr (FAST) {
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+          for (int p = 0; p < MT / 2; ++p) {
+            ld_tile_pair(in_p, in_s, row0 + 16 * nt, 0, p, lane, y1[nt][2 * p], y1[nt][2 * p + 1]);
+            ld_tile_pair(dy_p, dy_s, row0 + 16 * nt, H, p, lane, d2[nt][2 * p], d2[nt][2 * p + 1]);
+          }
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+          for (int p = 0; p < MT / 2; ++p) {
+            ld_tile_pair(in_p, in_s, row0 + 16 * nt, H, p, lane, y2[nt][2 * p], y2[nt][2 * p + 1]);
+            ld_tile_pair(dy_p, dy_s, row0 + 16 * nt, 0, p, lane, dy1[nt][2 * p], dy1[nt][2 * p + 1]);
+          }
+      } else {
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          y1[nt][mt] = ld_tile<FAST>(in_p, in_s, row0 + 16 * nt, a.rows, 0, H, mt, lane, in_v);
-          d2[nt][mt] = ld_tile<FAST>(dy_p, dy_s, row0 + 16 * nt, a.rows, H, H, mt, lane, dy_v);
+          y1[nt][mt] = load_tile_packed<WIDE>(in_p, in_s, row0 + 16 * nt, a.rows, 0, H, mt, lane, in_v);
+          d2[nt][mt] = load_tile_packed<WIDE>(dy_p, dy_s, row0 + 16 * nt, a.rows, H, H, mt, lane, dy_v);
         }
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          y2[nt][mt] = ld_tile<FAST>(in_p, in_s, row0 + 16 * nt, a.rows, H, H, mt, lane, in_v);
-          dy1[nt][mt] = ld_tile<FAST>(dy_p, dy_s, row0 + 16 * nt, a.rows, 0, H, mt, lane, dy_v);
+          y2[nt][mt] = load_tile_packed<WIDE>(in_p, in_s, row0 + 16 * nt, a.rows, H, H, mt, lane, in_v);
+          dy1[nt][mt] = load_tile_packed<WIDE>(dy_p, dy_s, row0 + 16 * nt, a.rows, 0, H, mt, lane, dy_v);
         }
+      }
       // ---- G:  y2 = x2 + G(y1)  =>  x2 = y2 - G(y1),  dy1 += (dG/dy1)^T dy2
       sub_backward<T, MT, KC, ACT>(y1, d2, sout, du, dwG1, dwG2, g2acc, dbG1, dbG2, fw + 2 * LAYER, fw + 3 * LAYER,
                                    tw + 2 * LAYER, tw + 3 * LAYER, bias + 2 * HP, bias + 3 * HP, sel, act, lane);
@@ -443,27 +490,55 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
     {
       // the other halves again (L2 hits), in flight during F
       uint2 y1[2][4], d2[2][4];
+      if constexpr (FAST) {
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+          for (int p = 0; p < MT / 2; ++p) {
+            ld_tile_pair(in_p, in_s, row0 + 16 * nt, 0, p, lane, y1[nt][2 * p], y1[nt][2 * p + 1]);
+            ld_tile_pair(dy_p, dy_s, row0 + 16 * nt, H, p, lane, d2[nt][2 * p], d2[nt][2 * p + 1]);
+          }
+      } else {
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          y1[nt][mt] = ld_tile<FAST>(in_p, in_s, row0 + 16 * nt, a.rows, 0, H, mt, lane, in_v);
-          d2[nt][mt] = ld_tile<FAST>(dy_p, dy_s, row0 + 16 * nt, a.rows, H, H, mt, lane, dy_v);
+          y1[nt][mt] = load_tile_packed<WIDE>(in_p, in_s, row0 + 16 * nt, a.rows, 0, H, mt, lane, in_v);
+          d2[nt][mt] = load_tile_packed<WIDE>(dy_p, dy_s, row0 + 16 * nt, a.rows, H, H, mt, lane, dy_v);
         }
+      }
       // ---- F:  y1 = x1 + F(x2)  =>  x1 = y1 - F(x2),  dx2 = dy2 + (dF/dx2)^T dy1
       sub_backward<T, MT, KC, ACT>(x2, d1, sout, du, dwF1, dwF2, nullptr, dbF1, dbF2, fw, fw + LAYER, tw, tw + LAYER, bias,
                                    bias + HP, sel, act, lane);
+      if constexpr (FAST) {
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+          for (int p = 0; p < MT / 2; ++p) {
+            uint2 x1[2], dx2[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+              x1[e] = pack4<T>(unpack4<T>(y1[nt][2 * p + e]) - sout[nt][2 * p + e]);
+              dx2[e] = pack4<T>(unpack4<T>(d2[nt][2 * p + e]) + du[nt][2 * p + e]);
+            }
+            st_tile_pair(a.out, a.out_stride, row0 + 16 * nt, 0, p, lane, x1[0], x1[1]);
+            st_tile_pair(a.out, a.out_stride, row0 + 16 * nt, H, p, lane, x2[nt][2 * p], x2[nt][2 * p + 1]);
+            st_tile_pair(a.dx, a.dx_stride, row0 + 16 * nt, 0, p, lane, d1[nt][2 * p], d1[nt][2 * p + 1]);
+            st_tile_pair(a.dx, a.dx_stride, row0 + 16 * nt, H, p, lane, dx2[0], dx2[1]);
+          }
+      } else {
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           const uint2 x1 = pack4<T>(unpack4<T>(y1[nt][mt]) - sout[nt][mt]);
           const uint2 dx2 = pack4<T>(unpack4<T>(d2[nt][mt]) + du[nt][mt]);
-          st_tile<FAST>(a.out, a.out_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, x1, a.vec_out);
-          st_tile<FAST>(a.out, a.out_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, x2[nt][mt], a.vec_out);
-          st_tile<FAST>(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, d1[nt][mt], a.vec_dx);
-          st_tile<FAST>(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, dx2, a.vec_dx);
+          store_tile_packed<WIDE>(a.out, a.out_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, x1, a.vec_out);
+          store_tile_packed<WIDE>(a.out, a.out_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, x2[nt][mt], a.vec_out);
+          store_tile_packed<WIDE>(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, 0, H, mt, lane, d1[nt][mt], a.vec_dx);
+          store_tile_packed<WIDE>(a.dx, a.dx_stride, row0 + 16 * nt, a.rows, H, H, mt, lane, dx2, a.vec_dx);
         }
+      }
     }
   }
 
@@ -521,22 +596,22 @@ __global__ __launch_bounds__(256) void rev_bwd_block_k(RevArgs a) {
   for (int i = 0; i < MT; ++i)
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
-      flush_tile(gw1, H, i, j, lane, dwF1[i][j]);
-      flush_tile(gw2, H, i, j, lane, dwF2[i][j]);
-      flush_tile(gw1 + (size_t)H * H, H, i, j, lane, dwG1[i][j]);
+      flush_tile<false, WIDE>(gw1, H, i, j, lane, dwF1[i][j]);
+      flush_tile<WIDE, false>(gw2, H, i, j, lane, dwF2[i][j]);
+      flush_tile<false, WIDE>(gw1 + (size_t)H * H, H, i, j, lane, dwG1[i][j]);
       if (G2_LDS) {
         constexpr int PER_WAVE = MT * MT * 64;
         const int at = (i * MT + j) * 64 + lane;  // wave 0's g2acc is the first of the four
         dwG2[i][j] = (g2acc[at] + g2acc[PER_WAVE + at]) + (g2acc[2 * PER_WAVE + at] + g2acc[3 * PER_WAVE + at]);
       }
-      flush_tile(gw2 + (size_t)H * H, H, i, j, lane, dwG2[i][j]);
+      flush_tile<WIDE, false>(gw2 + (size_t)H * H, H, i, j, lane, dwG2[i][j]);
     }
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
     flush_db_rev(gb1, H, i, lane, dbF1[i]);
     flush_db_rev(gb1 ? gb1 + H : nullptr, H, i, lane, dbG1[i]);
-    flush_db_rev(gb2, H, i, lane, dbF2[i]);
-    flush_db_rev(gb2 ? gb2 + H : nullptr, H, i, lane, dbG2[i]);
+    flush_db_rev<WIDE>(gb2, H, i, lane, dbF2[i]);
+    flush_db_rev<WIDE>(gb2 ? gb2 + H : nullptr, H, i, lane, dbG2[i]);
   }
   }
   // wave 0 has read the other waves' LDS accumulators and the reduction area: both are rewritten for the next coupling
@@ -571,6 +646,7 @@ static int rev_validate(int64_t rows, int half, int blocks, int act, int dtype) 
 static bool vec8_ok(const void* p, int64_t stride, int half) {
   return ((uintptr_t)p % 8 == 0) && (stride % 4 == 0) && (half % 4 == 0);
 }
+static bool vec16_ok(const void* p, int64_t stride) { return ((uintptr_t)p % 16 == 0) && (stride % 8 == 0); }
 
 template <typename T, int HP>
 static int launch_rev_fwd(RevArgs a, hipStream_t s) {
@@ -611,7 +687,7 @@ static int launch_rev_bwd(RevArgs a, hipStream_t s) {
   // the weight-gradient accumulators take most of the register file: one wave per SIMD
   const int64_t cap = (int64_t)rev_cus();
   if (blocks > cap) blocks = cap;
-  const bool fast = a.half == HP && a.rows % 32 == 0 && a.vec_in && a.vec_out && a.vec_dy && a.vec_dx;
+  const bool fast = a.half == HP && a.rows % 32 == 0 && a.vec_in && a.vec_out && a.vec_dy && a.vec_dx && a.wide_ok;
   const void* kern = a.act == NF_ACT_GELU   ? (fast ? (const void*)rev_bwd_block_k<T, HP, NF_ACT_GELU, true>
                                                     : (const void*)rev_bwd_block_k<T, HP, NF_ACT_GELU, false>)
                      : a.act == NF_ACT_RELU ? (fast ? (const void*)rev_bwd_block_k<T, HP, NF_ACT_RELU, true>
@@ -683,7 +759,8 @@ extern "C" int nf_revmlp_bwd(const void* y, int64_t y_stride, const void* dy, in
   // first (the first reads (y, dy), the others continue in place on (x_rec, dx)); anything else one launch per coupling.
   const int hp = half <= 32 ? 32 : 64;
   const bool fused = half == hp && rows % 32 == 0 && (act == NF_ACT_GELU || act == NF_ACT_RELU) && vec8_ok(y, y_stride, half) &&
-                     vec8_ok(x_rec, x_rec_stride, half) && vec8_ok(dy, dy_stride, half) && vec8_ok(dx, dx_stride, half);
+                     vec8_ok(x_rec, x_rec_stride, half) && vec8_ok(dy, dy_stride, half) && vec8_ok(dx, dx_stride, half) &&
+                     vec16_ok(y, y_stride) && vec16_ok(x_rec, x_rec_stride) && vec16_ok(dy, dy_stride) && vec16_ok(dx, dx_stride);
   for (int k = blocks - 1; k >= 0; --k) {
     RevArgs a = {};
     const bool first = k == blocks - 1;
@@ -712,6 +789,7 @@ extern "C" int nf_revmlp_bwd(const void* y, int64_t y_stride, const void* dy, in
     a.vec_out = vec8_ok(a.out, a.out_stride, half);
     a.vec_dy = vec8_ok(a.dy, a.dy_stride, half);
     a.vec_dx = vec8_ok(a.dx, a.dx_stride, half);
+    a.wide_ok = fused;  // the unchecked kernel is the fused launch's
     int rc;
     if (half <= 32)
       rc = dtype == NF_BF16 ? launch_rev_bwd<BF16, 32>(a, s) : launch_rev_bwd<F16, 32>(a, s);
