@@ -309,14 +309,22 @@ __device__ __forceinline__ void sub_backward(const uint2 (&u)[2][4], const uint2
     for (int j = 0; j < MT; ++j) tb[j] = transpose_tile<T>(tf[0][j >> 1], tf[1][j >> 1], sel[j & 1]);
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
-      const Frag da = transpose_tile<T>(df[0][i >> 1], df[1][i >> 1], sel[i & 1]);
       if (dw2_lds != nullptr) {
+        // the row's accumulator tiles are asked for before the transpose that their products wait for anyway
+        f32x4_t c[MT];
 #pragma unroll
-        for (int j = 0; j < MT; ++j) {
-          f32x4_t* slot = dw2_lds + (i * MT + j) * 64 + lane;
-          *slot = mfma16<T>(da, tb[j], *slot);
-        }
-      } else {
+        for (int j = 0; j < MT; ++j) c[j] = dw2_lds[(i * MT + j) * 64 + lane];
+        const Frag da = transpose_tile<T>(df[0][i >> 1], df[1][i >> 1], sel[i & 1]);
+#pragma unroll
+        for (int j = 0; j < MT; ++j) c[j] = mfma16<T>(da, tb[j], c[j]);
+#pragma unroll
+        for (int j = 0; j < MT; ++j) dw2_lds[(i * MT + j) * 64 + lane] = c[j];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) db2[i] = dot2_ones<T>(da.w[q], db2[i]);
+        continue;
+      }
+      const Frag da = transpose_tile<T>(df[0][i >> 1], df[1][i >> 1], sel[i & 1]);
+      {
 #pragma unroll
         for (int j = 0; j < MT; ++j) dw2[i][j] = mfma16<T>(da, tb[j], dw2[i][j]);
       }
