@@ -114,6 +114,17 @@ __device__ __forceinline__ float normal_cdf_pdf(float z, float* pdf) {
   return z >= 0.0f ? 1.0f - q : q;
 }
 
+// The same with the three-term form (Abramowitz & Stegun 7.1.25, absolute error of Phi and of Phi + z phi below 1.1e-5:
+// half of what the forward's polynomial allows itself), fifteen instructions for both instead of eighteen; the scale
+// 1/sqrt 2 of the argument is folded into the constants.
+__device__ __forceinline__ float normal_cdf_pdf3(float z, float* pdf) {
+  const float t = __builtin_amdgcn_rcpf(fmaf(0.33267252f, fabsf(z), 1.0f));  // 1 / (1 + 0.47047 |z| / sqrt 2); v_rcp_f32, 1 ulp
+  const float e = __builtin_amdgcn_exp2f(z * z * -0.72134752f);              // exp(-z^2 / 2)
+  const float q = t * (0.1740121f + t * (-0.0479399f + t * 0.3739278f)) * e;  // Phi(-|z|), the 1/2 folded into the coefficients
+  *pdf = 0.3989422804014327f * e;
+  return z >= 0.0f ? 1.0f - q : q;
+}
+
 // ---- activations (triton_helpers/ops.py:37-66 of the reference; gelu = erf form) ----
 __device__ __forceinline__ float act_fwd(float z, int act) {
   switch (act) {

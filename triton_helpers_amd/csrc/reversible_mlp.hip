@@ -250,7 +250,7 @@ template <int ACT>
 __device__ __forceinline__ void act_both(float z, float& h, float& g) {
   if (ACT == NF_ACT_GELU) {
     float pdf;
-    const float cdf = normal_cdf_pdf(z, &pdf);
+    const float cdf = normal_cdf_pdf3(z, &pdf);
     h = z * cdf;
     g = cdf + z * pdf;
   } else if (ACT == NF_ACT_RELU) {
