@@ -9,8 +9,11 @@
 // (x2 = y2 - G(y1), x1 = y1 - F(x2)) while it back-propagates, and writes (x, dx), which it reads
 // back in place for the block below after restaging that block's weights.  No activation
 // of the forward pass is ever stored.  The four weight gradients of a block accumulate in
-// float32 registers over the wave's whole row loop; their operands (rows along K) are matrix-core
-// transposes of the row-per-lane fragments, so LDS only holds weights.
+// float32 registers over the wave's whole row loop (the fourth of a 64-wide block in LDS); their
+// operands (rows along K) are matrix-core transposes of the row-per-lane fragments, so LDS otherwise
+// only holds weights.  The backward numbers the stream's features in "wide order" (wide_feature()
+// in mlp_tile.h), which lets a lane reach the eight features of two accumulator tiles with one
+// 16-byte access; the staged weights and the flushed gradients absorb the permutation.
 //
 // There is no counterpart in the reference; the layer math is that of its fused MLP
 // (triton_helpers/layers/fully_fused_mlp/kernel.py:17-74).
