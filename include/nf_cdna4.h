@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define NF_ABI_VERSION 8
+#define NF_ABI_VERSION 9
 
 /* element types */
 enum { NF_F32 = 0, NF_F16 = 1, NF_BF16 = 2 };
@@ -69,7 +69,8 @@ enum {
   NF_HASH_FORCE_GENERIC = 1,   /* use the one-thread-per-(point,level) kernel even where a faster kernel applies */
   NF_HASH_FORCE_ATOMIC = 2,    /* backward: scatter with global atomics even where the LDS-tile kernels apply */
   NF_HASH_FORCE_PLANES = 4,    /* backward: of the two LDS-tile variants take the bit-plane one (smaller workspace) */
-  NF_HASH_FWD_STAGED = 8       /* forward: the LDS-staged tile kernel instead of the register-resident level sweep */
+  NF_HASH_FWD_STAGED = 8,      /* forward: the LDS-staged tile kernel instead of the register-resident level sweep */
+  NF_HASH_BWD_RECORDS = 16     /* backward: the sorted-record kernels even where a level is so few bins that the walk without records applies */
 };
 
 int nf_abi_version(void);
@@ -96,7 +97,9 @@ int nf_hash_encode_bwd(const void* coords, int coords_dtype, int64_t coords_stri
                        int64_t workspace_bytes, int flags, void* stream);
 
 /* Scratch bytes nf_hash_encode_bwd can use for this call shape and these flags (NF_HASH_FORCE_PLANES gives the
- * size of the smaller variant); 0 when the workspace would not be used.
+ * size of the smaller variant; tables of at most 2^14 rows per level take a walk without records and ask for
+ * 4 bytes -- 8 with a float32 gradient -- per point, level and feature pair unless NF_HASH_BWD_RECORDS is set);
+ * 0 when the workspace would not be used.
  * (No counterpart in the reference: its backward allocates nothing besides the gradient table,
  * triton_helpers/layers/hash_encoding/kernel.py:636.) */
 int64_t nf_hash_encode_bwd_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype, int flags);

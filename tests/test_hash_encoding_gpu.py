@@ -445,6 +445,77 @@ def test_backward_binned_dense_levels_of_several_bins(do_dtype):
     assert float(got.cpu()[want == 0].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize(
+    "N,D,F,T,L,lo,hi,do_dtype",
+    [
+        (150001, 3, 2, 2**14, 16, 16, 512, torch.float16),   # the reference's default geometry (kernel.py:682-686)
+        (140000, 3, 2, 2**14, 16, 16, 512, torch.float32),
+        (131072, 2, 2, 2**13, 8, 16, 512, torch.bfloat16),
+        (135000, 3, 4, 12345, 8, 8, 256, torch.float16),     # two passes of feature pairs, exact 64-bit remainder
+        (133000, 3, 1, 2**14, 4, 16, 128, torch.float16),    # odd feature counts: the last pair has one feature
+        (133000, 3, 3, 2**14, 4, 16, 128, torch.float32),
+        (2**21 + 5000, 3, 2, 2**14, 2, 16, 64, torch.float16),  # more than one piece of 2^21 points
+    ],
+)
+def test_backward_without_records(N, D, F, T, L, lo, hi, do_dtype, monkeypatch):
+    """Tables whose levels are at most two bins (2^14 rows) take the walk without records: a workgroup per level and
+    feature (or per level, for a level of one bin) hashes a slice of the points and adds every corner to its LDS tile.
+    Against the oracle, against the sorted-record kernels (flag NF_HASH_BWD_RECORDS), with a smaller workspace, and
+    with rows that no point touches left exactly zero."""
+    from triton_helpers_amd import _lib
+
+    hk = _hk()
+    torch.manual_seed(5)
+    x = torch.rand(N, D)
+    x[:500, 0] = 1.0                                   # the upper edge of the first coordinate
+    x[500:1000] = torch.randint(0, hi, (500, D)).float() / hi   # grid nodes of the finest level: weights exactly 0 and 1
+    x[1000:20000] = torch.rand(1, D) * 0.9 + 1e-3 * torch.rand(19000, D)  # a cluster in one cell of the coarse levels
+    E = O.level_row_offsets(L, T, D, lo, hi)[-1]
+    do = torch.randn(N, L * F).to(do_dtype)
+    want = O.encode_backward(x, do, E, F, None, T, L, lo, hi)
+    geom = hk.level_geometry(T, L, D, F, lo, hi)
+    lib = _lib.load()
+    need = lib.nf_hash_encode_bwd_workspace_bytes(N, geom, _lib.dtype_code(do_dtype), 0)
+    need_records = lib.nf_hash_encode_bwd_workspace_bytes(N, geom, _lib.dtype_code(do_dtype), _lib.NF_HASH_BWD_RECORDS)
+    assert 0 < need < need_records, (need, need_records)
+    got = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, F, None, T, lo, hi, L).cpu()
+    monkeypatch.setattr(hk, "_FLAGS", _lib.NF_HASH_BWD_RECORDS)
+    records = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, F, None, T, lo, hi, L).cpu()
+    peak = float(want.abs().max())
+    torch.testing.assert_close(got, want, rtol=1e-3, atol=1e-5 * peak)   # float weights: tighter than the records' bound
+    torch.testing.assert_close(records, want, rtol=1e-3, atol=1e-4 * peak)
+    touched = O.encode_backward(x, torch.ones_like(do, dtype=torch.float32), E, F, None, T, L, lo, hi) != 0
+    assert float(got[~touched].abs().max()) == 0.0 if bool((~touched).any()) else True
+
+
+def test_backward_without_records_nonfinite_gradient():
+    """An inf in the upstream gradient of one level: that level's touched rows come out NaN, as from the record kernels,
+    and every other level is unaffected."""
+    from triton_helpers_amd import _lib
+
+    hk = _hk()
+    torch.manual_seed(6)
+    N, D, F, T, L, lo, hi = 140000, 3, 2, 2**14, 4, 16, 128
+    x = torch.rand(N, D)
+    offs = O.level_row_offsets(L, T, D, lo, hi)
+    E = offs[-1]
+    do = torch.randn(N, L * F).half()
+    clean = O.encode_backward(x, do, E, F, None, T, L, lo, hi)
+    do[777, 2 * 2] = float("inf")
+    got = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, F, None, T, lo, hi, L).cpu()
+    hk_flags = hk._FLAGS
+    try:
+        hk._FLAGS = _lib.NF_HASH_BWD_RECORDS
+        records = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, F, None, T, lo, hi, L).cpu()
+    finally:
+        hk._FLAGS = hk_flags
+    lvl = slice(offs[2], offs[3])
+    assert torch.equal(torch.isnan(got), torch.isnan(records))
+    assert bool(torch.isnan(got[lvl]).any()) and not bool(torch.isnan(got[: offs[2]]).any()) and not bool(torch.isnan(got[offs[3] :]).any())
+    keep = ~torch.isnan(got)
+    torch.testing.assert_close(got[keep], clean[keep], rtol=1e-3, atol=1e-5 * float(clean.abs().max()))
+
+
 @pytest.mark.parametrize("level", [1, 2])
 @pytest.mark.parametrize("do_dtype", [torch.float16, torch.float32])
 def test_backward_binned_nonfinite_gradient(do_dtype, level):
@@ -675,19 +746,23 @@ def test_full_size_properties_config1():
     torch.testing.assert_close(oc.float(), torch.full_like(oc, 0.25, dtype=torch.float32), rtol=1e-3, atol=0)
 
 
-def test_backward_in_pieces_beyond_two_million_points():
-    """Batches above 2^21 points run through the sort-and-accumulate pipeline in pieces: the workspace stops growing and
-    the gradient equals the sum of the halves' gradients computed separately."""
+@pytest.mark.parametrize("records", [False, True])
+def test_backward_in_pieces_beyond_two_million_points(records, monkeypatch):
+    """Batches above 2^21 points run in pieces, through the walk without records (this geometry's default) and through
+    the sort-and-accumulate pipeline alike: the workspace stops growing and the gradient equals the sum of the halves'
+    gradients computed separately."""
     from triton_helpers_amd import _lib
 
     hk = _hk()
+    flags = _lib.NF_HASH_BWD_RECORDS if records else 0
+    monkeypatch.setattr(hk, "_FLAGS", flags)
     T, L, lo, hi = 2**14, 16, 16, 512
     E = O.level_row_offsets(L, T, 3, lo, hi)[-1]
     from triton_helpers_amd.layers.hash_encoding.helpers import level_geometry
 
     geom = level_geometry(T, L, 3, 2, lo, hi)
     lib = _lib.load()
-    assert lib.nf_hash_encode_bwd_workspace_bytes(2**22, geom, _lib.NF_F16, 0) == lib.nf_hash_encode_bwd_workspace_bytes(2**21, geom, _lib.NF_F16, 0)
+    assert lib.nf_hash_encode_bwd_workspace_bytes(2**22, geom, _lib.NF_F16, flags) == lib.nf_hash_encode_bwd_workspace_bytes(2**21, geom, _lib.NF_F16, flags)
     N = 2**21 + 12345
     g = torch.Generator().manual_seed(3)
     x = torch.rand(N, 3, generator=g).to(DEV)

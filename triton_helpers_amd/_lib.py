@@ -14,7 +14,7 @@ import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "libnf_cdna4.so"
 
-NF_ABI_VERSION = 8
+NF_ABI_VERSION = 9
 NF_F32, NF_F16, NF_BF16 = 0, 1, 2
 NF_ACT = {"none": 0, "relu": 1, "silu": 2, "relu2": 3, "gelu": 4}
 NF_MAX_LEVELS = 32
@@ -24,6 +24,7 @@ NF_HASH_FORCE_GENERIC = 1
 NF_HASH_FORCE_ATOMIC = 2
 NF_HASH_FORCE_PLANES = 4
 NF_HASH_FWD_STAGED = 8
+NF_HASH_BWD_RECORDS = 16
 NF_ADAM_CLEAR_GRAD, NF_ADAM_SKIP_NONFINITE = 1, 2
 
 _DTYPE_CODE = {torch.float32: NF_F32, torch.float16: NF_F16, torch.bfloat16: NF_BF16}

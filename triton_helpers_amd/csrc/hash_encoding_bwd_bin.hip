@@ -782,6 +782,196 @@ __global__ __launch_bounds__(ACC_THREADS) void hash_bwd_bin_accum_k(const typena
 }
 
 // ---------------------------------------------------------------------------------------
+// Levels of a few bins: no records
+// ---------------------------------------------------------------------------------------
+// When a level's table is only a few bins (the reference's default of 2^14 rows per level is two), a sorted record per
+// corner pair costs more than hashing a point once per bin: a workgroup owns one bin and a slice of the points, walks
+// the slice, hashes each point's corners and adds those that fall into its bin to the same 64-bit fixed-point LDS tile
+// as the record kernels, then adds the tile to the table.  The upstream gradient is transposed first into level-major
+// pairs, so that a bin's walk reads 4 (float32: 8) contiguous bytes per point instead of touching a whole row; the same
+// pass takes the per-level maxima that set the fixed-point scales.
+constexpr int DIRECT_THREADS = 1024;
+constexpr int DIRECT_PREP_THREADS = 256;
+
+// pairs[(level * np + p) * N + n] = features 2p, 2p + 1 of the level's gradient of point n (np = ceil(feat / 2); a missing
+// partner is zero); gmax[level] = largest |gradient| pattern of the level over all its features
+template <bool G32>
+__global__ __launch_bounds__(DIRECT_PREP_THREADS) void hash_bwd_direct_prep_k(const void* dout_v, int64_t dout_stride, int64_t N,
+                                                                               int levels, int feat, uint32_t* pairs, uint32_t* gmax) {
+  __shared__ uint32_t lmax[NF_MAX_LEVELS];
+  const int tid = threadIdx.x, lane = tid & 63;
+  if (tid < NF_MAX_LEVELS) lmax[tid] = 0u;
+  __syncthreads();
+  const int64_t n = (int64_t)blockIdx.x * DIRECT_PREP_THREADS + tid;
+  const bool valid = n < N;
+  const int np = (feat + 1) / 2;
+  const uint16_t* row16 = reinterpret_cast<const uint16_t*>(dout_v) + (valid ? n : 0) * dout_stride;
+  const float* row32 = reinterpret_cast<const float*>(dout_v) + (valid ? n : 0) * dout_stride;
+  // an even row width with 4-byte aligned rows: a pair is one dword
+  const bool dword_pairs = !G32 && (feat & 1) == 0 && ((uintptr_t)dout_v & 3u) == 0 && (dout_stride & 1) == 0;
+  // rows of up to sixteen levels of one pair each, 16-byte aligned: the row in four loads, level l in dword l
+  const bool row_vec = !G32 && feat == 2 && levels <= 16 && (levels & 3) == 0 && ((uintptr_t)dout_v & 15u) == 0 && (dout_stride & 7) == 0;
+  if (row_vec) {
+    uint32_t gr[16];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint4 t = make_uint4(0u, 0u, 0u, 0u);
+      if (valid && 4 * i < levels) t = reinterpret_cast<const uint4*>(row16)[i];
+      gr[4 * i] = t.x;
+      gr[4 * i + 1] = t.y;
+      gr[4 * i + 2] = t.z;
+      gr[4 * i + 3] = t.w;
+    }
+#pragma unroll
+    for (int l = 0; l < 16; ++l) {
+      if (l >= levels) break;
+      if (valid) pairs[(int64_t)l * N + n] = gr[l];
+      const uint32_t pk = gr[l] & 0x7fff7fffu;
+      const uint32_t m = wave_max_u32(max(pk & 0xffffu, pk >> 16));
+      if (lane == 63 && m) atomicMax(lmax + l, m);
+    }
+  } else
+  for (int l = 0; l < levels; ++l) {
+    uint32_t m = 0u;
+    for (int p = 0; p < np; ++p) {
+      const int e0 = l * feat + 2 * p;
+      const bool two = 2 * p + 1 < feat;
+      const int64_t at = ((int64_t)l * np + p) * N + n;
+      if (G32) {
+        uint2 pair = make_uint2(0u, 0u);
+        if (valid) {
+          pair.x = __float_as_uint(row32[e0]);
+          if (two) pair.y = __float_as_uint(row32[e0 + 1]);
+          reinterpret_cast<uint2*>(pairs)[at] = pair;
+        }
+        const uint32_t a0 = pair.x & 0x7fffffffu, a1 = pair.y & 0x7fffffffu;
+        m = max(m, max(a0, a1));
+      } else {
+        uint32_t packed = 0u;
+        if (valid) {
+          if (dword_pairs) {
+            packed = reinterpret_cast<const uint32_t*>(row16)[e0 >> 1];
+          } else {
+            packed = row16[e0];
+            if (two) packed |= (uint32_t)row16[e0 + 1] << 16;
+          }
+          pairs[at] = packed;
+        }
+        const uint32_t pk = packed & 0x7fff7fffu;
+        m = max(m, max(pk & 0xffffu, pk >> 16));
+      }
+    }
+    m = wave_max_u32(m);
+    if (lane == 63 && m) atomicMax(lmax + l, m);
+  }
+  __syncthreads();
+  if (tid < levels) {
+    const uint32_t m = lmax[tid];
+    if (m > *(volatile uint32_t*)(gmax + tid)) atomicMax(gmax + tid, m);
+  }
+}
+
+// blockIdx.x: a task, numbered like the bins of BinPlan; blockIdx.y: the slice of the points.  Every level here is one or
+// two bins.  A level of one bin is one task whose tile holds both features of the pair; a level of two bins is two
+// tasks, one per feature of the pair, whose tile holds that feature of all the level's rows: either way every corner of a
+// point lands in the tile, so the walk has no test per corner and its LDS adds run with all lanes.
+template <typename GT, int D>
+__global__ __launch_bounds__(DIRECT_THREADS) void hash_bwd_direct_k(const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                                     const uint32_t* pairs, int64_t N, DevGeom g, BinPlan bp,
+                                                                     const int64_t* primes, float scale, const uint32_t* gmax,
+                                                                     float* dtable, int feat, int p, int64_t slice_points) {
+  typedef typename BinRec<GT>::type Rec;
+  constexpr bool G32 = sizeof(Rec) == 16;
+  extern __shared__ unsigned long long acc_tile[];  // 2 * BIN_ROWS sums
+  const int tid = threadIdx.x;
+  int l = 0;
+  while (l + 1 < bp.n_levels && (int)blockIdx.x >= bp.binbase[l + 1]) ++l;
+  const uint32_t which = blockIdx.x - (uint32_t)bp.binbase[l];
+  const bool by_feature = bp.nbins[l] == 2;
+  const int np = (feat + 1) / 2, f0 = 2 * p;
+  const bool has_pair = f0 + 1 < feat;
+  if (by_feature && which == 1u && !has_pair) return;  // an odd feature count: the last pair has one feature
+  const uint32_t nrows = g.rows[l];                    // <= 2 * BIN_ROWS, and <= BIN_ROWS unless by_feature
+  // fixed-point scale 2^se of the level, as in the record kernels:  |w * g| * 2^se < 2^30
+  const float gm = BinRec<GT>::level_max(gmax[l]);
+  const bool nonfinite = !(gm <= 3.0e38f);
+  int se = 0;
+  if (!nonfinite && gm > 0.0f) {
+    int ex;
+    frexpf(gm, &ex);
+    se = 30 - ex;
+    se = se > 120 ? 120 : se;
+  }
+  // |g| * 2^se < 2^30: the scaled gradient is a float (the two steps are exact powers of two inside float range)
+  const float s_lo = nonfinite ? 0.0f : ldexpf(1.0f, se / 2), s_hi = ldexpf(1.0f, se - se / 2);
+  const uint32_t ncells = by_feature ? nrows : 2u * BIN_ROWS;
+  for (uint32_t i = tid; i < ncells; i += DIRECT_THREADS) acc_tile[i] = 0ull;
+  lds_barrier();
+  const bool hashed = l >= g.first_hash;
+  const float fres = (float)g.res[l];
+  const uint32_t res = (uint32_t)g.res[l], mask = g.rows[l] - 1u;
+  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], D > 2 ? (uint32_t)primes[D > 2 ? 2 : 0] : 0u};
+  const uint32_t* level_pairs = pairs + (((int64_t)l * np + p) * N) * (G32 ? 2 : 1);
+  const int64_t n_begin = (int64_t)blockIdx.y * slice_points;
+  const int64_t n_end = n_begin + slice_points < N ? n_begin + slice_points : N;
+  // one point per thread and turn: the sixteen waves of the workgroup keep enough loads in flight, and more points per
+  // thread only cost registers (two: +4 %, eight: +70 %)
+  for (int64_t n = n_begin + tid; n < n_end; n += DIRECT_THREADS) {
+    float v[3] = {0.0f, 0.0f, 0.0f};
+    Rec rec = BinRec<GT>::zero();
+    load_point_d<D>(coords, cdt, csn, csd, n, scale, v);
+    if constexpr (G32) {
+      const uint2 t = reinterpret_cast<const uint2*>(level_pairs)[n];
+      rec.z = t.x;
+      rec.w = t.y;
+    } else {
+      rec.z = level_pairs[n];
+    }
+    uint32_t row[1 << D];
+    float w[1 << D];
+    cell_rows<D>(v, fres, hashed, res, mask, pi, primes, row, w);
+    const float g0 = BinRec<GT>::g0(rec) * s_lo * s_hi, g1 = BinRec<GT>::g1(rec) * s_lo * s_hi;
+    if (by_feature) {
+      const float gs = which ? g1 : g0;
+#pragma unroll
+      for (int j = 0; j < (1 << D); ++j) {
+        // a level with an inf or a nan in its gradient only marks the rows it touches
+        const int32_t fv = nonfinite ? (int32_t)(w[j] != 0.0f) : __float2int_rn(w[j] * gs);
+        if (fv) atomicAdd(acc_tile + row[j], (unsigned long long)(long long)fv);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < (1 << D); ++j) {
+        int32_t f0v, f1v;
+        if (nonfinite) {
+          f0v = w[j] != 0.0f;
+          f1v = has_pair && f0v;
+        } else {
+          f0v = __float2int_rn(w[j] * g0);
+          f1v = __float2int_rn(w[j] * g1);
+        }
+        if (f0v) atomicAdd(acc_tile + row[j], (unsigned long long)(long long)f0v);
+        if (f1v) atomicAdd(acc_tile + (uint32_t)BIN_ROWS + row[j], (unsigned long long)(long long)f1v);
+      }
+    }
+  }
+  lds_barrier();
+  float* dst = dtable + g.row_offset[l] * feat + f0;
+  const float qnan = __uint_as_float(0x7fc00000u);
+  const uint32_t nvals = by_feature ? nrows : 2u * nrows;
+  for (uint32_t i = tid; i < nvals; i += DIRECT_THREADS) {
+    // by feature: value i is row i of feature `which`; else value i is feature i & 1 of row i >> 1
+    const uint32_t r = by_feature ? i : i >> 1, f = by_feature ? which : (i & 1u);
+    if (f && !has_pair) continue;
+    const long long a = (long long)acc_tile[by_feature ? r : f * (uint32_t)BIN_ROWS + r];
+    if (a == 0) continue;
+    // |a| < 2^53 is exact in double and so is the division by 2^se: one rounding, to float
+    const float x = nonfinite ? qnan : (float)ldexp((double)a, -se);
+    if (x != 0.0f) unsafeAtomicAdd(dst + (int64_t)r * feat + f, x);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------------
 // Plan for levels la .. lb-1 (the kernels see them as levels 0 .. lb-la-1 of a shifted geometry).
@@ -871,8 +1061,27 @@ static int64_t bin_ws(void* workspace, const BinPlan& bp, int64_t N, int64_t R, 
 // and cost 2.5 % of a 2^21-point training step: every piece pays the fixed part of the pipeline again.)
 constexpr int64_t BIN_CHUNK_POINTS = (int64_t)1 << 21;
 
-int64_t bwd_bin_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype) {
+// The walk without records hashes every point once per task of a level (two for a level of two bins); the records pay a
+// count, a fill and an accumulate pass per level whatever its size.  With every level at most two bins (2^14 rows, the
+// reference's default table size) the walk is the faster one; four bins would already cost it more hashing than the
+// records' passes take.
+constexpr int DIRECT_MAX_BINS_PER_LEVEL = 2;
+constexpr int64_t DIRECT_MIN_POINTS = (int64_t)1 << 17;
+static bool direct_ok(int64_t n_points, const nf_hash_geom* geom, int flags) {
+  if ((flags & NF_HASH_BWD_RECORDS) || n_points < DIRECT_MIN_POINTS) return false;
+  if (geom->dims != 2 && geom->dims != 3) return false;
+  for (int l = 0; l < geom->levels; ++l)
+    if (geom->rows[l] > (int64_t)DIRECT_MAX_BINS_PER_LEVEL * BIN_ROWS) return false;
+  return true;
+}
+// gmax[32] (padded to 256 bytes) | pairs[levels][ceil(feat / 2)][n_points] of 4 (float32 gradient: 8) bytes
+static int64_t direct_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype) {
+  return 256 + (int64_t)geom->levels * ((geom->feat + 1) / 2) * n_points * (dout_dtype == NF_F32 ? 8 : 4);
+}
+
+int64_t bwd_bin_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype, int flags) {
   if (n_points > BIN_CHUNK_POINTS) n_points = BIN_CHUNK_POINTS;
+  if (direct_ok(n_points, geom, flags)) return direct_workspace_bytes(n_points, geom, dout_dtype);
   LevelGroups first;
   if (!bin_groups(n_points, geom, &first)) return 0;
   int64_t bytes = 0;
@@ -896,14 +1105,87 @@ static int launch_bwd_bin_piece(const void* coords, int cdt, int64_t csn, int64_
                                 float* dtable, int64_t N, const nf_hash_geom* geom, const DevGeom& g, const int64_t* primes, float scale,
                                 void* workspace, hipStream_t s);
 
+static int launch_bwd_direct(const void* coords, int cdt, int64_t csn, int64_t csd, const void* dout, int ddt, int64_t dout_stride,
+                             float* dtable, int64_t N, const nf_hash_geom* geom, const DevGeom& g, const int64_t* primes, float scale,
+                             void* workspace, hipStream_t s);
+
 int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const void* dout, int ddt, int64_t dout_stride,
                    float* dtable, int64_t N, const nf_hash_geom* geom, const DevGeom& g, const int64_t* primes, float scale,
-                   void* workspace, hipStream_t s) {
+                   void* workspace, int flags, hipStream_t s) {
+  // the choice is made once, on the size the workspace was asked for: every piece then fits it
+  const bool direct = direct_ok(N < BIN_CHUNK_POINTS ? N : BIN_CHUNK_POINTS, geom, flags);
   for (int64_t n0 = 0; n0 < N; n0 += BIN_CHUNK_POINTS) {
     const int64_t n = N - n0 < BIN_CHUNK_POINTS ? N - n0 : BIN_CHUNK_POINTS;
     const char* c = (const char*)coords + n0 * csn * dtype_size(cdt);
     const char* d = (const char*)dout + n0 * dout_stride * dtype_size(ddt);
-    if (int rc = launch_bwd_bin_piece(c, cdt, csn, csd, d, ddt, dout_stride, dtable, n, geom, g, primes, scale, workspace, s)) return rc;
+    const int rc = direct ? launch_bwd_direct(c, cdt, csn, csd, d, ddt, dout_stride, dtable, n, geom, g, primes, scale, workspace, s)
+                          : launch_bwd_bin_piece(c, cdt, csn, csd, d, ddt, dout_stride, dtable, n, geom, g, primes, scale, workspace, s);
+    if (rc) return rc;
+  }
+  return 0;
+}
+
+static int direct_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) cus = p.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+static int launch_bwd_direct(const void* coords, int cdt, int64_t csn, int64_t csd, const void* dout, int ddt, int64_t dout_stride,
+                             float* dtable, int64_t N, const nf_hash_geom* geom, const DevGeom& g, const int64_t* primes, float scale,
+                             void* workspace, hipStream_t s) {
+  NF_REQUIRE(((uintptr_t)workspace & 15u) == 0, NF_EALIGN, "workspace must be 16-byte aligned");
+  BinPlan bp;
+  int64_t R;
+  uint32_t max_tasks;
+  NF_REQUIRE(bin_plan(N, geom, 0, geom->levels, &bp, &R, &max_tasks, false), NF_EUNSUPPORTED,
+             "backward without records does not cover this geometry");
+  const int NB = bp.binbase[bp.n_levels];
+  uint32_t* gmax = reinterpret_cast<uint32_t*>(workspace);
+  uint32_t* pairs = gmax + 64;
+  const bool g32 = ddt == NF_F32;
+  hipLaunchKernelGGL(hash_bwd_bin_zero_k, dim3(1), dim3(64), 0, s, gmax, 32);
+  if (int rc = check_launch("hash_bwd_bin_zero")) return rc;
+  const unsigned prep_blocks = (unsigned)((N + DIRECT_PREP_THREADS - 1) / DIRECT_PREP_THREADS);
+  if (g32)
+    hipLaunchKernelGGL(hash_bwd_direct_prep_k<true>, dim3(prep_blocks), dim3(DIRECT_PREP_THREADS), 0, s, dout, dout_stride, N,
+                       g.levels, g.feat, pairs, gmax);
+  else
+    hipLaunchKernelGGL(hash_bwd_direct_prep_k<false>, dim3(prep_blocks), dim3(DIRECT_PREP_THREADS), 0, s, dout, dout_stride, N,
+                       g.levels, g.feat, pairs, gmax);
+  if (int rc = check_launch("hash_bwd_direct_prep")) return rc;
+  // at most two workgroups per compute unit in all, so that they run as two full rounds (one fits at a time: the tile is
+  // 128 KiB of LDS; four rounds: +3 %, eight: +11 %), in slices of whole turns of the point loop and of at least 16384 points
+  const int64_t round = (int64_t)DIRECT_THREADS;
+  int64_t slices = (int64_t)2 * direct_cus() / NB;
+  if (slices < 1) slices = 1;
+  int64_t slice_points = (N + slices - 1) / slices;
+  if (slice_points < 16384) slice_points = 16384;
+  slice_points = (slice_points + round - 1) / round * round;
+  slices = (N + slice_points - 1) / slice_points;
+  const size_t lds = (size_t)2 * BIN_ROWS * sizeof(unsigned long long);
+  const void* kern = g.dims == 3 ? (ddt == NF_F32    ? (const void*)hash_bwd_direct_k<F32, 3>
+                                    : ddt == NF_BF16 ? (const void*)hash_bwd_direct_k<BF16, 3>
+                                                     : (const void*)hash_bwd_direct_k<F16, 3>)
+                                 : (ddt == NF_F32    ? (const void*)hash_bwd_direct_k<F32, 2>
+                                    : ddt == NF_BF16 ? (const void*)hash_bwd_direct_k<BF16, 2>
+                                                     : (const void*)hash_bwd_direct_k<F16, 2>);
+  hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  const uint32_t* cpairs = pairs;
+  const uint32_t* cgmax = gmax;
+  const int feat = geom->feat;
+  for (int p = 0; p < (feat + 1) / 2; ++p) {
+    void* args[] = {(void*)&coords, (void*)&cdt, (void*)&csn, (void*)&csd, (void*)&cpairs, (void*)&N, (void*)&g, (void*)&bp,
+                    (void*)&primes, (void*)&scale, (void*)&cgmax, (void*)&dtable, (void*)&feat, (void*)&p, (void*)&slice_points};
+    e = hipLaunchKernel(kern, dim3((unsigned)NB, (unsigned)slices), dim3(DIRECT_THREADS), args, lds, s);
+    if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(hash_bwd_direct): %s", hipGetErrorString(e));
+    if (int rc = check_launch("hash_bwd_direct")) return rc;
   }
   return 0;
 }
