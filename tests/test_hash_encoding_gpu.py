@@ -455,6 +455,8 @@ def test_backward_binned_dense_levels_of_several_bins(do_dtype):
         (133000, 3, 1, 2**14, 4, 16, 128, torch.float16),    # odd feature counts: the last pair has one feature
         (133000, 3, 3, 2**14, 4, 16, 128, torch.float32),
         (2**21 + 5000, 3, 2, 2**14, 2, 16, 64, torch.float16),  # more than one piece of 2^21 points
+        (4099, 3, 2, 2**14, 16, 16, 512, torch.float16),        # batches too small for the record kernels take the walk as well
+        (20000, 3, 2, 2**14, 16, 16, 512, torch.float32),
     ],
 )
 def test_backward_without_records(N, D, F, T, L, lo, hi, do_dtype, monkeypatch):
@@ -469,7 +471,8 @@ def test_backward_without_records(N, D, F, T, L, lo, hi, do_dtype, monkeypatch):
     x = torch.rand(N, D)
     x[:500, 0] = 1.0                                   # the upper edge of the first coordinate
     x[500:1000] = torch.randint(0, hi, (500, D)).float() / hi   # grid nodes of the finest level: weights exactly 0 and 1
-    x[1000:20000] = torch.rand(1, D) * 0.9 + 1e-3 * torch.rand(19000, D)  # a cluster in one cell of the coarse levels
+    k = min(N, 20000)
+    x[1000:k] = torch.rand(1, D) * 0.9 + 1e-3 * torch.rand(k - 1000, D)  # a cluster in one cell of the coarse levels
     E = O.level_row_offsets(L, T, D, lo, hi)[-1]
     do = torch.randn(N, L * F).to(do_dtype)
     want = O.encode_backward(x, do, E, F, None, T, L, lo, hi)
@@ -477,7 +480,7 @@ def test_backward_without_records(N, D, F, T, L, lo, hi, do_dtype, monkeypatch):
     lib = _lib.load()
     need = lib.nf_hash_encode_bwd_workspace_bytes(N, geom, _lib.dtype_code(do_dtype), 0)
     need_records = lib.nf_hash_encode_bwd_workspace_bytes(N, geom, _lib.dtype_code(do_dtype), _lib.NF_HASH_BWD_RECORDS)
-    assert 0 < need < need_records, (need, need_records)
+    assert 0 < need and (need < need_records or need_records == 0), (need, need_records)  # (no records below 32768 points)
     got = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, F, None, T, lo, hi, L).cpu()
     monkeypatch.setattr(hk, "_FLAGS", _lib.NF_HASH_BWD_RECORDS)
     records = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, F, None, T, lo, hi, L).cpu()

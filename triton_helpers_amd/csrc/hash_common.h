@@ -192,6 +192,8 @@ int launch_bwd_scan(const void* coords, int cdt, int64_t csn, int64_t csd, const
 
 // backward by binning the contributions per table stretch (hash_encoding_bwd_bin.hip)
 int64_t bwd_bin_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype, int flags);
+// whether launch_bwd_bin would walk the points without records (small tables; also for batches too small for the records)
+bool bwd_direct_applies(int64_t n_points, const nf_hash_geom* geom, int flags);
 int launch_bwd_bin(const void* coords, int cdt, int64_t csn, int64_t csd, const void* dout, int ddt, int64_t dout_stride,
                    float* dtable, int64_t N, const nf_hash_geom* geom, const DevGeom& g, const int64_t* primes, float scale,
                    void* workspace, int flags, hipStream_t s);

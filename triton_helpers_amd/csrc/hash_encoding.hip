@@ -687,7 +687,8 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
 }
 
 extern "C" int64_t nf_hash_encode_bwd_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype, int flags) {
-  if (geom == nullptr || n_points < SCAN_MIN_POINTS || (flags & (NF_HASH_FORCE_GENERIC | NF_HASH_FORCE_ATOMIC))) return 0;
+  if (geom == nullptr || (flags & (NF_HASH_FORCE_GENERIC | NF_HASH_FORCE_ATOMIC))) return 0;
+  if (n_points < SCAN_MIN_POINTS && ((flags & NF_HASH_FORCE_PLANES) || !bwd_direct_applies(n_points, geom, flags))) return 0;
   const int64_t scan = bwd_scan_workspace_bytes(n_points, geom, dout_dtype);
   if (flags & NF_HASH_FORCE_PLANES) return scan;
   const int64_t bin = bwd_bin_workspace_bytes(n_points, geom, dout_dtype, flags);
@@ -711,13 +712,14 @@ extern "C" int nf_hash_encode_bwd(const void* coords, int coords_dtype, int64_t 
   hipStream_t s = (hipStream_t)stream;
 
   // large batches: accumulate in LDS tiles (needs the caller's workspace for the sorted records or the bit-planes)
-  if (!(flags & (NF_HASH_FORCE_GENERIC | NF_HASH_FORCE_ATOMIC)) && n_points >= SCAN_MIN_POINTS && workspace != nullptr &&
+  if (!(flags & (NF_HASH_FORCE_GENERIC | NF_HASH_FORCE_ATOMIC)) && workspace != nullptr &&
+      (n_points >= SCAN_MIN_POINTS || (!(flags & NF_HASH_FORCE_PLANES) && bwd_direct_applies(n_points, geom, flags))) &&
       ((uintptr_t)dout % (dout_dtype == NF_F32 ? 8 : 4) == 0) && (dout_stride_n % 2 == 0) && ((uintptr_t)workspace % 4 == 0)) {
     const int64_t need_bin = bwd_bin_workspace_bytes(n_points, geom, dout_dtype, flags);
     if (!(flags & NF_HASH_FORCE_PLANES) && need_bin > 0 && workspace_bytes >= need_bin && ((uintptr_t)workspace % 16 == 0))
       return launch_bwd_bin(coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, geom, g, primes,
                             scale, workspace, flags, s);
-    const int64_t need = bwd_scan_workspace_bytes(n_points, geom, dout_dtype);
+    const int64_t need = n_points >= SCAN_MIN_POINTS ? bwd_scan_workspace_bytes(n_points, geom, dout_dtype) : 0;
     if (need > 0 && workspace_bytes >= need)
       return launch_bwd_scan(coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, geom, g,
                              primes, scale, workspace, s);

@@ -1066,13 +1066,16 @@ constexpr int64_t BIN_CHUNK_POINTS = (int64_t)1 << 21;
 // reference's default table size) the walk is the faster one; four bins would already cost it more hashing than the
 // records' passes take.
 constexpr int DIRECT_MAX_BINS_PER_LEVEL = 2;
-constexpr int64_t DIRECT_MIN_POINTS = (int64_t)1 << 17;
+constexpr int64_t DIRECT_MIN_POINTS = 4096;  // below: one launch of scattered atomics is as quick
 static bool direct_ok(int64_t n_points, const nf_hash_geom* geom, int flags) {
   if ((flags & NF_HASH_BWD_RECORDS) || n_points < DIRECT_MIN_POINTS) return false;
   if (geom->dims != 2 && geom->dims != 3) return false;
   for (int l = 0; l < geom->levels; ++l)
     if (geom->rows[l] > (int64_t)DIRECT_MAX_BINS_PER_LEVEL * BIN_ROWS) return false;
   return true;
+}
+bool bwd_direct_applies(int64_t n_points, const nf_hash_geom* geom, int flags) {
+  return direct_ok(n_points < BIN_CHUNK_POINTS ? n_points : BIN_CHUNK_POINTS, geom, flags);
 }
 // gmax[32] (padded to 256 bytes) | pairs[levels][ceil(feat / 2)][n_points] of 4 (float32 gradient: 8) bytes
 static int64_t direct_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype) {
@@ -1160,12 +1163,12 @@ static int launch_bwd_direct(const void* coords, int cdt, int64_t csn, int64_t c
                        g.levels, g.feat, pairs, gmax);
   if (int rc = check_launch("hash_bwd_direct_prep")) return rc;
   // at most two workgroups per compute unit in all, so that they run as two full rounds (one fits at a time: the tile is
-  // 128 KiB of LDS; four rounds: +3 %, eight: +11 %), in slices of whole turns of the point loop and of at least 16384 points
+  // 128 KiB of LDS; four rounds: +3 %, eight: +11 %), in slices of whole turns of the point loop and of at least 4096 points
   const int64_t round = (int64_t)DIRECT_THREADS;
   int64_t slices = (int64_t)2 * direct_cus() / NB;
   if (slices < 1) slices = 1;
   int64_t slice_points = (N + slices - 1) / slices;
-  if (slice_points < 16384) slice_points = 16384;
+  if (slice_points < 4096) slice_points = 4096;
   slice_points = (slice_points + round - 1) / round * round;
   slices = (N + slice_points - 1) / slice_points;
   const size_t lds = (size_t)2 * BIN_ROWS * sizeof(unsigned long long);
