@@ -914,46 +914,48 @@ __global__ __launch_bounds__(DIRECT_THREADS) void hash_bwd_direct_k(const void* 
   const uint32_t* level_pairs = pairs + (((int64_t)l * np + p) * N) * (G32 ? 2 : 1);
   const int64_t n_begin = (int64_t)blockIdx.y * slice_points;
   const int64_t n_end = n_begin + slice_points < N ? n_begin + slice_points : N;
-  // one point per thread and turn: the sixteen waves of the workgroup keep enough loads in flight, and more points per
-  // thread only cost registers (two: +4 %, eight: +70 %)
-  for (int64_t n = n_begin + tid; n < n_end; n += DIRECT_THREADS) {
-    float v[3] = {0.0f, 0.0f, 0.0f};
-    Rec rec = BinRec<GT>::zero();
-    load_point_d<D>(coords, cdt, csn, csd, n, scale, v);
-    if constexpr (G32) {
-      const uint2 t = reinterpret_cast<const uint2*>(level_pairs)[n];
-      rec.z = t.x;
-      rec.w = t.y;
-    } else {
-      rec.z = level_pairs[n];
-    }
-    uint32_t row[1 << D];
-    float w[1 << D];
-    cell_rows<D>(v, fres, hashed, res, mask, pi, primes, row, w);
-    const float g0 = BinRec<GT>::g0(rec) * s_lo * s_hi, g1 = BinRec<GT>::g1(rec) * s_lo * s_hi;
-    if (by_feature) {
+  // One point per thread and turn: the sixteen waves of the workgroup keep enough loads in flight, and more points per
+  // thread only cost registers (two: +4 %, eight: +70 %).  The loop exists in four copies, by the kind of tile and for
+  // levels with an inf or a nan in their gradient (which only mark the rows they touch), so that it carries no branch.
+  auto walk = [&](auto by_feature_c, auto nonfinite_c) {
+    constexpr bool BY_FEATURE = decltype(by_feature_c)::value, NONFINITE = decltype(nonfinite_c)::value;
+    for (int64_t n = n_begin + tid; n < n_end; n += DIRECT_THREADS) {
+      float v[3] = {0.0f, 0.0f, 0.0f};
+      Rec rec = BinRec<GT>::zero();
+      load_point_d<D>(coords, cdt, csn, csd, n, scale, v);
+      if constexpr (G32) {
+        const uint2 t = reinterpret_cast<const uint2*>(level_pairs)[n];
+        rec.z = t.x;
+        rec.w = t.y;
+      } else {
+        rec.z = level_pairs[n];
+      }
+      uint32_t row[1 << D];
+      float w[1 << D];
+      cell_rows<D>(v, fres, hashed, res, mask, pi, primes, row, w);
+      const float g0 = BinRec<GT>::g0(rec) * s_lo * s_hi, g1 = BinRec<GT>::g1(rec) * s_lo * s_hi;
       const float gs = which ? g1 : g0;
 #pragma unroll
       for (int j = 0; j < (1 << D); ++j) {
-        // a level with an inf or a nan in its gradient only marks the rows it touches
-        const int32_t fv = nonfinite ? (int32_t)(w[j] != 0.0f) : __float2int_rn(w[j] * gs);
-        if (fv) atomicAdd(acc_tile + row[j], (unsigned long long)(long long)fv);
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < (1 << D); ++j) {
-        int32_t f0v, f1v;
-        if (nonfinite) {
-          f0v = w[j] != 0.0f;
-          f1v = has_pair && f0v;
+        // zero contributions are rare here: the adds carry no test
+        if constexpr (BY_FEATURE) {
+          const int32_t fv = NONFINITE ? (int32_t)(w[j] != 0.0f) : __float2int_rn(w[j] * gs);
+          atomicAdd(acc_tile + row[j], (unsigned long long)(long long)fv);
         } else {
-          f0v = __float2int_rn(w[j] * g0);
-          f1v = __float2int_rn(w[j] * g1);
+          const int32_t f0v = NONFINITE ? (int32_t)(w[j] != 0.0f) : __float2int_rn(w[j] * g0);
+          const int32_t f1v = NONFINITE ? (int32_t)(has_pair && w[j] != 0.0f) : __float2int_rn(w[j] * g1);
+          atomicAdd(acc_tile + row[j], (unsigned long long)(long long)f0v);
+          atomicAdd(acc_tile + (uint32_t)BIN_ROWS + row[j], (unsigned long long)(long long)f1v);
         }
-        if (f0v) atomicAdd(acc_tile + row[j], (unsigned long long)(long long)f0v);
-        if (f1v) atomicAdd(acc_tile + (uint32_t)BIN_ROWS + row[j], (unsigned long long)(long long)f1v);
       }
     }
+  };
+  if (by_feature) {
+    if (nonfinite) walk(std::true_type{}, std::true_type{});
+    else walk(std::true_type{}, std::false_type{});
+  } else {
+    if (nonfinite) walk(std::false_type{}, std::true_type{});
+    else walk(std::false_type{}, std::false_type{});
   }
   lds_barrier();
   float* dst = dtable + g.row_offset[l] * feat + f0;
