@@ -52,7 +52,6 @@ constexpr uint32_t SLICE_RECORDS = 98304;     // a bin with at most this many re
 constexpr uint32_t SPLIT_RECORDS = 32768;     // a bigger bin is cut into tasks of about this many
 constexpr int MAX_BINS_PER_LEVEL = 2048;        // 2^24 rows
 constexpr int MAX_BINS_TOTAL = 2560;          // LDS of the count and fill kernels
-constexpr int AGG_MAX_BINS = 16;              // levels with at most this many bins rank through wave ballots
 
 struct BinPlan {
   int n_levels;
@@ -206,24 +205,6 @@ __device__ __forceinline__ void load_point_d(const void* coords, int cdt, int64_
   }
 }
 
-// Position of every active lane among the wave's lanes with the same bin, on top of one LDS add per distinct bin.
-__device__ __forceinline__ uint32_t wave_rank(uint32_t* cnt, uint32_t bin, bool active, int lane) {
-  uint32_t rank = 0;
-  unsigned long long todo = __ballot(active);
-  while (todo) {
-    const int leader = __ffsll((long long)todo) - 1;
-    const uint32_t b = (uint32_t)__shfl((int)bin, leader);
-    const bool mine = active && bin == b;
-    const unsigned long long m = __ballot(mine);
-    uint32_t base = 0;
-    if (lane == leader) base = atomicAdd(cnt + b, (uint32_t)__popcll(m));
-    base = (uint32_t)__shfl((int)base, leader);
-    if (mine) rank = base + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
-    todo &= ~m;
-  }
-  return rank;
-}
-
 // Largest value of a wave, valid in lane 63: prefix maxima inside each row of 16 lanes, then lane 15 of rows 0 / 2 into
 // rows 1 / 3 and lane 31 into rows 2 / 3 (data-parallel primitives of the vector ALU; nothing goes through LDS).
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t m) {
@@ -278,10 +259,7 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_count_k(const void* 
         const Located3 q = locate(v, (float)g.res[l]);
         const uint32_t b = q.c[0] + q.c[1] * res + q.c[2] * res * res;
         const uint32_t k0 = b >> BIN_ROWS_LOG2, k1 = (b + res * res + res + 1u) >> BIN_ROWS_LOG2;
-        if (nb <= AGG_MAX_BINS) {
-          wave_rank(cnt, k0, valid, lane);
-          if (__any(valid && k1 != k0)) wave_rank(cnt, k1, valid && k1 != k0, lane);
-        } else if (valid) {
+        if (valid) {
           atomicAdd(cnt + k0, 1u);
           if (k1 != k0) atomicAdd(cnt + k1, 1u);
         }
@@ -293,10 +271,7 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_count_k(const void* 
 #pragma unroll
     for (int c = 0; c < PAIRS; ++c) {
       const uint32_t b0 = row[2 * c] >> BIN_ROWS_LOG2, b1 = row[2 * c + 1] >> BIN_ROWS_LOG2;
-      if (nb <= AGG_MAX_BINS) {
-        wave_rank(cnt, b0, valid, lane);
-        if (__any(valid && b1 != b0)) wave_rank(cnt, b1, valid && b1 != b0, lane);
-      } else if (valid) {
+      if (valid) {
         atomicAdd(cnt + b0, 1u);
         if (b1 != b0) atomicAdd(cnt + b1, 1u);
       }
@@ -506,7 +481,6 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
       const bool two = k1 != k0;
       uint32_t pos0;
       if (nb == 1) pos0 = (uint32_t)tid;  // the valid points are the first of the workgroup
-      else if (nb <= AGG_MAX_BINS) pos0 = wave_rank(lcur, k0, valid, lane);
       else pos0 = valid ? atomicAdd(lcur + k0, 1u) : 0u;
       if (valid) {
         const uint3 rec = make_cell_record((int32_t)(b - (k0 << BIN_ROWS_LOG2)), q.fr, packed);
@@ -514,9 +488,7 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
       }
       if (nb > 1 && __any(valid && two)) {
         const bool on = valid && two;
-        uint32_t pos1;
-        if (nb <= AGG_MAX_BINS) pos1 = wave_rank(lcur, k1, on, lane);
-        else pos1 = on ? atomicAdd(lcur + k1, 1u) : 0u;
+        const uint32_t pos1 = on ? atomicAdd(lcur + k1, 1u) : 0u;
         if (on) {
           const uint3 rec = make_cell_record((int32_t)b - (int32_t)(k1 << BIN_ROWS_LOG2), q.fr, packed);
           stage[pos1] = make_uint4(rec.x, rec.y, rec.z, pos1 + ldelta[k1]);
@@ -541,9 +513,6 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
       if (nb == 1) {
 #pragma unroll
         for (int c = 0; c < PAIRS; ++c) pos[c] = (uint32_t)tid * (uint32_t)PAIRS + (uint32_t)c;  // the valid points are the first of the workgroup
-      } else if (nb <= AGG_MAX_BINS) {
-#pragma unroll
-        for (int c = 0; c < PAIRS; ++c) pos[c] = wave_rank(lcur, b0[c], valid, lane);
       } else {
 #pragma unroll
         for (int c = 0; c < PAIRS; ++c) pos[c] = valid ? atomicAdd(lcur + b0[c], 1u) : 0u;
@@ -564,9 +533,7 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
         for (int c = 0; c < PAIRS; ++c) {
           const bool on = valid && split[c];
           if (!__any(on)) continue;
-          uint32_t pos1;
-          if (nb <= AGG_MAX_BINS) pos1 = wave_rank(lcur, b1[c], on, lane);
-          else pos1 = on ? atomicAdd(lcur + b1[c], 1u) : 0u;
+          const uint32_t pos1 = on ? atomicAdd(lcur + b1[c], 1u) : 0u;
           if (on) {
             const uint32_t r1 = row[2 * c + 1];
             const uint3 rec = make_record(r1 & BIN_MASK, r1 & BIN_MASK, w[2 * c + 1], 0.0f, packed);
