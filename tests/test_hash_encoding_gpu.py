@@ -179,6 +179,45 @@ def test_tiled_and_generic_agree_bitwise(monkeypatch):
     assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,D,T,L,lo,hi", [(1, 3, 2**19, 16, 16, 7006), (257, 3, 2**19, 16, 16, 7006), (5000, 3, 2**17, 2, 16, 700),
+                                            (8191, 2, 2**19, 16, 16, 7006), (60001, 3, 2**19, 16, 16, 7006), (100000, 2, 2**15, 8, 8, 300)])
+def test_small_batches_one_thread_per_point_and_level(N, D, T, L, lo, hi, dtype, monkeypatch):
+    """Batches below the sweep's minimum (forward) and below the sorted-record kernels' minimum (backward) run one
+    thread per (point, level) on 16-bit pairs in two and three dimensions.  Forward: bit-equal to
+    the generic kernel (flag 1) and, where it applies, to the LDS-staged tile kernel (flag 8), and within one ulp of
+    the oracle.  Backward: against the oracle and the generic kernel, a coordinate scale included."""
+    from triton_helpers_amd import _lib
+
+    hk = _hk()
+    torch.manual_seed(8)
+    scale = 2.5
+    x = torch.rand(N, D)
+    x[: N // 8, 0] = 1.0
+    table = _table(T, L, D, lo, hi, 2, dtype=dtype, amp=1.0)
+    E = table.shape[0]
+    xs = (x * scale).to(DEV)
+    outs = {}
+    for flag in (0, _lib.NF_HASH_FORCE_GENERIC, _lib.NF_HASH_FWD_STAGED):
+        monkeypatch.setattr(hk, "_FLAGS", flag)
+        outs[flag] = hk.hash_encoding(xs, table.to(DEV), None, None, T, lo, hi, L, scale=scale)
+    assert torch.equal(outs[0], outs[_lib.NF_HASH_FORCE_GENERIC]) and torch.equal(outs[0], outs[_lib.NF_HASH_FWD_STAGED])
+    want = O.encode_forward(xs.cpu() / scale, table.float(), None, T, L, lo, hi)
+    eps = 2.0**-10 if dtype == torch.float16 else 2.0**-7
+    torch.testing.assert_close(outs[0].cpu().float(), want, rtol=eps, atol=eps * 1e-3)
+
+    do = torch.randn(N, L * 2).to(dtype)
+    do[::7] = 0  # rows of zero gradient are skipped
+    want_g = O.encode_backward(xs.cpu() / scale, do, E, 2, None, T, L, lo, hi)
+    grads = {}
+    for flag in (_lib.NF_HASH_FORCE_ATOMIC, _lib.NF_HASH_FORCE_GENERIC):
+        monkeypatch.setattr(hk, "_FLAGS", flag)
+        grads[flag] = hk.hash_encoding_table_grad(xs, do.to(DEV), E, 2, None, T, lo, hi, L, scale=scale).cpu()
+    peak = float(want_g.abs().max())
+    for got in grads.values():
+        torch.testing.assert_close(got, want_g, rtol=1e-4, atol=1e-5 * peak)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("L,hi", [(16, 7006), (8, 512), (4, 64)])
 def test_forward_kernels_agree_bitwise_at_sweep_sizes(L, hi, dtype, monkeypatch):

@@ -507,13 +507,100 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_bwd_tiled_k(const void* coo
   }
 }
 
+// Small batches: one thread per (point, level), the levels of a point side by side in blockIdx.y.  A thread per point
+// walks its levels one after the other, and a batch of a few thousand points is then a handful of workgroups that wait
+// out sixteen rounds of memory latency (forward) or queue five hundred atomics per thread behind each other (backward)
+// while most of the chip idles.  Same arithmetic, in the same order, as the kernels above.
+template <typename TT, int D>
+__global__ __launch_bounds__(TILE_THREADS) void hash_fwd_level_k(const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                                 const uint32_t* table, uint16_t* out, int64_t out_stride,
+                                                                 int64_t N, DevGeom g, const int64_t* primes, float scale) {
+  const int l = blockIdx.y;
+  const int64_t n = (int64_t)blockIdx.x * TILE_THREADS + threadIdx.x;
+  if (n >= N) return;
+  constexpr int CN = 1 << D;
+  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], D > 2 ? (uint32_t)primes[D > 2 ? 2 : 0] : 0u};
+  const uint32_t res = (uint32_t)g.res[l];
+  const float fres = (float)g.res[l];
+  const uint32_t* tab = table + g.row_offset[l];
+  uint32_t c[3];
+  float fr[3];
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    float v = load_as_f32(coords, n * csn + d * csd, cdt);
+    v = scale != 1.0f ? v / scale : v;
+    const float pos = v * fres;
+    const float fl = floorf(pos);
+    c[d] = cell_index(fl, fres);
+    fr[d] = pos - fl;
+  }
+  const Corner8 r = D == 3 ? rows_d3(c, l >= g.first_hash, res, g.rows[l] - 1, pi) : rows_d2(c, l >= g.first_hash, res, g.rows[l] - 1, pi);
+  uint32_t v[CN];
+#pragma unroll
+  for (int j = 0; j < CN; ++j) v[j] = tab[r.row[j]];
+  float w[8];
+  if (D == 3) weights_d3(fr, w);
+  else weights_d2(fr, w);
+  float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+  for (int j = 0; j < CN; ++j) {
+    a0 = a0 + w[j] * TT::to_f32((uint16_t)(v[j] & 0xffffu));
+    a1 = a1 + w[j] * TT::to_f32((uint16_t)(v[j] >> 16));
+  }
+  *reinterpret_cast<uint32_t*>(out + n * out_stride + 2 * l) = (uint32_t)TT::from_f32(a0) | ((uint32_t)TT::from_f32(a1) << 16);
+}
+
+template <typename GT, int D>
+__global__ __launch_bounds__(TILE_THREADS) void hash_bwd_level_k(const void* coords, int cdt, int64_t csn, int64_t csd,
+                                                                 const uint16_t* dout, int64_t dout_stride, float* dtable,
+                                                                 int64_t N, DevGeom g, const int64_t* primes, float scale) {
+  const int l = blockIdx.y;
+  const int64_t n = (int64_t)blockIdx.x * TILE_THREADS + threadIdx.x;
+  if (n >= N) return;
+  const uint32_t packed = *reinterpret_cast<const uint32_t*>(dout + n * dout_stride + 2 * l);
+  // a zero upstream gradient (both features) contributes nothing
+  if ((packed & 0x7fff7fffu) == 0u) return;
+  constexpr int CN = 1 << D;
+  const float g0 = GT::to_f32((uint16_t)(packed & 0xffffu));
+  const float g1 = GT::to_f32((uint16_t)(packed >> 16));
+  const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], D > 2 ? (uint32_t)primes[D > 2 ? 2 : 0] : 0u};
+  const uint32_t res = (uint32_t)g.res[l];
+  const float fres = (float)g.res[l];
+  float* tab = dtable + g.row_offset[l] * 2;
+  uint32_t c[3];
+  float fr[3];
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    float v = load_as_f32(coords, n * csn + d * csd, cdt);
+    v = scale != 1.0f ? v / scale : v;
+    const float pos = v * fres;
+    const float fl = floorf(pos);
+    c[d] = cell_index(fl, fres);
+    fr[d] = pos - fl;
+  }
+  const Corner8 r = D == 3 ? rows_d3(c, l >= g.first_hash, res, g.rows[l] - 1, pi) : rows_d2(c, l >= g.first_hash, res, g.rows[l] - 1, pi);
+  float w[8];
+  if (D == 3) weights_d3(fr, w);
+  else weights_d2(fr, w);
+#pragma unroll
+  for (int j = 0; j < CN; ++j) {
+    float* dst = tab + 2 * (size_t)r.row[j];
+    unsafeAtomicAdd(dst, w[j] * g0);
+    unsafeAtomicAdd(dst + 1, w[j] * g1);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------
 // below this many points the scattered-atomic kernels are faster than planning + scanning
 constexpr int64_t SCAN_MIN_POINTS = 32768;
+constexpr int64_t BIN_MIN_POINTS = 8192;  // below: the sort's fixed cost (about 100 us) exceeds the scattered atomics' 13 ns per point
 constexpr int SWEEP_PPT = 4;
 constexpr int64_t SWEEP_MIN_POINTS = (int64_t)256 * TILE_THREADS * SWEEP_PPT;
+// the forward per (point, level) serves batches up to this where the staged kernel is the alternative (three
+// dimensions: 45 against 53 us at 2^16 points, 75 against 52 us at 2^17); in two dimensions up to the sweep's minimum
+constexpr int64_t LEVEL_MAX_POINTS = 65536;
 
 static bool tiled_ok(const nf_hash_geom* g, int table_dt, const void* rows_ptr, int64_t row_stride, int feat = 2, int dims = 3) {
   if (g->dims != dims || g->feat != feat || table_dt == NF_F32) return false;
@@ -525,6 +612,18 @@ static bool tiled_ok(const nf_hash_geom* g, int table_dt, const void* rows_ptr, 
   }
   if (((uintptr_t)rows_ptr & 15u) != 0 || (row_stride * 2) % 16 != 0) return false;
   return true;
+}
+
+// the per-(point, level) kernels for small batches: rows of one 16-bit pair, two or three dimensions, hashed levels of
+// a power of two of rows, pairs that can be read and written as one 32-bit word
+static bool level_ok(const nf_hash_geom* g, int table_dt, const void* rows_ptr, int64_t row_stride) {
+  if ((g->dims != 2 && g->dims != 3) || g->feat != 2 || table_dt == NF_F32) return false;
+  for (int l = g->first_hash_level; l < g->levels; ++l) {
+    if (l < 0) return false;
+    const int64_t r = g->rows[l];
+    if ((r & (r - 1)) != 0) return false;
+  }
+  return ((uintptr_t)rows_ptr & 3u) == 0 && row_stride % 2 == 0;
 }
 
 static bool sweep32_ok(const nf_hash_geom* g, const void* table, const void* rows_ptr, int64_t row_stride) {
@@ -657,6 +756,19 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
                          (const uint32_t*)table, (uint16_t*)out, out_stride_n, n_points, g, primes, scale);
     return check_launch("hash_fwd_sweep");
   }
+  // batches below the sweep's minimum: a thread per (point, level)
+  if (!(flags & (NF_HASH_FORCE_GENERIC | NF_HASH_FWD_STAGED)) && level_ok(geom, table_dtype, out, out_stride_n) &&
+      (n_points <= LEVEL_MAX_POINTS || !tiled_ok(geom, table_dtype, out, out_stride_n))) {
+    dim3 grid((unsigned)((n_points + TILE_THREADS - 1) / TILE_THREADS), (unsigned)g.levels);
+    const void* kern = table_dtype == NF_F16 ? (g.dims == 3 ? (const void*)hash_fwd_level_k<F16, 3> : (const void*)hash_fwd_level_k<F16, 2>)
+                                             : (g.dims == 3 ? (const void*)hash_fwd_level_k<BF16, 3> : (const void*)hash_fwd_level_k<BF16, 2>);
+    const uint32_t* tab = (const uint32_t*)table;
+    uint16_t* o = (uint16_t*)out;
+    void* args[] = {&coords, &coords_dtype, &csn, &csd, &tab, &o, &out_stride_n, &n_points, &g, &primes, &scale};
+    const hipError_t e = hipLaunchKernel(kern, grid, dim3(TILE_THREADS), args, 0, s);
+    if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(hash_fwd_level): %s", hipGetErrorString(e));
+    return check_launch("hash_fwd_level");
+  }
   if (!(flags & NF_HASH_FORCE_GENERIC) && tiled_ok(geom, table_dtype, out, out_stride_n)) {
     constexpr int PPT = 2;
     constexpr int P = TILE_THREADS * PPT;
@@ -686,10 +798,16 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
   }
 }
 
+// whether a batch is large enough for one of the backward's LDS-tile variants
+static bool bwd_tiles_apply(int64_t n_points, const nf_hash_geom* geom, int flags) {
+  if (flags & NF_HASH_FORCE_PLANES) return n_points >= SCAN_MIN_POINTS;
+  return n_points >= BIN_MIN_POINTS || bwd_direct_applies(n_points, geom, flags);
+}
+
 extern "C" int64_t nf_hash_encode_bwd_workspace_bytes(int64_t n_points, const nf_hash_geom* geom, int dout_dtype, int flags) {
   if (geom == nullptr || (flags & (NF_HASH_FORCE_GENERIC | NF_HASH_FORCE_ATOMIC))) return 0;
-  if (n_points < SCAN_MIN_POINTS && ((flags & NF_HASH_FORCE_PLANES) || !bwd_direct_applies(n_points, geom, flags))) return 0;
-  const int64_t scan = bwd_scan_workspace_bytes(n_points, geom, dout_dtype);
+  if (!bwd_tiles_apply(n_points, geom, flags)) return 0;
+  const int64_t scan = n_points >= SCAN_MIN_POINTS ? bwd_scan_workspace_bytes(n_points, geom, dout_dtype) : 0;
   if (flags & NF_HASH_FORCE_PLANES) return scan;
   const int64_t bin = bwd_bin_workspace_bytes(n_points, geom, dout_dtype, flags);
   return bin > 0 ? bin : scan;  // the bit-planes are what runs where the other kernels do not cover the geometry
@@ -713,7 +831,7 @@ extern "C" int nf_hash_encode_bwd(const void* coords, int coords_dtype, int64_t 
 
   // large batches: accumulate in LDS tiles (needs the caller's workspace for the sorted records or the bit-planes)
   if (!(flags & (NF_HASH_FORCE_GENERIC | NF_HASH_FORCE_ATOMIC)) && workspace != nullptr &&
-      (n_points >= SCAN_MIN_POINTS || (!(flags & NF_HASH_FORCE_PLANES) && bwd_direct_applies(n_points, geom, flags))) &&
+      bwd_tiles_apply(n_points, geom, flags) &&
       ((uintptr_t)dout % (dout_dtype == NF_F32 ? 8 : 4) == 0) && (dout_stride_n % 2 == 0) && ((uintptr_t)workspace % 4 == 0)) {
     const int64_t need_bin = bwd_bin_workspace_bytes(n_points, geom, dout_dtype, flags);
     if (!(flags & NF_HASH_FORCE_PLANES) && need_bin > 0 && workspace_bytes >= need_bin && ((uintptr_t)workspace % 16 == 0))
@@ -723,6 +841,18 @@ extern "C" int nf_hash_encode_bwd(const void* coords, int coords_dtype, int64_t 
     if (need > 0 && workspace_bytes >= need)
       return launch_bwd_scan(coords, coords_dtype, csn, csd, dout, dout_dtype, dout_stride_n, dtable, n_points, geom, g,
                              primes, scale, workspace, s);
+  }
+  // small batches: a thread per (point, level)
+  if (!(flags & NF_HASH_FORCE_GENERIC) && level_ok(geom, dout_dtype, dout, dout_stride_n) &&
+      (n_points < BIN_MIN_POINTS || !tiled_ok(geom, dout_dtype, dout, dout_stride_n))) {
+    dim3 grid((unsigned)((n_points + TILE_THREADS - 1) / TILE_THREADS), (unsigned)g.levels);
+    const void* kern = dout_dtype == NF_F16 ? (g.dims == 3 ? (const void*)hash_bwd_level_k<F16, 3> : (const void*)hash_bwd_level_k<F16, 2>)
+                                            : (g.dims == 3 ? (const void*)hash_bwd_level_k<BF16, 3> : (const void*)hash_bwd_level_k<BF16, 2>);
+    const uint16_t* d = (const uint16_t*)dout;
+    void* args[] = {&coords, &coords_dtype, &csn, &csd, &d, &dout_stride_n, &dtable, &n_points, &g, &primes, &scale};
+    const hipError_t e = hipLaunchKernel(kern, grid, dim3(TILE_THREADS), args, 0, s);
+    if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(hash_bwd_level): %s", hipGetErrorString(e));
+    return check_launch("hash_bwd_level");
   }
   if (!(flags & NF_HASH_FORCE_GENERIC) && tiled_ok(geom, dout_dtype, dout, dout_stride_n)) {
     constexpr int PPT = 2;
