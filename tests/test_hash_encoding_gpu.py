@@ -308,7 +308,7 @@ def test_forward_config0_full_size():
 @pytest.mark.parametrize("N,D,F,T,L,lo,hi,scale", CASES + [(65536, 3, 2, 2**20, 16, 16, 512, 1.0), (131072, 3, 2, 2**14, 16, 16, 512, 1.0)])
 @pytest.mark.parametrize("do_dtype,flags", [(torch.float32, 1), (torch.float32, 0), (torch.float16, 0), (torch.float16, 1), (torch.float16, 2)])
 def test_backward_vs_oracle(N, D, F, T, L, lo, hi, scale, do_dtype, flags, monkeypatch):
-    """flags: 0 = default dispatch (LDS-tile kernels from 32768 points), 1 = generic, 2 = scattered atomics."""
+    """flags: 0 = default dispatch (LDS-tile kernels from 8192 points), 1 = generic, 2 = scattered atomics."""
     hk = _hk()
     monkeypatch.setattr(hk, "_FLAGS", flags)
     torch.manual_seed(0)
@@ -519,7 +519,7 @@ def test_backward_without_records(N, D, F, T, L, lo, hi, do_dtype, monkeypatch):
     lib = _lib.load()
     need = lib.nf_hash_encode_bwd_workspace_bytes(N, geom, _lib.dtype_code(do_dtype), 0)
     need_records = lib.nf_hash_encode_bwd_workspace_bytes(N, geom, _lib.dtype_code(do_dtype), _lib.NF_HASH_BWD_RECORDS)
-    assert 0 < need and (need < need_records or need_records == 0), (need, need_records)  # (no records below 32768 points)
+    assert 0 < need and (need < need_records or need_records == 0), (need, need_records)  # (no records below 8192 points)
     got = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, F, None, T, lo, hi, L).cpu()
     monkeypatch.setattr(hk, "_FLAGS", _lib.NF_HASH_BWD_RECORDS)
     records = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, F, None, T, lo, hi, L).cpu()
