@@ -179,6 +179,35 @@ def test_tiled_and_generic_agree_bitwise(monkeypatch):
     assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("D,F,dtype,off", [(3, 4, torch.float32, 0), (3, 8, torch.float32, 0), (3, 6, torch.float32, 0), (2, 6, torch.float16, 0),
+                                            (4, 2, torch.bfloat16, 0), (1, 2, torch.float32, 0), (3, 24, torch.float16, 0), (3, 4, torch.float32, 2),
+                                            (3, 8, torch.float16, 4), (3, 3, torch.float16, 0)])
+def test_generic_forward_reads_rows_in_pieces(D, F, dtype, off, monkeypatch):
+    """The per-(point, level) forward reads a row in pieces of up to 16 bytes where the row width and the alignment of
+    table and output allow it (float32 rows of 4 features: one load per corner instead of four).  Bit-equal to the
+    one-feature-at-a-time form (flag 1); `off` elements of misalignment of table and output make it fall back to
+    narrower pieces; 1.0e6 points on the float32 four-feature case keep the many-workgroup path covered elsewhere."""
+    from triton_helpers_amd import _lib
+
+    hk = _hk()
+    torch.manual_seed(9)
+    N, T, L, lo, hi = 3001, 2**12, 4, 4, 40
+    pi = torch.tensor([1, 2654435761, 805459861, 3674653429], dtype=torch.int64)
+    x = torch.rand(N, D)
+    E = O.level_row_offsets(L, T, D, lo, hi)[-1]
+    store = torch.zeros(E * F + 8, dtype=dtype, device=DEV)
+    table = store[off : off + E * F].view(E, F)
+    table.copy_((torch.rand(E, F) * 2 - 1).to(dtype))
+    outs = {}
+    for flag in (0, _lib.NF_HASH_FORCE_GENERIC):
+        monkeypatch.setattr(hk, "_FLAGS", flag)
+        outs[flag] = hk.hash_encoding(x.to(DEV), table, None, pi.to(DEV), T, lo, hi, L)
+    assert torch.equal(outs[0], outs[_lib.NF_HASH_FORCE_GENERIC])
+    want = O.encode_forward(x, table.float().cpu(), pi, T, L, lo, hi)
+    rtol, atol = (1e-5, 1e-6) if dtype == torch.float32 else ((2.0**-10, 1e-4) if dtype == torch.float16 else (2.0**-7, 1e-3))
+    torch.testing.assert_close(outs[0].cpu().float(), want, rtol=rtol, atol=atol)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("N,D,T,L,lo,hi", [(1, 3, 2**19, 16, 16, 7006), (257, 3, 2**19, 16, 16, 7006), (5000, 3, 2**17, 2, 16, 700),
                                             (8191, 2, 2**19, 16, 16, 7006), (60001, 3, 2**19, 16, 16, 7006), (100000, 2, 2**15, 8, 8, 300)])

@@ -34,11 +34,14 @@ __device__ __forceinline__ void load_primes(const int64_t* primes, uint64_t* pi)
   for (int d = 0; d < D; ++d) pi[d] = (uint64_t)primes[d];
 }
 
-template <int D, typename TT>
+// V = features per load: rows whose width, base and output allow it are read V features (4, 8 or 16 bytes) at a time,
+// every feature summed over the corners in the same order as with V = 1
+template <int D, typename TT, int V = 1>
 __global__ __launch_bounds__(256) void hash_fwd_generic_k(const void* coords, int cdt, int64_t csn, int64_t csd,
                                                           const typename TT::storage* table,
                                                           typename TT::storage* out, int64_t out_stride, int64_t N,
                                                           DevGeom g, const int64_t* primes, float scale) {
+  typedef typename TT::storage S;
   const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int l = blockIdx.y;
   if (n >= N) return;
@@ -46,7 +49,7 @@ __global__ __launch_bounds__(256) void hash_fwd_generic_k(const void* coords, in
   load_primes<D>(primes, pi);
   const bool hashed = l >= g.first_hash;
   const Cell<D> cell = locate<D>(coords, cdt, csn, csd, n, scale, g.res[l]);
-  const typename TT::storage* tab = table + g.row_offset[l] * g.feat;
+  const S* tab = table + g.row_offset[l] * g.feat;
   uint64_t rows[1 << D];
   float w[1 << D];
 #pragma unroll
@@ -54,11 +57,31 @@ __global__ __launch_bounds__(256) void hash_fwd_generic_k(const void* coords, in
     rows[j] = corner_row<D>(cell, j, hashed, (uint32_t)g.res[l], g.rows[l], pi);
     w[j] = corner_weight<D>(cell, j);
   }
-  for (int f = 0; f < g.feat; ++f) {
-    float acc = 0.0f;
+  if constexpr (V == 1) {
+    for (int f = 0; f < g.feat; ++f) {
+      float acc = 0.0f;
 #pragma unroll
-    for (int j = 0; j < (1 << D); ++j) acc = acc + w[j] * TT::to_f32(tab[rows[j] * g.feat + f]);
-    out[n * out_stride + (int64_t)l * g.feat + f] = TT::from_f32(acc);
+      for (int j = 0; j < (1 << D); ++j) acc = acc + w[j] * TT::to_f32(tab[rows[j] * g.feat + f]);
+      out[n * out_stride + (int64_t)l * g.feat + f] = TT::from_f32(acc);
+    }
+  } else {
+    struct alignas(V * sizeof(S)) Piece { S v[V]; };
+    for (int f = 0; f < g.feat; f += V) {
+      float acc[V];
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] = 0.0f;
+      Piece q[1 << D];
+#pragma unroll
+      for (int j = 0; j < (1 << D); ++j) q[j] = *reinterpret_cast<const Piece*>(tab + rows[j] * g.feat + f);
+#pragma unroll
+      for (int j = 0; j < (1 << D); ++j)
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc[e] = acc[e] + w[j] * TT::to_f32(q[j].v[e]);
+      Piece r;
+#pragma unroll
+      for (int e = 0; e < V; ++e) r.v[e] = TT::from_f32(acc[e]);
+      *reinterpret_cast<Piece*>(out + n * out_stride + (int64_t)l * g.feat + f) = r;
+    }
   }
 }
 
@@ -638,21 +661,42 @@ static bool sweep32_ok(const nf_hash_geom* g, const void* table, const void* row
 
 template <int D, typename TT>
 static void launch_fwd_generic(const void* coords, int cdt, int64_t csn, int64_t csd, const void* table, void* out,
-                               int64_t out_stride, int64_t N, const DevGeom& g, const int64_t* primes, float scale,
+                               int64_t out_stride, int64_t N, const DevGeom& g, const int64_t* primes, float scale, bool vec,
                                hipStream_t s) {
+  typedef typename TT::storage S;
   dim3 grid((unsigned)((N + 255) / 256), (unsigned)g.levels);
-  hipLaunchKernelGGL((hash_fwd_generic_k<D, TT>), grid, dim3(256), 0, s, coords, cdt, csn, csd,
-                     (const typename TT::storage*)table, (typename TT::storage*)out, out_stride, N, g, primes, scale);
+  // the widest piece of 16, 8 or 4 bytes that divides a row and keeps every row of the table and of the output aligned
+  int v = 1;
+  if (vec && D <= 4)
+    for (int bytes = 16; bytes > (int)sizeof(S); bytes >>= 1) {
+      const int c = bytes / (int)sizeof(S);
+      if (g.feat % c == 0 && out_stride % c == 0 && (uintptr_t)table % bytes == 0 && (uintptr_t)out % bytes == 0) {
+        v = c;
+        break;
+      }
+    }
+  const void* kern = (const void*)hash_fwd_generic_k<D, TT, 1>;
+  if constexpr (D <= 4) {
+    if (v == 2) kern = (const void*)hash_fwd_generic_k<D, TT, 2>;
+    if (v == 4) kern = (const void*)hash_fwd_generic_k<D, TT, 4>;
+    if constexpr (sizeof(S) == 2)
+      if (v == 8) kern = (const void*)hash_fwd_generic_k<D, TT, 8>;
+  }
+  const S* tab = (const S*)table;
+  S* o = (S*)out;
+  DevGeom gg = g;
+  void* args[] = {&coords, &cdt, &csn, &csd, &tab, &o, &out_stride, &N, &gg, &primes, &scale};
+  (void)hipLaunchKernel(kern, grid, dim3(256), args, 0, s);  // the caller reads the launch status
 }
 
 template <int D>
 static int dispatch_fwd_generic(int table_dt, const void* coords, int cdt, int64_t csn, int64_t csd, const void* table,
                                 void* out, int64_t out_stride, int64_t N, const DevGeom& g, const int64_t* primes,
-                                float scale, hipStream_t s) {
+                                float scale, bool vec, hipStream_t s) {
   switch (table_dt) {
-    case NF_F32: launch_fwd_generic<D, F32>(coords, cdt, csn, csd, table, out, out_stride, N, g, primes, scale, s); break;
-    case NF_F16: launch_fwd_generic<D, F16>(coords, cdt, csn, csd, table, out, out_stride, N, g, primes, scale, s); break;
-    default: launch_fwd_generic<D, BF16>(coords, cdt, csn, csd, table, out, out_stride, N, g, primes, scale, s); break;
+    case NF_F32: launch_fwd_generic<D, F32>(coords, cdt, csn, csd, table, out, out_stride, N, g, primes, scale, vec, s); break;
+    case NF_F16: launch_fwd_generic<D, F16>(coords, cdt, csn, csd, table, out, out_stride, N, g, primes, scale, vec, s); break;
+    default: launch_fwd_generic<D, BF16>(coords, cdt, csn, csd, table, out, out_stride, N, g, primes, scale, vec, s); break;
   }
   return check_launch("hash_fwd_generic");
 }
@@ -788,13 +832,14 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
     return geom->feat == 4 ? launch_fwd_tiled_wide<2>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s)
                            : launch_fwd_tiled_wide<4>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
   }
+  const bool vec = !(flags & NF_HASH_FORCE_GENERIC);  // the flag keeps the scalar form as the other kernels' bit-exact check
   switch (g.dims) {
-    case 1: return dispatch_fwd_generic<1>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
-    case 2: return dispatch_fwd_generic<2>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
-    case 3: return dispatch_fwd_generic<3>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
-    case 4: return dispatch_fwd_generic<4>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
-    case 5: return dispatch_fwd_generic<5>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
-    default: return dispatch_fwd_generic<6>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, s);
+    case 1: return dispatch_fwd_generic<1>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, vec, s);
+    case 2: return dispatch_fwd_generic<2>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, vec, s);
+    case 3: return dispatch_fwd_generic<3>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, vec, s);
+    case 4: return dispatch_fwd_generic<4>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, vec, s);
+    case 5: return dispatch_fwd_generic<5>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, vec, s);
+    default: return dispatch_fwd_generic<6>(table_dtype, coords, coords_dtype, csn, csd, table, out, out_stride_n, n_points, g, primes, scale, vec, s);
   }
 }
 

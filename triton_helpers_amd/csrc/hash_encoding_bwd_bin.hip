@@ -396,11 +396,29 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
   const float* grow32 = reinterpret_cast<const float*>(dout_v) + (valid ? n : 0) * dout_stride;
   uint32_t gr[16];
   // this pass covers features f0, f0 + 1 of every level: the pair of level l sits at element l * feat + f0 of the row
-  const bool row_vec = !G32 && feat == 2 && bp.n_levels <= 16 && (bp.n_levels & 3) == 0 && ((uintptr_t)dout & 15u) == 0 && (dout_stride & 7) == 0;
+  // (rows of 2, 4 or 8 features in 16-byte pieces: with 4 or 8 features a piece holds the pairs of two levels or of one,
+  // and the pass keeps its own; per-level 4-byte reads touch a point's 128 or 256 bytes sixteen times instead)
+  const bool row_vec = !G32 && (feat == 2 || feat == 4 || feat == 8) && bp.n_levels <= 16 && (bp.n_levels & 3) == 0 &&
+                       ((uintptr_t)dout & 15u) == 0 && (dout_stride & 7) == 0;
+  const bool row_vec32 = G32 && feat == 2 && (bp.n_levels & 3) == 0 && ((uintptr_t)dout_v & 15u) == 0 && (dout_stride & 3) == 0;
+  uint2 held[3] = {make_uint2(0u, 0u), make_uint2(0u, 0u), make_uint2(0u, 0u)};
+  const int pair_in_level = f0 >> 1;
+  auto word = [](const uint4& q, int c) { return c == 0 ? q.x : c == 1 ? q.y : c == 2 ? q.z : q.w; };
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     uint4 t = make_uint4(0u, 0u, 0u, 0u);
-    if (row_vec && valid && 4 * i < bp.n_levels) t = reinterpret_cast<const uint4*>(grow)[i];
+    if (row_vec && valid && 4 * i < bp.n_levels) {
+      const uint4* g4 = reinterpret_cast<const uint4*>(grow);
+      if (feat == 2) {
+        t = g4[i];
+      } else if (feat == 4) {
+        const uint4 a = g4[2 * i], b = g4[2 * i + 1];
+        t = pair_in_level ? make_uint4(a.y, a.w, b.y, b.w) : make_uint4(a.x, a.z, b.x, b.z);
+      } else {
+        const uint4 q0 = g4[4 * i], q1 = g4[4 * i + 1], q2 = g4[4 * i + 2], q3 = g4[4 * i + 3];
+        t = make_uint4(word(q0, pair_in_level), word(q1, pair_in_level), word(q2, pair_in_level), word(q3, pair_in_level));
+      }
+    }
     gr[4 * i] = t.x;
     gr[4 * i + 1] = t.y;
     gr[4 * i + 2] = t.z;
@@ -442,6 +460,16 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
         if (feat & 1) {  // an odd row width: the pair is not 8-byte aligned, and the last feature has no partner
           pair.x = __float_as_uint(grow32[l * feat + f0]);
           if (f0 + 1 < feat) pair.y = __float_as_uint(grow32[l * feat + f0 + 1]);
+        } else if (row_vec32) {  // four levels' pairs in two 16-byte reads: a quarter of the passes over the point's 128 bytes
+          if ((l & 3) == 0) {
+            const uint4 q0 = *reinterpret_cast<const uint4*>(grow32 + 2 * l), q1 = *reinterpret_cast<const uint4*>(grow32 + 2 * l + 4);
+            pair = make_uint2(q0.x, q0.y);
+            held[0] = make_uint2(q0.z, q0.w);
+            held[1] = make_uint2(q1.x, q1.y);
+            held[2] = make_uint2(q1.z, q1.w);
+          } else {
+            pair = (l & 3) == 1 ? held[0] : (l & 3) == 2 ? held[1] : held[2];
+          }
         } else {
           pair = *reinterpret_cast<const uint2*>(grow32 + l * feat + f0);
         }
