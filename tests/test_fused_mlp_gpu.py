@@ -80,6 +80,10 @@ SHAPES = [
     ((1, 4099), 64, 64, 16, 2),
     ((2, 1000), 32, 64, 64, 2),
     ((1, 200), 48, 64, 40, 2),
+    # one hidden layer of width 64: the ReLU backward runs the two-layer kernels behind an identity layer
+    ((1, 1000), 32, 64, 16, 1),
+    ((1, 4099), 64, 64, 64, 1),
+    ((2, 77), 27, 64, 3, 1),
     # two or three hidden-to-hidden layers of width 64: ReLU takes the register-resident backward for deeper nets
     ((1, 1000), 32, 64, 16, 4),
     ((1, 1000), 32, 64, 16, 3),
@@ -431,7 +435,7 @@ def test_module_autocast(depth):
 
 
 @pytest.mark.parametrize("x_dtype,w_dtype", [(torch.float16, torch.bfloat16), (torch.bfloat16, torch.float16)])
-@pytest.mark.parametrize("depth,bias", [(2, True), (2, False), (3, True)])
+@pytest.mark.parametrize("depth,bias", [(2, True), (2, False), (3, True), (1, True)])
 def test_input_in_the_other_16bit_dtype(x_dtype, w_dtype, depth, bias):
     """x stored in the other 16-bit dtype than the parameters (an fp16 encoder output in front of bf16 weights): the
     result is bit-identical to casting x first, y comes in the parameters' dtype and dx in x's."""

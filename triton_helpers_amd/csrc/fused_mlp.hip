@@ -728,6 +728,44 @@ static void set_rows(MlpArgs& g, const uint16_t* x, int64_t x_stride, uint16_t* 
   g.dx_vec = dx ? vec_store_ok(dx, dx_stride, g.d_in) : 0;
 }
 
+// ---------------------------------------------------------------------------------------
+// One hidden layer (depth 1, d_in -> 64 -> d_out, ReLU) on the backward kernels built for two.
+// Behind a ReLU every hidden value is >= 0, so an identity layer with a ReLU of its own between the hidden layer and the
+// output changes nothing: h2 = relu(I h1) = h1 bit for bit (one non-zero term per float32 sum, a value that is already
+// a 16-bit number), the gradient crosses the identity unchanged, meets the same gate and rounds to the 16-bit number it
+// already is.  The extra 64 x 64 products cost a third of the two-layer kernel's work, which is still several times
+// quicker than the general kernel; the identity's own weight gradient goes to a sink nobody reads.
+// The identity (one per 16-bit type) and the sink are file-scope device arrays; the identity is written by a tiny kernel on
+// the caller's stream in front of every such backward (no cross-stream ordering to rely on, same values every time), and
+// concurrent calls share the sink, whose contents mean nothing.
+// ---------------------------------------------------------------------------------------
+static __device__ __align__(256) uint16_t identity_hidden[2][64 * 64];  // [bfloat16, float16]
+static __device__ __align__(256) float identity_sink[64 * 64 + 64];     // dW (float32, or 16-bit rounded) and db of the identity
+
+__global__ __launch_bounds__(256) void identity_fill_k(uint16_t* w) {
+  const int i = blockIdx.x * 256 + threadIdx.x;  // 2 x 4096 elements
+  const int e = i & 4095;
+  w[i] = (e >> 6) == (e & 63) ? (i < 4096 ? (uint16_t)0x3F80u : (uint16_t)0x3C00u) : (uint16_t)0u;
+}
+
+static bool identity_layer_applies(int d_hidden, int depth, int act, int dtype) {
+  return depth == 1 && d_hidden == 64 && act == NF_ACT_RELU && (dtype == NF_BF16 || dtype == NF_F16);
+}
+
+// the identity in `dtype` and the sink, on the current device; the fill is queued on `s`
+static int identity_layer(int dtype, hipStream_t s, const uint16_t** w, float** sink) {
+  uint16_t* base = nullptr;
+  float* sk = nullptr;
+  hipError_t e = hipGetSymbolAddress((void**)&base, HIP_SYMBOL(identity_hidden));
+  if (e == hipSuccess) e = hipGetSymbolAddress((void**)&sk, HIP_SYMBOL(identity_sink));
+  if (e != hipSuccess) return fail((int)e, "hipGetSymbolAddress(identity layer): %s", hipGetErrorString(e));
+  hipLaunchKernelGGL(identity_fill_k, dim3(2 * 4096 / 256), dim3(256), 0, s, base);
+  if (int rc = check_launch("identity_fill")) return rc;
+  *w = base + (dtype == NF_BF16 ? 0 : 4096);
+  *sink = sk;
+  return 0;
+}
+
 }  // namespace nf
 
 using namespace nf;
@@ -810,6 +848,12 @@ extern "C" int nf_mlp_bwd(const void* x, int64_t x_stride, const void* dy, int64
   a.x_conv = x_dtype == dtype ? 0 : (x_dtype == NF_F16 ? 1 : 2);
   set_rows(a, (const uint16_t*)x, x_stride, nullptr, 0, (const uint16_t*)dy, dy_stride, (uint16_t*)dx, dx_stride);
   hipStream_t s = (hipStream_t)stream;
+  if (identity_layer_applies(d_hidden, depth, act, dtype)) {
+    float* sink = nullptr;
+    if (int rc = identity_layer(dtype, s, &a.w_hid, &sink)) return rc;
+    a.b_hid = nullptr; a.dw_hid = sink; a.db_hid = nullptr; a.depth = 2;
+    return bwd_one(a, dtype, s);
+  }
   const std::vector<int> first = plan_launches(depth + 1, bwd_max_linear(d_hidden, act));
   const int n = (int)first.size() - 1;
   if (n == 1) return bwd_one(a, dtype, s);
@@ -867,7 +911,8 @@ extern "C" int nf_mlp_bwd_rounded(const void* x, int64_t x_stride, const void* d
   NF_REQUIRE(dtype != NF_F32 && (x_dtype == NF_F16 || x_dtype == NF_BF16), NF_EUNSUPPORTED,
              "rounded weight gradients: 16-bit tensors only (dtype code %d, x_dtype code %d)", dtype, x_dtype);
   NF_REQUIRE(rows > 0, NF_EUNSUPPORTED, "rounded weight gradients: no rows (the buffers would stay unwritten)");
-  NF_REQUIRE(x && dy && w_in && w_hid && w_out && dw_in && dw_hid && dw_out, NF_EINVAL, "NULL pointer argument");
+  const bool identity = identity_layer_applies(d_hidden, depth, act, dtype);  // one hidden layer: see identity_layer()
+  NF_REQUIRE(x && dy && w_in && w_out && dw_in && dw_out && (identity || (w_hid && dw_hid)), NF_EINVAL, "NULL pointer argument");
   NF_REQUIRE(x_stride >= d_in && dy_stride >= d_out && (dx == nullptr || dx_stride >= d_in), NF_EINVAL,
              "row stride smaller than row width");
   const int64_t need = nf_mlp_bwd_rounded_workspace_bytes(d_in, d_hidden, d_out);
@@ -881,6 +926,12 @@ extern "C" int nf_mlp_bwd_rounded(const void* x, int64_t x_stride, const void* d
   a.in_act = NF_ACT_NONE;
   a.x_conv = x_dtype == dtype ? 0 : (x_dtype == NF_F16 ? 1 : 2);
   set_rows(a, (const uint16_t*)x, x_stride, nullptr, 0, (const uint16_t*)dy, dy_stride, (uint16_t*)dx, dx_stride);
+  if (identity) {
+    float* sink = nullptr;
+    if (int rc = identity_layer(dtype, (hipStream_t)stream, &a.w_hid, &sink)) return rc;
+    a.b_hid = nullptr; a.depth = 2;
+    dw_hid = nullptr; db_hid = nullptr;  // the sum over the slots leaves out pieces without a destination
+  }
   void* const out[6] = {dw_in, db_in, dw_hid, db_hid, dw_out, db_out};
   bool handled = false;
   const int rc = launch_mlp_bwd2_w8_rounded(a, dtype, out, workspace, (hipStream_t)stream, &handled);

@@ -226,15 +226,17 @@ class _fully_fused_mlp(Function):
             x, w_in, b_in, w_out, b_out, w_hid, b_hid = (_half(t) for t in (x, w_in, b_in, w_out, b_out, w_hid, b_hid))
         if do.dtype != w_in.dtype:
             do = do.to(w_in.dtype)
-        if x.dtype != w_in.dtype and not (w_in.dtype != torch.float32 and ctx.depth == 2 and D_hidden > 32 and ctx.activation == "relu"):
-            x = x.to(w_in.dtype)  # only the one-hidden-layer ReLU backward converts on the fly
+        converts = (ctx.depth == 2 and D_hidden > 32) or (ctx.depth == 1 and D_hidden == 64)
+        if x.dtype != w_in.dtype and not (w_in.dtype != torch.float32 and converts and ctx.activation == "relu"):
+            x = x.to(w_in.dtype)  # only the ReLU backward of one or two 64-wide hidden layers converts on the fly
         do2 = _rows2d(do, D_out)
         need_dx = ctx.needs_input_grad[0]
         decoder = D_in <= 32 and D_out <= 16  # the wider shapes need x in the parameters' dtype
-        if (not wide and w_in.dtype != torch.float32 and ctx.depth == 2 and D_hidden == 64 and D_in <= 64 and D_out <= 64
+        # (one hidden layer runs on the same kernels behind an identity layer that the library supplies)
+        if (not wide and w_in.dtype != torch.float32 and ctx.depth in (1, 2) and D_hidden == 64 and D_in <= 64 and D_out <= 64
                 and (decoder or x.dtype == w_in.dtype)
                 and D_in % 4 == 0 and D_out % 4 == 0 and ctx.activation == "relu" and do2.shape[0] > 0):
-            done = _backward_rounded(x, do2, w_in, b_in, w_out, b_out, w_hid, b_hid, need_dx, D_in, D_hidden, D_out)
+            done = _backward_rounded(x, do2, w_in, b_in, w_out, b_out, w_hid, b_hid, need_dx, D_in, D_hidden, D_out, ctx.depth)
             if done is not None:
                 return done
         grads = _lib.GradBuffers(w_in, b_in, w_out, b_out, w_hid, b_hid)
@@ -284,7 +286,7 @@ def _rounded_plan(lib, like, D_in, D_hidden, D_out):
     return plan
 
 
-def _backward_rounded(x, do2, w_in, b_in, w_out, b_out, w_hid, b_hid, need_dx, D_in, D_hidden, D_out):
+def _backward_rounded(x, do2, w_in, b_in, w_out, b_out, w_hid, b_hid, need_dx, D_in, D_hidden, D_out, depth=2):
     """Backward of the one-hidden-layer ReLU shapes through ``nf_mlp_bwd_rounded``: the weight gradients come back summed
     in a fixed order and rounded to the parameters' dtype, into one uninitialised buffer (no clearing, no cast kernel).
     ``None`` when the library declines (rows not 8-byte aligned): the caller takes the general path.  The buffer is
@@ -302,7 +304,7 @@ def _backward_rounded(x, do2, w_in, b_in, w_out, b_out, w_hid, b_hid, need_dx, D
         x2.data_ptr(), x2.stride(0), do2.data_ptr(), do2.stride(0), _lib.ptr(dx), D_in,
         w_in.data_ptr(), _lib.ptr(b_in), _lib.ptr(w_hid), _lib.ptr(b_hid), w_out.data_ptr(), _lib.ptr(b_out),
         p[0], p[1], p[4], p[5], p[2], p[3],
-        x2.shape[0], D_in, D_hidden, D_out, 2, _lib.NF_ACT["relu"], _lib.dtype_code(w_in.dtype), _lib.dtype_code(x.dtype),
+        x2.shape[0], D_in, D_hidden, D_out, depth, _lib.NF_ACT["relu"], _lib.dtype_code(w_in.dtype), _lib.dtype_code(x.dtype),
         ws.data_ptr(), ws_bytes, _lib.current_stream(x.device),
     )
     if rc == _lib.NF_EUNSUPPORTED:
