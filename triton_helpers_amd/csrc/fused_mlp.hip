@@ -504,18 +504,24 @@ __global__ __launch_bounds__(256) void mlp_bwd_k(MlpArgs a) {
   }
 }
 
-// db_out = column sums of dy; tiny and memory-bound, done apart from the fused kernel.
+// db_out = column sums of dy; tiny and memory-bound, done apart from the fused kernel.  The 256 threads of a workgroup
+// cover 256 / cols rows at a time, cols = d_out rounded up to a power of two (a one-column dy keeps every lane busy).
 template <typename T>
-__global__ __launch_bounds__(256) void db_out_k(const uint16_t* dy, int64_t stride, int64_t rows, int d_out, float* db_out) {
+__global__ __launch_bounds__(256) void db_out_k(const uint16_t* dy, int64_t stride, int64_t rows, int d_out, int cols_log2, float* db_out) {
   __shared__ float part[256];
-  const int c = threadIdx.x % 64;  // column handled (d_out <= 64)
-  const int rl = threadIdx.x / 64;
+  const int cols = 1 << cols_log2, rows_per_turn = 256 >> cols_log2;
+  const int c = threadIdx.x & (cols - 1), rl = threadIdx.x >> cols_log2;
   float s = 0.0f;
   if (c < d_out)
-    for (int64_t r = (int64_t)blockIdx.x * 4 + rl; r < rows; r += (int64_t)gridDim.x * 4) s += T::to_f32(dy[r * stride + c]);
+    for (int64_t r = (int64_t)blockIdx.x * rows_per_turn + rl; r < rows; r += (int64_t)gridDim.x * rows_per_turn)
+      s += T::to_f32(dy[r * stride + c]);
   part[threadIdx.x] = s;
   __syncthreads();
-  if (rl == 0 && c < d_out) unsafeAtomicAdd(db_out + c, part[c] + part[64 + c] + part[128 + c] + part[192 + c]);
+  for (int h = 128; h >= cols; h >>= 1) {  // thread t and t + h hold the same column
+    if ((int)threadIdx.x < h) part[threadIdx.x] += part[threadIdx.x + h];
+    __syncthreads();
+  }
+  if ((int)threadIdx.x < d_out) unsafeAtomicAdd(db_out + threadIdx.x, part[threadIdx.x]);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -593,7 +599,9 @@ static int launch_bwd(const MlpArgs& a0, hipStream_t s) {
   if (a.db_out != nullptr) {
     int64_t b = (a.rows + 1023) / 1024;
     if (b > 1024) b = 1024;
-    hipLaunchKernelGGL((db_out_k<T>), dim3((unsigned)b), dim3(256), 0, s, a.dy, a.dy_stride, a.rows, a.d_out, a.db_out);
+    int cols_log2 = 0;
+    while ((1 << cols_log2) < a.d_out) ++cols_log2;
+    hipLaunchKernelGGL((db_out_k<T>), dim3((unsigned)b), dim3(256), 0, s, a.dy, a.dy_stride, a.rows, a.d_out, cols_log2, a.db_out);
     return check_launch("db_out");
   }
   return 0;
