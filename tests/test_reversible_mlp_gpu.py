@@ -126,6 +126,36 @@ def test_unchecked_and_checked_kernels_agree(rows, H, blocks, act, dtype):
             torch.testing.assert_close(a.float(), b.float(), rtol=1e-2, atol=1e-2 * scale)
 
 
+@pytest.mark.parametrize("act", ["gelu", "relu", "silu"])
+@pytest.mark.parametrize("rows,H,blocks", [(4096 + 17, 64, 4), (8192 + 31, 32, 2), (5000, 64, 1)])
+def test_large_ragged_batch_runs_as_main_part_plus_tail(rows, H, blocks, act):
+    """From 4096 rows a batch whose row count is not a multiple of 32 runs as two calls: the multiple of 32 (the kernels
+    without per-tile checks where the rest allows) and the last rows.  Rows are independent, so y and dx equal, bit for
+    bit, what the two parts give when the caller splits them, and the weight gradients are the sum of the parts'."""
+    rk = _rk()
+    dtype = torch.bfloat16
+    torch.manual_seed(3)
+    w1, b1, w2, b2 = (t.to(DEV) for t in _params(blocks, H, True, dtype))
+    x = torch.randn(rows, 2 * H, device=DEV).to(dtype)
+    dy = torch.randn(rows, 2 * H, device=DEV).to(dtype)
+
+    def run(xs, dys):
+        leaves = [t.clone().requires_grad_(True) for t in (w1, b1, w2, b2)]
+        xv = xs.clone().requires_grad_(True)
+        y = rk.reversible_mlp(xv, *leaves, act)
+        y.backward(dys)
+        return y.detach(), xv.grad, [t.grad.float() for t in leaves]
+
+    m = rows - rows % 32
+    y, dx, g = run(x, dy)
+    y0, dx0, g0 = run(x[:m], dy[:m])
+    y1, dx1, g1 = run(x[m:], dy[m:])
+    assert torch.equal(y, torch.cat([y0, y1])) and torch.equal(dx, torch.cat([dx0, dx1]))
+    for a, b0, b1_ in zip(g, g0, g1):
+        want = b0 + b1_
+        torch.testing.assert_close(a, want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("rows,H,blocks", [(1000, 64, 4), (1024, 64, 4), (512, 32, 3)])
 def test_relu_forward(rows, H, blocks, dtype):

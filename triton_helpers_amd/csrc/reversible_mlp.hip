@@ -654,6 +654,8 @@ static int rev_validate(int64_t rows, int half, int blocks, int act, int dtype) 
   return 0;
 }
 
+constexpr int64_t SPLIT_MIN_ROWS = 4096;  // from here on a ragged end is worth a launch of its own
+
 static bool vec8_ok(const void* p, int64_t stride, int half) {
   return ((uintptr_t)p % 8 == 0) && (stride % 4 == 0) && (half % 4 == 0);
 }
@@ -725,6 +727,14 @@ extern "C" int nf_revmlp_fwd(const void* x, int64_t x_stride, void* y, int64_t y
   if (rows == 0) return 0;
   NF_REQUIRE(x && y && w1 && w2, NF_EINVAL, "NULL pointer argument");
   NF_REQUIRE(x_stride >= 2 * half && y_stride >= 2 * half, NF_EINVAL, "row stride smaller than 2*half");
+  // Rows are independent: a large batch with a ragged end runs as its multiple of 32 rows (the variants without per-tile
+  // checks, where the rest of the call allows them) plus a call of its own for the last rows.
+  if (rows >= SPLIT_MIN_ROWS && rows % 32 != 0) {
+    const int64_t main_rows = rows - rows % 32;
+    if (int rc = nf_revmlp_fwd(x, x_stride, y, y_stride, w1, b1, w2, b2, main_rows, half, blocks, act, dtype, stream)) return rc;
+    return nf_revmlp_fwd((const uint16_t*)x + main_rows * x_stride, x_stride, (uint16_t*)y + main_rows * y_stride, y_stride, w1, b1, w2, b2,
+                         rows - main_rows, half, blocks, act, dtype, stream);
+  }
   hipStream_t s = (hipStream_t)stream;
   const int es = 2;
   for (int k0 = 0; k0 < blocks; k0 += FWD_GROUP) {
@@ -765,6 +775,16 @@ extern "C" int nf_revmlp_bwd(const void* y, int64_t y_stride, const void* dy, in
              "NULL pointer argument (x_rec is required: it carries the reconstructed input between blocks)");
   NF_REQUIRE(y_stride >= 2 * half && dy_stride >= 2 * half && dx_stride >= 2 * half && x_rec_stride >= 2 * half, NF_EINVAL,
              "row stride smaller than 2*half");
+  // a ragged end as a call of its own (see nf_revmlp_fwd): both calls add into the same weight-gradient accumulators
+  if (rows >= SPLIT_MIN_ROWS && rows % 32 != 0) {
+    const int64_t m = rows - rows % 32;
+    if (int rc = nf_revmlp_bwd(y, y_stride, dy, dy_stride, dx, dx_stride, x_rec, x_rec_stride, w1, b1, w2, b2, dw1, db1, dw2, db2, m, half,
+                               blocks, act, dtype, stream))
+      return rc;
+    return nf_revmlp_bwd((const uint16_t*)y + m * y_stride, y_stride, (const uint16_t*)dy + m * dy_stride, dy_stride,
+                         (uint16_t*)dx + m * dx_stride, dx_stride, (uint16_t*)x_rec + m * x_rec_stride, x_rec_stride, w1, b1, w2, b2, dw1, db1,
+                         dw2, db2, rows - m, half, blocks, act, dtype, stream);
+  }
   hipStream_t s = (hipStream_t)stream;
   // Full-width, aligned, unragged calls of the two common activations take one launch that walks all couplings, last
   // first (the first reads (y, dy), the others continue in place on (x_rec, dx)); anything else one launch per coupling.
