@@ -678,6 +678,32 @@ def test_features_are_appended_and_ignored_in_backward():
     torch.testing.assert_close(e.grad.cpu().float(), wantg, rtol=2e-3, atol=2e-3)
 
 
+@pytest.mark.parametrize("dtype,n_feat", [(torch.float16, 3), (torch.float32, 3), (torch.float16, 4), (torch.bfloat16, 1)])
+def test_appended_features_off_16_byte_rows_at_large_batches(dtype, n_feat):
+    """Three appended features (view directions) leave output and gradient rows off 16-byte boundaries.  From 4096
+    points the encoding is then written to a packed buffer and concatenated, and the backward packs the encoding's
+    gradient columns first, so both directions keep the fast kernels: same values as the call without features, bit for
+    bit in the forward, and the table gradient against the oracle."""
+    hk = _hk()
+    g = GOLDEN["bench"]
+    T, L, lo, hi = g["T"], 16, 16, 7006
+    N = 20000 + 3
+    torch.manual_seed(4)
+    x = torch.rand(2, N, 3, device=DEV)                     # leading batch dimensions as in the reference's shapes
+    feats = torch.randn(2, N, n_feat, device=DEV).to(dtype)
+    table = _table(T, L, 3, lo, hi, dtype=dtype, amp=1.0).to(DEV)
+    e = table.clone().requires_grad_(True)
+    o = hk.hash_encoding(x, e, feats, None, T, lo, hi, L)
+    plain = hk.hash_encoding(x, table, None, None, T, lo, hi, L)
+    assert o.shape == (2, N, 32 + n_feat) and o.dtype == dtype
+    assert torch.equal(o[..., :32], plain) and torch.equal(o[..., 32:], feats)
+    do = torch.randn(2, N, 32 + n_feat, device=DEV).to(dtype)
+    o.backward(do)
+    want = O.encode_backward(x.reshape(-1, 3).cpu(), do.reshape(-1, 32 + n_feat)[:, :32].cpu(), table.shape[0], 2, None, T, L, lo, hi)
+    tol = 2e-3 if dtype != torch.float32 else 1e-4
+    torch.testing.assert_close(e.grad.cpu().float(), want, rtol=max(tol, 2.0**-8 if dtype == torch.bfloat16 else 0), atol=tol * float(want.abs().max()))
+
+
 def test_module_autocast():
     # reference test_hash_encoding.py:507-530
     from triton_helpers_amd.layers.hash_encoding import HashEncoding

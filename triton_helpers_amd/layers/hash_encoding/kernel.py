@@ -44,6 +44,7 @@ PI_3: Final = 805_459_861
 DIVIDER_CONFIGS: Dict[Any, int] = {}
 BWD_DIVIDER_CONFIGS: Dict[Any, int] = {}
 
+_REPACK_MIN_POINTS = 4096  # batches from which misaligned output / gradient rows go through a packed buffer
 _FLAGS = 0  # test hook: _lib.NF_HASH_FORCE_GENERIC / NF_HASH_FORCE_ATOMIC / NF_HASH_FORCE_PLANES select other kernels
 
 
@@ -132,6 +133,10 @@ def hash_encoding_table_grad(
     assert de.dtype == torch.float32 and de.is_contiguous() and de.shape == (num_embeddings, d_embed)
     coords2d = _flat_coords(coords)
     do2d = _as_rows(do, do.shape[-1])
+    if do2d.shape[0] >= _REPACK_MIN_POINTS and ((do2d.stride(0) * do2d.element_size()) % 16 != 0 or do2d.data_ptr() % 16 != 0):
+        # gradient rows off 16-byte boundaries (the output carried appended features): the LDS-tile kernels read whole
+        # aligned rows, so the encoding's columns are packed first (one pass instead of scattered atomics per corner)
+        do2d = do2d[:, : levels * d_embed].contiguous()
     _launch_backward(coords2d, do2d, de, pi, max_entries_per_level, min_res, max_res, levels, scale)
     return de
 
@@ -198,15 +203,22 @@ class HashEncoding(torch.autograd.Function):
             pi = pi.to(torch.int64)
 
         D_out = D_embed * levels + D_feature
-        o = embeddings.new_empty(*coords.shape[:-1], D_out)
         table = embeddings.detach()
         if not table.is_contiguous():
             table = table.contiguous()
         coords2d = _flat_coords(coords.detach())
-        _launch_forward(coords2d, table, pi, o.view(-1, D_out), max_entries_per_level, min_res, max_res, levels, scale)
-
-        if features is not None:
-            o[..., D_embed * levels :] = features
+        if features is not None and coords2d.shape[0] >= _REPACK_MIN_POINTS and (D_out * embeddings.element_size()) % 16 != 0:
+            # appended features that leave the output rows off 16-byte boundaries (three view-direction components, say):
+            # the fast kernels write whole aligned rows, so the encoding goes to a buffer of its own and one
+            # concatenation builds the output (a pass over the output instead of the per-(point, level) kernel)
+            enc = embeddings.new_empty(*coords.shape[:-1], D_embed * levels)
+            _launch_forward(coords2d, table, pi, enc.view(-1, D_embed * levels), max_entries_per_level, min_res, max_res, levels, scale)
+            o = torch.cat([enc, features.to(enc.dtype)], dim=-1)
+        else:
+            o = embeddings.new_empty(*coords.shape[:-1], D_out)
+            _launch_forward(coords2d, table, pi, o.view(-1, D_out), max_entries_per_level, min_res, max_res, levels, scale)
+            if features is not None:
+                o[..., D_embed * levels :] = features
 
         ctx.save_for_backward(coords, embeddings, pi)
         ctx.max_entries_per_level = max_entries_per_level
