@@ -186,8 +186,10 @@ int64_t nf_mlp_workspace_bytes(int64_t rows, int d_hidden, int depth, int act, i
 
 /* x_dtype may be the other 16-bit type than `dtype` (an fp16 encoder output feeding bf16 weights): the rows are
  * converted while they are loaded, as a cast kernel in front would, and the backward writes dx in x_dtype.
- * nf_mlp_bwd takes a differing x_dtype for depth == 2, d_hidden > 32, ReLU and 8-byte aligned rows only
- * (NF_EUNSUPPORTED otherwise).
+ * nf_mlp_bwd takes a differing x_dtype for depth == 2, d_hidden > 32 (or depth == 1, d_hidden == 64), ReLU and 8-byte
+ * aligned rows only (NF_EUNSUPPORTED otherwise).
+ * depth == 1 (no hidden-to-hidden layer; w_hid, b_hid, dw_hid, db_hid NULL) with d_hidden == 64 and ReLU runs the
+ * kernels of depth == 2 behind an identity layer that the library keeps on the device: after a ReLU, relu(I h) == h.
  *
  * Backward.  dx [rows, d_in] in x_dtype; the dw_ and db_ arguments are float32 accumulators shaped like the
  * weights/biases, NOT cleared by the call (db_* may be NULL; dx may be NULL). */
@@ -201,9 +203,9 @@ int nf_mlp_bwd(const void* x, int64_t x_stride, const void* dy, int64_t dy_strid
  * `dtype`, and is WRITTEN with the sum over all rows, rounded once -- nothing to clear before the call and nothing to
  * cast after it (the reference's host-side sum(0) of per-program partials in the storage dtype,
  * triton_helpers/layers/fully_fused_mlp/kernel.py:627-633, in one place).  The workgroups' partial sums are added in a
- * fixed order, so the same inputs give the same bits on every run.  Built for the decoder shape -- depth == 2,
- * d_hidden == 64, d_in <= 32, d_out <= 16 (both multiples of 4), ReLU, 8-byte aligned rows -- and NF_EUNSUPPORTED
- * otherwise, before anything is launched.  workspace: 16-byte aligned, nf_mlp_bwd_rounded_workspace_bytes() bytes. */
+ * fixed order, so the same inputs give the same bits on every run.  Built for depth == 2 (or depth == 1 with w_hid
+ * and dw_hid NULL), d_hidden == 64, d_in <= 64, d_out <= 64 (both multiples of 4), ReLU, 8-byte aligned rows, and beyond
+ * d_in 32 / d_out 16 x stored in `dtype`; NF_EUNSUPPORTED otherwise, before anything is launched.  workspace: 16-byte aligned, nf_mlp_bwd_rounded_workspace_bytes() bytes. */
 int nf_mlp_bwd_rounded(const void* x, int64_t x_stride, const void* dy, int64_t dy_stride, void* dx, int64_t dx_stride,
                        const void* w_in, const void* b_in, const void* w_hid, const void* b_hid, const void* w_out,
                        const void* b_out, void* dw_in, void* db_in, void* dw_hid, void* db_hid, void* dw_out,
