@@ -98,7 +98,7 @@ def _offset_8_bytes(t):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("act", ["gelu", "relu"])
+@pytest.mark.parametrize("act", ["gelu", "relu", "silu"])
 @pytest.mark.parametrize("rows,H,blocks", [(4096, 64, 4), (1024, 32, 2), (288, 64, 5)])
 def test_unchecked_and_checked_kernels_agree(rows, H, blocks, act, dtype):
     """Aligned unragged calls run the kernels without per-tile checks (the backward as one launch over all

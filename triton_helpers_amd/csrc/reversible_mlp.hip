@@ -671,12 +671,13 @@ static int launch_rev_fwd(RevArgs a, hipStream_t s) {
   int64_t blocks = (chunks + waves - 1) / waves;
   const int64_t cap = (int64_t)rev_cus() * (lds > 80 * 1024 ? 1 : 2);
   if (blocks > cap) blocks = cap;
-  // full-width, aligned, unragged calls of the two common activations take the variants without per-tile checks
+  // full-width, aligned, unragged calls of GELU, ReLU and SiLU take the variants without per-tile checks
   const bool fast = a.half == HP && a.rows % 32 == 0 && a.vec_in && a.vec_out;
   const void* kern = a.act == NF_ACT_GELU   ? (fast ? (const void*)rev_fwd_k<T, HP, NF_ACT_GELU, true>
                                                     : (const void*)rev_fwd_k<T, HP, NF_ACT_GELU, false>)
                      : a.act == NF_ACT_RELU ? (fast ? (const void*)rev_fwd_k<T, HP, NF_ACT_RELU, true>
                                                     : (const void*)rev_fwd_k<T, HP, NF_ACT_RELU, false>)
+                     : (a.act == NF_ACT_SILU && fast) ? (const void*)rev_fwd_k<T, HP, NF_ACT_SILU, true>
                                             : (const void*)rev_fwd_k<T, HP, -1, false>;
   if (lds > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -705,6 +706,7 @@ static int launch_rev_bwd(RevArgs a, hipStream_t s) {
                                                     : (const void*)rev_bwd_block_k<T, HP, NF_ACT_GELU, false>)
                      : a.act == NF_ACT_RELU ? (fast ? (const void*)rev_bwd_block_k<T, HP, NF_ACT_RELU, true>
                                                     : (const void*)rev_bwd_block_k<T, HP, NF_ACT_RELU, false>)
+                     : (a.act == NF_ACT_SILU && fast) ? (const void*)rev_bwd_block_k<T, HP, NF_ACT_SILU, true>
                                             : (const void*)rev_bwd_block_k<T, HP, -1, false>;
   if (lds > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -786,10 +788,10 @@ extern "C" int nf_revmlp_bwd(const void* y, int64_t y_stride, const void* dy, in
                          dw2, db2, rows - m, half, blocks, act, dtype, stream);
   }
   hipStream_t s = (hipStream_t)stream;
-  // Full-width, aligned, unragged calls of the two common activations take one launch that walks all couplings, last
+  // Full-width, aligned, unragged calls of GELU, ReLU and SiLU take one launch that walks all couplings, last
   // first (the first reads (y, dy), the others continue in place on (x_rec, dx)); anything else one launch per coupling.
   const int hp = half <= 32 ? 32 : 64;
-  const bool fused = half == hp && rows % 32 == 0 && (act == NF_ACT_GELU || act == NF_ACT_RELU) && vec8_ok(y, y_stride, half) &&
+  const bool fused = half == hp && rows % 32 == 0 && (act == NF_ACT_GELU || act == NF_ACT_RELU || act == NF_ACT_SILU) && vec8_ok(y, y_stride, half) &&
                      vec8_ok(x_rec, x_rec_stride, half) && vec8_ok(dy, dy_stride, half) && vec8_ok(dx, dx_stride, half) &&
                      vec16_ok(y, y_stride) && vec16_ok(x_rec, x_rec_stride) && vec16_ok(dy, dy_stride) && vec16_ok(dx, dx_stride);
   for (int k = blocks - 1; k >= 0; --k) {
