@@ -559,6 +559,56 @@ def test_backward_without_records(N, D, F, T, L, lo, hi, do_dtype, monkeypatch):
     assert float(got[~touched].abs().max()) == 0.0 if bool((~touched).any()) else True
 
 
+@pytest.mark.parametrize(
+    "N,D,F,T,L,lo,hi,do_dtype",
+    [
+        (30000, 1, 2, 2**12, 8, 16, 16000, torch.float16),   # dense and hashed 1-D levels
+        (9000, 4, 2, 2**13, 4, 2, 24, torch.float16),        # 4-D: 16 corners per cell
+        (12000, 4, 4, 5000, 2, 3, 9, torch.float32),         # a table size that is not a power of two, two feature pairs
+        (5000, 4, 1, 2**14, 8, 2, 40, torch.bfloat16),
+        # larger 4-D tables: the sorted-record kernels, once per corner of the fourth coordinate
+        (9000, 4, 2, 2**17, 4, 4, 40, torch.float16),        # dense levels of several bins and hashed ones
+        (40000, 4, 2, 2**19, 8, 2, 64, torch.float16),
+        (12000, 4, 4, 50000, 2, 3, 30, torch.float32),       # a size that is not a power of two: exact 64-bit remainder
+        (20000, 4, 3, 2**16, 2, 8, 20, torch.bfloat16),
+        (9000, 5, 2, 2**16, 2, 2, 8, torch.float16),         # five and six dimensions: four and eight passes
+        (8500, 6, 2, 2**15, 2, 2, 5, torch.float32),
+    ],
+)
+def test_backward_without_records_in_one_and_four_dimensions(N, D, F, T, L, lo, hi, do_dtype, monkeypatch):
+    """Small tables walk the points without records in one to four dimensions; other tables in four to six dimensions
+    run the 3-D record kernels once per corner of the extra coordinates (their term joins the hash, the dense index and
+    the weights).  The alternative is scattered atomics (2^20 points: 18 ms in 1-D, 38 ms in 4-D).  Against the oracle
+    and against the atomic kernels (flag NF_HASH_FORCE_ATOMIC)."""
+    from triton_helpers_amd import _lib
+
+    hk = _hk()
+    torch.manual_seed(12)
+    pi = torch.tensor([1, 2654435761, 805459861, 3674653429, 2097192037, 1434869437], dtype=torch.int64)
+    x = torch.rand(N, D).clamp(max=0.999999)
+    x[:300] = (torch.randint(0, hi, (300, D)).float() / hi).clamp(max=0.999999)   # grid nodes: weights exactly 0 and 1
+    x[300:3000] = (torch.rand(1, D) * 0.9 + 1e-3 * torch.rand(2700, D)).clamp(max=0.999999)  # a cluster
+    x[3000] = 0.0
+    E = O.level_row_offsets(L, T, D, lo, hi)[-1]
+    do = torch.randn(N, L * F).to(do_dtype)
+    want = O.encode_backward(x, do, E, F, pi[:D], T, L, lo, hi)
+    geom = hk.level_geometry(T, L, D, F, lo, hi)
+    lib = _lib.load()
+    assert lib.nf_hash_encode_bwd_workspace_bytes(N, geom, _lib.dtype_code(do_dtype), 0) > 0
+    if D == 1:
+        assert lib.nf_hash_encode_bwd_workspace_bytes(N, geom, _lib.dtype_code(do_dtype), _lib.NF_HASH_BWD_RECORDS) == 0
+    got = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, F, pi[:D].to(DEV), T, lo, hi, L).cpu()
+    monkeypatch.setattr(hk, "_FLAGS", _lib.NF_HASH_FORCE_ATOMIC)
+    atomic = hk.hash_encoding_table_grad(x.to(DEV), do.to(DEV), E, F, pi[:D].to(DEV), T, lo, hi, L).cpu()
+    peak = float(want.abs().max())
+    records = max(O.level_row_counts(L, T, D, lo, hi)) > 2 * 8192   # more than two bins on some level: sorted records
+    torch.testing.assert_close(got, want, rtol=1e-3, atol=(1e-4 if records else 1e-5) * peak)
+    torch.testing.assert_close(atomic, want, rtol=1e-3, atol=1e-4 * peak)
+    touched = O.encode_backward(x, torch.ones_like(do, dtype=torch.float32), E, F, pi[:D], T, L, lo, hi) != 0
+    if bool((~touched).any()):
+        assert float(got[~touched].abs().max()) == 0.0
+
+
 def test_backward_without_records_nonfinite_gradient():
     """An inf in the upstream gradient of one level: that level's touched rows come out NaN, as from the record kernels,
     and every other level is unaffected."""

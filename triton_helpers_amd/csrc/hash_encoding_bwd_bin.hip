@@ -99,7 +99,8 @@ struct Located3 {
   uint32_t c[3];
   float fr[3];
 };
-__device__ __forceinline__ Located3 locate(const float (&v)[3], float fres) {
+template <int VD>
+__device__ __forceinline__ Located3 locate(const float (&v)[VD], float fres) {
   Located3 r;
 #pragma unroll
   for (int d = 0; d < 3; ++d) {
@@ -119,14 +120,61 @@ __device__ __forceinline__ void load_point(const void* coords, int cdt, int64_t 
   }
 }
 
+// Dimensions beyond the third (sorted-record kernels, 4-D to 6-D points): a 4-D cell is its 3-D cell twice, once per
+// corner of the fourth coordinate, so the 3-D pipeline runs once per such corner (`hi`, one bit per extra dimension).  The
+// extra coordinates enter a pass as one term of the hash (xor), one of the dense index (add) and one factor of the weights.
+struct ExtraDims {
+  uint32_t hx;     // xor term of the 32-bit hash (hashed levels of a power of two of rows)
+  uint64_t hx64;   // the same in 64 bits (hashed levels of any other size)
+  uint32_t add;    // term of the dense index
+  float w;         // factor of every corner weight
+};
+template <int DX, int VD>
+__device__ __forceinline__ ExtraDims extra_dims(const float (&v)[VD], float fres, uint32_t res, int hi, const int64_t* primes) {
+  static_assert(VD >= 3 + DX, "coordinate array too short");
+  ExtraDims e = {0u, 0ull, 0u, 1.0f};
+  uint32_t stride = res * res * res;
+#pragma unroll
+  for (int d = 0; d < DX; ++d) {
+    const float pos = v[3 + d] * fres;
+    const float fl = floorf(pos);
+    const uint32_t bit = (uint32_t)(hi >> d) & 1u;
+    const uint32_t c = cell_index(fl, fres) + bit;
+    const float fr = pos - fl;
+    e.hx ^= c * (uint32_t)primes[3 + d];
+    e.hx64 ^= (uint64_t)c * (uint64_t)primes[3 + d];
+    e.add += c * stride;
+    stride *= res;
+    const float wd = bit ? fr : 1.0f - fr;
+    e.w = d == 0 ? wd : e.w * wd;
+  }
+  return e;
+}
+
 // Table rows (and trilinear / bilinear weights) of the 2^D corners of a point's cell, corner j = bit pattern of its
 // offsets with x in bit 0, so that corners 2c and 2c+1 are an x-pair.  D = 3 or 2.
 // A hashed level whose size is not a power of two takes the exact remainder of the 64-bit hash (the reference's
 // CPU form) instead of the 32-bit wrap-around and mask.
-template <int D>
-__device__ __forceinline__ void cell_rows(const float (&v)[3], float fres, bool hashed, uint32_t res, uint32_t mask,
-                                          const uint32_t (&pi)[3], const int64_t* primes, uint32_t (&row)[1 << D], float* w) {
+template <int D, int VD>
+__device__ __forceinline__ void cell_rows(const float (&v)[VD], float fres, bool hashed, uint32_t res, uint32_t mask,
+                                          const uint32_t (&pi)[3], const int64_t* primes, uint32_t (&row)[1 << D], float* w,
+                                          const ExtraDims* ex = nullptr) {
   const uint32_t n_rows = mask + 1u;
+  if constexpr (D != 2 && D != 3) {
+    // one, or more than three dimensions (the walk without records only): the per-(point, level) kernels' exact forms
+    static_assert(VD >= D, "coordinate array too short");
+    uint64_t p64[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) p64[d] = (uint64_t)primes[d];
+    const Cell<D> cell = locate_cell<D>(v, (int)res);
+#pragma unroll
+    for (int j = 0; j < (1 << D); ++j) {
+      const uint32_t r = (uint32_t)corner_row<D>(cell, j, hashed, res, n_rows, p64);
+      row[j] = r < n_rows ? r : mask;  // (every row is inside its level; the tile that takes it is sized by the level)
+      if (w != nullptr) w[j] = corner_weight<D>(cell, j);
+    }
+    return;
+  } else {
   if (hashed && (n_rows & mask) != 0u) {
     uint32_t c[D];
     float fr[3] = {0.0f, 0.0f, 0.0f};
@@ -142,11 +190,15 @@ __device__ __forceinline__ void cell_rows(const float (&v)[3], float fres, bool 
       uint64_t h = 0;
 #pragma unroll
       for (int d = 0; d < D; ++d) h ^= (uint64_t)(c[d] + ((j >> d) & 1)) * (uint64_t)primes[d];
+      if (ex != nullptr) h ^= ex->hx64;
       row[j] = (uint32_t)(h % (uint64_t)n_rows);
     }
     if (w != nullptr) {
       if (D == 3) {
         weights_d3(fr, w);
+        if (ex != nullptr)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) w[j] = w[j] * ex->w;
       } else {
         const float gx = 1.0f - fr[0], gy = 1.0f - fr[1];
         w[0] = gx * gy;
@@ -163,6 +215,15 @@ __device__ __forceinline__ void cell_rows(const float (&v)[3], float fres, bool 
 #pragma unroll
     for (int j = 0; j < (1 << D); ++j) row[j] = r.row[j];
     if (w != nullptr) weights_d3(q.fr, w);
+    if (ex != nullptr) {
+      // (a & m) ^ (b & m) == (a ^ b) & m: the extra xor term joins the masked rows; dense rows take the extra index term
+      const uint32_t hx = ex->hx & mask;
+#pragma unroll
+      for (int j = 0; j < (1 << D); ++j) row[j] = hashed ? (row[j] ^ hx) : row[j] + ex->add;
+      if (w != nullptr)
+#pragma unroll
+        for (int j = 0; j < (1 << D); ++j) w[j] = w[j] * ex->w;
+    }
   } else {
     uint32_t c[2];
     float fr[2];
@@ -194,10 +255,11 @@ __device__ __forceinline__ void cell_rows(const float (&v)[3], float fres, bool 
       w[3] = fr[0] * fr[1];
     }
   }
+  }
 }
-template <int D>
+template <int D, int VD>
 __device__ __forceinline__ void load_point_d(const void* coords, int cdt, int64_t csn, int64_t csd, int64_t n, float scale,
-                                             float (&v)[3]) {
+                                             float (&v)[VD]) {
 #pragma unroll
   for (int d = 0; d < D; ++d) {
     v[d] = load_as_f32(coords, n * csn + d * csd, cdt);
@@ -226,10 +288,11 @@ __global__ void hash_bwd_bin_zero_k(uint32_t* p, int n) {
 // ---------------------------------------------------------------------------------------
 // count
 // ---------------------------------------------------------------------------------------
-template <int D>
+// DX: dimensions beyond the third (D == 3 then); hi: which corner of them this pass covers
+template <int D, int DX = 0>
 __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_count_k(const void* coords, int cdt, int64_t csn, int64_t csd,
                                                                     int64_t N, DevGeom g, BinPlan bp, const int64_t* primes,
-                                                                    float scale, uint32_t* hist, uint32_t* wg_counts) {
+                                                                    float scale, uint32_t* hist, uint32_t* wg_counts, int hi) {
   extern __shared__ uint32_t lh[];  // all bins of all levels
   const int tid = threadIdx.x, lane = tid & 63;
   const int NB = bp.binbase[bp.n_levels];
@@ -237,9 +300,9 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_count_k(const void* 
   lds_barrier();
   const int64_t n = (int64_t)blockIdx.x * FILL_POINTS + tid;
   const bool valid = n < N;
-  float v[3] = {0.0f, 0.0f, 0.0f};
+  float v[3 + DX] = {};
   constexpr int PAIRS = 1 << (D - 1);
-  if (valid) load_point_d<D>(coords, cdt, csn, csd, n, scale, v);
+  if (valid) load_point_d<D + DX>(coords, cdt, csn, csd, n, scale, v);
   const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], D > 2 ? (uint32_t)primes[D > 2 ? 2 : 0] : 0u};
   for (int l = 0; l < bp.n_levels; ++l) {
     uint32_t* cnt = lh + bp.binbase[l];
@@ -267,7 +330,12 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_count_k(const void* 
       }
     }
     uint32_t row[1 << D];
-    cell_rows<D>(v, (float)g.res[l], l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi, primes, row, nullptr);
+    if constexpr (DX > 0) {
+      const ExtraDims ex = extra_dims<DX>(v, (float)g.res[l], (uint32_t)g.res[l], hi, primes);
+      cell_rows<D>(v, (float)g.res[l], l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi, primes, row, nullptr, &ex);
+    } else {
+      cell_rows<D>(v, (float)g.res[l], l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi, primes, row, nullptr);
+    }
 #pragma unroll
     for (int c = 0; c < PAIRS; ++c) {
       const uint32_t b0 = row[2 * c] >> BIN_ROWS_LOG2, b1 = row[2 * c + 1] >> BIN_ROWS_LOG2;
@@ -358,12 +426,12 @@ __global__ __launch_bounds__(1024) void hash_bwd_bin_offsets_k(const uint32_t* h
 // G32 = false: 16-bit upstream gradient, 12-byte records {.., .., packed pair}.  G32 = true: float32 upstream gradient,
 // 16-byte records {.., .., g0, g1}; a staged entry then names the point instead of carrying the pair, and the copy-out
 // takes the pair from the workgroup's per-level gradient table in LDS (the stage has no room for 20-byte entries).
-template <bool G32, int D>
+template <bool G32, int D, int DX = 0>
 __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* coords, int cdt, int64_t csn, int64_t csd,
                                                                    const void* dout_v, int64_t dout_stride, int64_t N,
                                                                    DevGeom g, BinPlan bp, const int64_t* primes, float scale,
                                                                    const uint32_t* wg_counts, uint32_t* cursor, uint32_t* gmax,
-                                                                   uint32_t* records_v, int feat, int f0) {
+                                                                   uint32_t* records_v, int feat, int f0, int hi) {
   extern __shared__ __align__(16) unsigned char fill_smem[];
   const int NB = bp.binbase[bp.n_levels];
   const uint16_t* dout = reinterpret_cast<const uint16_t*>(dout_v);
@@ -387,9 +455,9 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
     delta[i] = c ? atomicAdd(cursor + i, c) : 0u;
   }
   if (tid < NF_MAX_LEVELS) lmax[tid] = 0u;
-  float v[3] = {0.0f, 0.0f, 0.0f};
+  float v[3 + DX] = {};
   constexpr int PAIRS = 1 << (D - 1);
-  if (valid) load_point_d<D>(coords, cdt, csn, csd, n, scale, v);
+  if (valid) load_point_d<D + DX>(coords, cdt, csn, csd, n, scale, v);
   const uint32_t pi[3] = {(uint32_t)primes[0], (uint32_t)primes[1], D > 2 ? (uint32_t)primes[D > 2 ? 2 : 0] : 0u};
   // this point's gradient row, read once (up to 16 levels live in registers); float32 rows are read level by level
   const uint32_t* grow = reinterpret_cast<const uint32_t*>(dout + (valid ? n : 0) * dout_stride);
@@ -525,7 +593,12 @@ __global__ __launch_bounds__(FILL_POINTS) void hash_bwd_bin_fill_k(const void* c
     } else {
       uint32_t row[1 << D];
       float w[1 << D];
-      cell_rows<D>(v, (float)g.res[l], l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi, primes, row, w);
+      if constexpr (DX > 0) {
+        const ExtraDims ex = extra_dims<DX>(v, (float)g.res[l], (uint32_t)g.res[l], hi, primes);
+        cell_rows<D>(v, (float)g.res[l], l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi, primes, row, w, &ex);
+      } else {
+        cell_rows<D>(v, (float)g.res[l], l >= g.first_hash, (uint32_t)g.res[l], g.rows[l] - 1u, pi, primes, row, w);
+      }
       // The x-pairs of the point (four in 3-D, two in 2-D): their ranks are asked for together, so that a wave waits
       // for LDS once per level and not once per pair.
       uint32_t b0[PAIRS], b1[PAIRS], pos[PAIRS], dlt[PAIRS];
@@ -915,7 +988,7 @@ __global__ __launch_bounds__(DIRECT_THREADS) void hash_bwd_direct_k(const void* 
   auto walk = [&](auto by_feature_c, auto nonfinite_c) {
     constexpr bool BY_FEATURE = decltype(by_feature_c)::value, NONFINITE = decltype(nonfinite_c)::value;
     for (int64_t n = n_begin + tid; n < n_end; n += DIRECT_THREADS) {
-      float v[3] = {0.0f, 0.0f, 0.0f};
+      float v[D > 3 ? D : 3] = {};
       Rec rec = BinRec<GT>::zero();
       load_point_d<D>(coords, cdt, csn, csd, n, scale, v);
       if constexpr (G32) {
@@ -987,8 +1060,8 @@ static bool bin_plan(int64_t N, const nf_hash_geom* geom, int la, int lb, BinPla
     const int64_t res = geom->res[l];
     bp->cell[l - la] = cells && geom->dims == 3 && l < geom->first_hash_level && res * res + res + 1 < BIN_ROWS;
     // a cell level leaves at most two records per point; an x-pair level has room for every pair to be split in two
-    // (normally half of it is used)
-    R += N * (bp->cell[l - la] ? 2 : geom->dims == 3 ? 8 : 4);
+    // (normally half of it is used); more than three dimensions run as passes of the 3-D pipeline
+    R += N * (bp->cell[l - la] ? 2 : geom->dims >= 3 ? 8 : 4);
     nb_total += (int)nb;
   }
   bp->binbase[lb - la] = nb_total;
@@ -1010,7 +1083,7 @@ struct LevelGroups {
 };
 static bool bin_groups(int64_t N, const nf_hash_geom* geom, LevelGroups* groups) {
   // features are taken two at a time (one pass of fill + accumulate per pair; the last feature of an odd count alone)
-  if ((geom->dims != 3 && geom->dims != 2) || geom->feat < 1 || N <= 0) return false;
+  if (geom->dims < 2 || geom->dims > NF_MAX_DIMS || geom->feat < 1 || N <= 0) return false;
   groups->n = 0;
   groups->first[0] = 0;
   int nb_total = 0;
@@ -1063,10 +1136,11 @@ constexpr int64_t BIN_CHUNK_POINTS = (int64_t)1 << 21;
 // reference's default table size) the walk is the faster one; four bins would already cost it more hashing than the
 // records' passes take.
 constexpr int DIRECT_MAX_BINS_PER_LEVEL = 2;
+constexpr int DIRECT_MAX_DIMS = 4;  // the walk is built for 1 to 4 dimensions (the sorted records for 2 and 3)
 constexpr int64_t DIRECT_MIN_POINTS = 4096;  // below: one launch of scattered atomics is as quick
 static bool direct_ok(int64_t n_points, const nf_hash_geom* geom, int flags) {
   if ((flags & NF_HASH_BWD_RECORDS) || n_points < DIRECT_MIN_POINTS) return false;
-  if (geom->dims != 2 && geom->dims != 3) return false;
+  if (geom->dims < 1 || geom->dims > DIRECT_MAX_DIMS) return false;
   for (int l = 0; l < geom->levels; ++l)
     if (geom->rows[l] > (int64_t)DIRECT_MAX_BINS_PER_LEVEL * BIN_ROWS) return false;
   return true;
@@ -1169,12 +1243,14 @@ static int launch_bwd_direct(const void* coords, int cdt, int64_t csn, int64_t c
   slice_points = (slice_points + round - 1) / round * round;
   slices = (N + slice_points - 1) / slice_points;
   const size_t lds = (size_t)2 * BIN_ROWS * sizeof(unsigned long long);
-  const void* kern = g.dims == 3 ? (ddt == NF_F32    ? (const void*)hash_bwd_direct_k<F32, 3>
-                                    : ddt == NF_BF16 ? (const void*)hash_bwd_direct_k<BF16, 3>
-                                                     : (const void*)hash_bwd_direct_k<F16, 3>)
-                                 : (ddt == NF_F32    ? (const void*)hash_bwd_direct_k<F32, 2>
-                                    : ddt == NF_BF16 ? (const void*)hash_bwd_direct_k<BF16, 2>
-                                                     : (const void*)hash_bwd_direct_k<F16, 2>);
+  auto pick = [&](auto d_c) -> const void* {
+    constexpr int DD = decltype(d_c)::value;
+    return ddt == NF_F32 ? (const void*)hash_bwd_direct_k<F32, DD> : ddt == NF_BF16 ? (const void*)hash_bwd_direct_k<BF16, DD> : (const void*)hash_bwd_direct_k<F16, DD>;
+  };
+  const void* kern = g.dims == 3   ? pick(std::integral_constant<int, 3>{})
+                     : g.dims == 2 ? pick(std::integral_constant<int, 2>{})
+                     : g.dims == 1 ? pick(std::integral_constant<int, 1>{})
+                                   : pick(std::integral_constant<int, 4>{});
   hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
   const uint32_t* cpairs = pairs;
@@ -1229,14 +1305,26 @@ static int launch_bwd_bin_group(const void* coords, int cdt, int64_t csn, int64_
   const int NBp = (NB + 3) & ~3;
   const unsigned blocks = (unsigned)((N + FILL_POINTS - 1) / FILL_POINTS);
 
+  // more than three dimensions: the whole pipeline once per corner of the extra coordinates (`hi`), see ExtraDims
+  const int passes = g.dims > 3 ? 1 << (g.dims - 3) : 1;
+  for (int hi = 0; hi < passes; ++hi) {
   hipLaunchKernelGGL(hash_bwd_bin_zero_k, dim3((unsigned)((NBp + 32 + 255) / 256)), dim3(256), 0, s, ws.hist, NBp + 32);
   if (int rc = check_launch("hash_bwd_bin_zero")) return rc;
-  if (g.dims == 3)
+  if (g.dims == 6)
+    hipLaunchKernelGGL((hash_bwd_bin_count_k<3, 3>), dim3(blocks), dim3(FILL_POINTS), (size_t)NB * 4, s, coords, cdt, csn, csd, N, g, bp,
+                       primes, scale, ws.hist, ws.wg_counts, hi);
+  else if (g.dims == 5)
+    hipLaunchKernelGGL((hash_bwd_bin_count_k<3, 2>), dim3(blocks), dim3(FILL_POINTS), (size_t)NB * 4, s, coords, cdt, csn, csd, N, g, bp,
+                       primes, scale, ws.hist, ws.wg_counts, hi);
+  else if (g.dims == 4)
+    hipLaunchKernelGGL((hash_bwd_bin_count_k<3, 1>), dim3(blocks), dim3(FILL_POINTS), (size_t)NB * 4, s, coords, cdt, csn, csd, N, g, bp,
+                       primes, scale, ws.hist, ws.wg_counts, hi);
+  else if (g.dims == 3)
     hipLaunchKernelGGL(hash_bwd_bin_count_k<3>, dim3(blocks), dim3(FILL_POINTS), (size_t)NB * 4, s, coords, cdt, csn, csd, N, g, bp,
-                       primes, scale, ws.hist, ws.wg_counts);
+                       primes, scale, ws.hist, ws.wg_counts, hi);
   else
     hipLaunchKernelGGL(hash_bwd_bin_count_k<2>, dim3(blocks), dim3(FILL_POINTS), (size_t)NB * 4, s, coords, cdt, csn, csd, N, g, bp,
-                       primes, scale, ws.hist, ws.wg_counts);
+                       primes, scale, ws.hist, ws.wg_counts, hi);
   if (int rc = check_launch("hash_bwd_bin_count")) return rc;
   hipLaunchKernelGGL(hash_bwd_bin_offsets_k, dim3(1), dim3(1024), 0, s, (const uint32_t*)ws.hist, ws.cursor, ws.n_tasks,
                      ws.tasks, NB, max_tasks);
@@ -1254,14 +1342,17 @@ static int launch_bwd_bin_group(const void* coords, int cdt, int64_t csn, int64_
   {
     const size_t lds = (size_t)FILL_RECORDS * sizeof(uint4) + (g32 ? (size_t)FILL_POINTS * sizeof(uint2) : 0) +
                        ((size_t)2 * NB + 2 * NF_MAX_LEVELS) * 4;
-    const void* kern = g.dims == 3 ? (g32 ? (const void*)hash_bwd_bin_fill_k<true, 3> : (const void*)hash_bwd_bin_fill_k<false, 3>)
-                                   : (g32 ? (const void*)hash_bwd_bin_fill_k<true, 2> : (const void*)hash_bwd_bin_fill_k<false, 2>);
+    const void* kern = g.dims == 6   ? (g32 ? (const void*)hash_bwd_bin_fill_k<true, 3, 3> : (const void*)hash_bwd_bin_fill_k<false, 3, 3>)
+                       : g.dims == 5 ? (g32 ? (const void*)hash_bwd_bin_fill_k<true, 3, 2> : (const void*)hash_bwd_bin_fill_k<false, 3, 2>)
+                       : g.dims == 4 ? (g32 ? (const void*)hash_bwd_bin_fill_k<true, 3, 1> : (const void*)hash_bwd_bin_fill_k<false, 3, 1>)
+                       : g.dims == 3 ? (g32 ? (const void*)hash_bwd_bin_fill_k<true, 3> : (const void*)hash_bwd_bin_fill_k<false, 3>)
+                                     : (g32 ? (const void*)hash_bwd_bin_fill_k<true, 2> : (const void*)hash_bwd_bin_fill_k<false, 2>);
     hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     const uint32_t* wc = ws.wg_counts;
     void* args[] = {(void*)&coords, (void*)&cdt,   (void*)&csn,    (void*)&csd,   (void*)&dout, (void*)&dout_stride, (void*)&N, (void*)&g,
                     (void*)&bp,     (void*)&primes, (void*)&scale, (void*)&wc,    (void*)&ws.cursor, (void*)&ws.gmax, (void*)&ws.records,
-                    (void*)&feat,   (void*)&f0};
+                    (void*)&feat,   (void*)&f0,     (void*)&hi};
     e = hipLaunchKernel(kern, dim3(blocks), dim3(FILL_POINTS), args, lds, s);
     if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(hash_bwd_bin_fill): %s", hipGetErrorString(e));
     if (int rc = check_launch("hash_bwd_bin_fill")) return rc;
@@ -1281,6 +1372,7 @@ static int launch_bwd_bin_group(const void* coords, int cdt, int64_t csn, int64_
     e = hipLaunchKernel(kern, dim3(max_tasks), dim3(ACC_THREADS), args, lds, s);
     if (e != hipSuccess) return fail((int)e, "hipLaunchKernel(hash_bwd_bin_accum): %s", hipGetErrorString(e));
     if (int rc = check_launch("hash_bwd_bin_accum")) return rc;
+  }
   }
   }
   return 0;
