@@ -197,7 +197,7 @@ def test_chained_launches_keep_signal(act, gain, d_in, d_hidden, d_out, depth, d
         assert rel(leaves[k].grad, want["d" + k]) <= tol, k
 
 
-@pytest.mark.parametrize("depth", [2, 6])
+@pytest.mark.parametrize("depth", [1, 2, 6])
 def test_step_replays_from_a_hip_graph(depth):
     """The library only enqueues kernels on the caller's stream (no allocation, no synchronisation, no memset), so a
     forward + backward step can be captured once and replayed.  Every replay, with new inputs copied into the captured
