@@ -50,6 +50,15 @@ constexpr int ACC_THREADS = 1024;
 constexpr int ACC_INFLIGHT = 8;               // records in flight per thread
 constexpr uint32_t SLICE_RECORDS = 98304;     // a bin with at most this many records is one accumulation task
 constexpr uint32_t SPLIT_RECORDS = 32768;     // a bigger bin is cut into tasks of about this many
+// A cell record stands for eight corners (sixteen LDS adds against an x-pair record's four).  In batches of up to
+// CELL_FINE_MAX_POINTS points a cell level's tasks are cut four times finer: with the x-pair limits a coarse level of one
+// or two bins was a single task of up to 98304 cell records, and from 2^16 to 2^17 points that one task (about 100 us)
+// outlasted the rest of the accumulate launch (2^16 points: 109 -> 49 us, 2^17: 128 -> 57, 2^18: 89 -> 76).  Larger
+// batches hide such a task behind the others, and four times as many flushes of the same few thousand rows cost them
+// 30 us at 2^20 points.
+constexpr uint32_t CELL_FINE = 4;
+constexpr int64_t CELL_FINE_MAX_POINTS = (int64_t)1 << 18;
+static uint32_t cell_task_div(int64_t n_points) { return n_points <= CELL_FINE_MAX_POINTS ? CELL_FINE : 1u; }
 constexpr int MAX_BINS_PER_LEVEL = 2048;        // 2^24 rows
 constexpr int MAX_BINS_TOTAL = 2560;          // LDS of the count and fill kernels
 
@@ -379,14 +388,19 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t x, uint32_t* w
 }
 
 __global__ __launch_bounds__(1024) void hash_bwd_bin_offsets_k(const uint32_t* hist, uint32_t* cursor, uint32_t* n_tasks,
-                                                               uint4* tasks, int NB, uint32_t max_tasks) {
+                                                               uint4* tasks, int NB, uint32_t max_tasks, BinPlan bp,
+                                                               uint32_t cell_div) {
   __shared__ uint32_t wave_sums[16];
   __shared__ uint32_t first_task[1025], bin_start[1024], bin_count[1024];  // of the 1024 bins of a pass
   uint32_t rec_run = 0, task_run = 0;
   for (int b0 = 0; b0 < NB; b0 += 1024) {
     const int b = b0 + (int)threadIdx.x;
     const uint32_t c = b < NB ? hist[b] : 0u;
-    const uint32_t slices = c <= SLICE_RECORDS ? (c ? 1u : 0u) : (c + SPLIT_RECORDS - 1u) / SPLIT_RECORDS;
+    int lvl = 0;
+    while (lvl + 1 < bp.n_levels && b >= bp.binbase[lvl + 1]) ++lvl;
+    const bool cell = bp.cell[lvl] != 0;
+    const uint32_t one = cell ? SLICE_RECORDS / cell_div : SLICE_RECORDS, cut = cell ? SPLIT_RECORDS / cell_div : SPLIT_RECORDS;
+    const uint32_t slices = c <= one ? (c ? 1u : 0u) : (c + cut - 1u) / cut;
     uint32_t rec_total, task_total;
     const uint32_t start = rec_run + block_exclusive_scan(c, wave_sums, &rec_total);
     const uint32_t t0 = block_exclusive_scan(slices, wave_sums, &task_total);
@@ -1050,7 +1064,7 @@ static bool bin_plan(int64_t N, const nf_hash_geom* geom, int la, int lb, BinPla
                      bool cells = false) {
   bp->n_levels = lb - la;
   int nb_total = 0;
-  int64_t R = 0;
+  int64_t R = 0, R_cell = 0;
   for (int l = la; l < lb; ++l) {
     const int64_t r = geom->rows[l];
     const int64_t nb = (r + BIN_ROWS - 1) / BIN_ROWS;
@@ -1062,13 +1076,14 @@ static bool bin_plan(int64_t N, const nf_hash_geom* geom, int la, int lb, BinPla
     // a cell level leaves at most two records per point; an x-pair level has room for every pair to be split in two
     // (normally half of it is used); more than three dimensions run as passes of the 3-D pipeline
     R += N * (bp->cell[l - la] ? 2 : geom->dims >= 3 ? 8 : 4);
+    if (bp->cell[l - la]) R_cell += N * 2;
     nb_total += (int)nb;
   }
   bp->binbase[lb - la] = nb_total;
   if (nb_total > MAX_BINS_TOTAL) return false;
   if (R >= ((int64_t)1 << 32) - 4 * ACC_THREADS * ACC_INFLIGHT) return false;  // 32-bit record positions
   *records = R;
-  *max_tasks = (uint32_t)(nb_total + R / SPLIT_RECORDS + 1);
+  *max_tasks = (uint32_t)(nb_total + (R - R_cell) / SPLIT_RECORDS + R_cell / (SPLIT_RECORDS / cell_task_div(N)) + 1);
   return true;
 }
 
@@ -1327,7 +1342,7 @@ static int launch_bwd_bin_group(const void* coords, int cdt, int64_t csn, int64_
                        primes, scale, ws.hist, ws.wg_counts, hi);
   if (int rc = check_launch("hash_bwd_bin_count")) return rc;
   hipLaunchKernelGGL(hash_bwd_bin_offsets_k, dim3(1), dim3(1024), 0, s, (const uint32_t*)ws.hist, ws.cursor, ws.n_tasks,
-                     ws.tasks, NB, max_tasks);
+                     ws.tasks, NB, max_tasks, bp, cell_task_div(N));
   if (int rc = check_launch("hash_bwd_bin_offsets")) return rc;
   const int feat = geom->feat;
   for (int f0 = 0; f0 < feat; f0 += 2) {
@@ -1336,7 +1351,7 @@ static int launch_bwd_bin_group(const void* coords, int cdt, int64_t csn, int64_
       hipLaunchKernelGGL(hash_bwd_bin_zero_k, dim3(1), dim3(256), 0, s, ws.gmax, 32);
       if (int rc = check_launch("hash_bwd_bin_zero")) return rc;
       hipLaunchKernelGGL(hash_bwd_bin_offsets_k, dim3(1), dim3(1024), 0, s, (const uint32_t*)ws.hist, ws.cursor, ws.n_tasks,
-                         ws.tasks, NB, max_tasks);
+                         ws.tasks, NB, max_tasks, bp, cell_task_div(N));
       if (int rc = check_launch("hash_bwd_bin_offsets")) return rc;
     }
   {
