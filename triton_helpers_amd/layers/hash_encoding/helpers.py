@@ -53,11 +53,13 @@ def get_first_hash_level(N_min: int, N_max: int, L: int, T: int, D: int) -> int:
     return L + 1
 
 
-def _starts(L: int, T: int, D: int, N_min: int, N_max: int) -> List[int]:
+@lru_cache(maxsize=256)
+def _starts(L: int, T: int, D: int, N_min: int, N_max: int) -> Tuple[int, ...]:
+    # cached: the forward checks the table's size against the last entry on every call
     starts = [0]
     for c in compute_embedding_counts(L, T, D, N_min, N_max):
         starts.append(starts[-1] + c)
-    return starts
+    return tuple(starts)
 
 
 def seek_to_level_embeddings(e: Tensor, l_i: int, L: int, T: int, D: int, N_min: int, N_max: int) -> Tensor:
