@@ -261,7 +261,7 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_tiled_k(const void* coo
           a0 = a0 + w[i][j] * TT::to_f32((uint16_t)(v[i][j][f] & 0xffffu));
           a1 = a1 + w[i][j] * TT::to_f32((uint16_t)(v[i][j][f] >> 16));
         }
-        stage[(l * FW + f) * LD + t + TILE_THREADS * i] = (uint32_t)TT::from_f32(a0) | ((uint32_t)TT::from_f32(a1) << 16);
+        stage[(l * FW + f) * LD + t + TILE_THREADS * i] = TT::pack(a0, a1);
       }
   }
   __syncthreads();
@@ -359,7 +359,7 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_sweep_k(const void* coo
             a0 = a0 + w[i][j] * TT::to_f32((uint16_t)(v[i][j] & 0xffffu));
             a1 = a1 + w[i][j] * TT::to_f32((uint16_t)(v[i][j] >> 16));
           }
-          enc[i0 + i][l] = (uint32_t)TT::from_f32(a0) | ((uint32_t)TT::from_f32(a1) << 16);
+          enc[i0 + i][l] = TT::pack(a0, a1);
         }
       }
     } else {
@@ -570,7 +570,7 @@ __global__ __launch_bounds__(TILE_THREADS) void hash_fwd_level_k(const void* coo
     a0 = a0 + w[j] * TT::to_f32((uint16_t)(v[j] & 0xffffu));
     a1 = a1 + w[j] * TT::to_f32((uint16_t)(v[j] >> 16));
   }
-  *reinterpret_cast<uint32_t*>(out + n * out_stride + 2 * l) = (uint32_t)TT::from_f32(a0) | ((uint32_t)TT::from_f32(a1) << 16);
+  *reinterpret_cast<uint32_t*>(out + n * out_stride + 2 * l) = TT::pack(a0, a1);
 }
 
 template <typename GT, int D>

@@ -33,12 +33,19 @@ inline bool dtype_ok(int dt) { return dt == NF_F32 || dt == NF_F16 || dt == NF_B
 // bf16 is handled as raw uint16_t bits; round-to-nearest-even like torch.
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
 
-__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // quiet NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+// (gfx950 converts two floats to packed bfloat16 or float16, round-to-nearest-even, in one instruction)
+typedef float nf_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 nf_bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 nf_f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
+  const nf_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, nf_bf16x2));
 }
+__device__ __forceinline__ uint32_t f32x2_to_f16x2_bits(float lo, float hi) {
+  const nf_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, nf_f16x2));
+}
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) { return (uint16_t)(f32x2_to_bf16x2_bits(f, 0.0f) & 0xffffu); }
 
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t b) {
   return __half2float(__ushort_as_half(b));
@@ -57,12 +64,14 @@ struct F16 {
   static constexpr int code = NF_F16;
   __device__ static __forceinline__ float to_f32(storage v) { return f16_bits_to_f32(v); }
   __device__ static __forceinline__ storage from_f32(float f) { return f32_to_f16_bits(f); }
+  __device__ static __forceinline__ uint32_t pack(float lo, float hi) { return f32x2_to_f16x2_bits(lo, hi); }
 };
 struct BF16 {
   typedef uint16_t storage;
   static constexpr int code = NF_BF16;
   __device__ static __forceinline__ float to_f32(storage v) { return bf16_bits_to_f32(v); }
   __device__ static __forceinline__ storage from_f32(float f) { return f32_to_bf16_bits(f); }
+  __device__ static __forceinline__ uint32_t pack(float lo, float hi) { return f32x2_to_bf16x2_bits(lo, hi); }
 };
 
 // Load element i of a tensor whose dtype is only known at run time (uniform branch).
