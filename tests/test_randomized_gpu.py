@@ -73,6 +73,51 @@ def test_hash_encoding_random_configurations(seed):
         assert bool(torch.isfinite(got).all()) and not bool((d > 1e-3 * want.abs() + 2e-4 * peak).any()), f"backward: {tag}"
 
 
+@pytest.mark.parametrize("seed", range(3))
+def test_hash_encoding_random_configurations_in_one_and_four_to_six_dimensions(seed):
+    """The same differential run where the caller brings the primes: one dimension and four to six (the walk without
+    records, the record passes per corner of the extra coordinates, the per-(point, level) kernels below their
+    minimum batch), forward and backward."""
+    from triton_helpers_amd.layers.hash_encoding import kernel as hk
+
+    primes = torch.tensor([1, 2654435761, 805459861, 3674653429, 2097192037, 1434869437], dtype=torch.int64)
+    for it in range(12):
+        rng = random.Random(seed * 100019 + it)
+        D = rng.choice([1, 4, 4, 4, 5, 6])
+        F = rng.choice([1, 2, 2, 3, 4])
+        L = rng.choice([2, 4, 8])
+        lo = rng.choice([2, 3, 4, 8])
+        hi = max(lo, rng.choice([4, 6, 9, 16, 24, 40] if D > 1 else [64, 512, 5000, 40000]))
+        T = rng.choice([2**10, 2**13, 2**14, 2**15, 2**17, 2**19, 5000, 50000, 3 * 2**15])
+        N = rng.choice([63, 4099, 8192, 9001, 20000])
+        if D >= 5:
+            N = min(N, 9001)
+        scale = rng.choice([1.0, 2.0])
+        do_dtype = rng.choice([torch.float16, torch.bfloat16, torch.float32])
+        tab_dtype = rng.choice([torch.float16, torch.float32])
+        tag = f"seed={seed} it={it} D={D} F={F} L={L} lo={lo} hi={hi} T={T} N={N} scale={scale} do={do_dtype} table={tab_dtype}"
+        E = O.level_row_offsets(L, T, D, lo, hi)[-1]
+        if E > 20_000_000:
+            continue
+        torch.manual_seed(seed * 7927 + it)
+        x = torch.rand(N, D).clamp(max=0.999999)  # (1, .., 1) is outside the oracle's dense tables
+        x[: N // 4] = (torch.randint(0, hi, (N // 4, D)).float() / hi).clamp(max=0.999999)
+        x[N // 4 : N // 2] = (torch.rand(1, D) * 0.9 + 1e-3 * torch.rand(N // 2 - N // 4, D)).clamp(max=0.999999)
+        pi = primes[:D]
+        g = torch.Generator().manual_seed(it)
+        table = (torch.rand(E, F, generator=g) * 2 - 1).to(tab_dtype)
+        do = torch.randn(N, L * F).to(do_dtype)
+        want = O.encode_forward(x, table.float(), pi, T, L, lo, hi)
+        got = hk.hash_encoding(x.to(DEV) * scale, table.to(DEV), None, pi.to(DEV), T, lo, hi, L, scale=scale)
+        d, peak = _rel(got, want)
+        tol = {torch.float32: 1e-5, torch.float16: 2e-3}[tab_dtype]
+        assert float(d.max()) <= tol * max(1.0, peak), f"forward: {tag}"
+        want = O.encode_backward(x, do, E, F, pi, T, L, lo, hi)
+        got = hk.hash_encoding_table_grad(x.to(DEV) * scale, do.to(DEV), E, F, pi.to(DEV), T, lo, hi, L, scale).cpu()
+        d, peak = _rel(got, want)
+        assert bool(torch.isfinite(got).all()) and not bool((d > 1e-3 * want.abs() + 2e-4 * peak).any()), f"backward: {tag}"
+
+
 @pytest.mark.parametrize("seed", range(4))
 def test_fused_mlp_random_configurations(seed):
     """Errors relative to each tensor's largest magnitude: 2e-2 for 16-bit storage (x depth / 4 beyond four layers),
