@@ -208,6 +208,37 @@ def test_generic_forward_reads_rows_in_pieces(D, F, dtype, off, monkeypatch):
     torch.testing.assert_close(outs[0].cpu().float(), want, rtol=rtol, atol=atol)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("N,D", [(5000, 3), (2**18 + 33, 3), (2**18 + 33, 2)])
+def test_thirty_two_levels(N, D, dtype, monkeypatch):
+    """More than sixteen levels run as one forward call per sixteen levels on their own columns of the output: bit-equal
+    to the per-(point, level) kernel (flag 1) and within the storage rounding of the oracle; the backward against the
+    oracle on a sample of the batch."""
+    from triton_helpers_amd import _lib
+
+    hk = _hk()
+    torch.manual_seed(13)
+    T, L, lo, hi = 2**15, 32, 4, 4096
+    x = torch.rand(N, D, device=DEV)
+    table = _table(T, L, D, lo, hi, dtype=dtype, amp=1.0).to(DEV)
+    E = table.shape[0]
+    outs = {}
+    for flag in (0, _lib.NF_HASH_FORCE_GENERIC):
+        monkeypatch.setattr(hk, "_FLAGS", flag)
+        outs[flag] = hk.hash_encoding(x, table, None, None, T, lo, hi, L)
+    assert outs[0].shape == (N, 64) and torch.equal(outs[0], outs[_lib.NF_HASH_FORCE_GENERIC])
+    idx = torch.randperm(N)[:3000]
+    want = O.encode_forward(x[idx.to(DEV)].cpu(), table.float().cpu(), None, T, L, lo, hi)
+    eps = 1e-5 if dtype == torch.float32 else 2.0**-10
+    torch.testing.assert_close(outs[0][idx.to(DEV)].cpu().float(), want, rtol=eps, atol=eps * 1e-3 if dtype != torch.float32 else 1e-6)
+    monkeypatch.setattr(hk, "_FLAGS", 0)
+    xs = x[idx.to(DEV)].contiguous().repeat(4, 1)[:9000]     # 9000 points: the sorted-record backward
+    do = torch.randn(xs.shape[0], 64, device=DEV).to(dtype)
+    want_g = O.encode_backward(xs.cpu(), do.cpu(), E, 2, None, T, L, lo, hi)
+    got_g = hk.hash_encoding_table_grad(xs, do, E, 2, None, T, lo, hi, L).cpu()
+    torch.testing.assert_close(got_g, want_g, rtol=1e-3, atol=1e-4 * float(want_g.abs().max()))
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("N,D,T,L,lo,hi", [(1, 3, 2**19, 16, 16, 7006), (257, 3, 2**19, 16, 16, 7006), (5000, 3, 2**17, 2, 16, 700),
                                             (8191, 2, 2**19, 16, 16, 7006), (60001, 3, 2**19, 16, 16, 7006), (100000, 2, 2**15, 8, 8, 300)])

@@ -743,6 +743,28 @@ extern "C" int nf_hash_encode_fwd(const void* coords, int coords_dtype, int64_t 
   NF_REQUIRE(n_points <= ((int64_t)1 << 31) * 256 - 1, NF_EINVAL, "n_points too large");
   hipStream_t s = (hipStream_t)stream;
 
+  // More than sixteen levels: the fast kernels keep a point's results of up to sixteen levels in registers, and the
+  // levels are independent, so the call runs as one call per sixteen levels on its own columns of the output
+  // (2^20 points, 32 levels: 1.03 -> 0.73 ms).
+  if (g.levels > 16 && !(flags & NF_HASH_FORCE_GENERIC)) {
+    for (int l0 = 0; l0 < g.levels; l0 += 16) {
+      nf_hash_geom part = *geom;
+      part.levels = g.levels - l0 < 16 ? g.levels - l0 : 16;
+      const int fh = geom->first_hash_level - l0;
+      part.first_hash_level = fh < 0 ? 0 : (fh > part.levels ? part.levels : fh);
+      for (int l = 0; l < part.levels; ++l) {
+        part.res[l] = geom->res[l0 + l];
+        part.rows[l] = geom->rows[l0 + l];
+        part.row_offset[l] = geom->row_offset[l0 + l];
+      }
+      void* cols = (char*)out + (size_t)l0 * g.feat * dtype_size(table_dtype);
+      if (int rc = nf_hash_encode_fwd(coords, coords_dtype, csn, csd, table, table_dtype, cols, out_stride_n, n_points, &part, primes, scale,
+                                      flags, stream))
+        return rc;
+    }
+    return 0;
+  }
+
   // float32 tables: the same sweep on 8-byte rows
   if (!(flags & (NF_HASH_FORCE_GENERIC | NF_HASH_FWD_STAGED)) && n_points >= SWEEP_MIN_POINTS && table_dtype == NF_F32 &&
       sweep32_ok(geom, table, out, out_stride_n)) {
